@@ -1,0 +1,223 @@
+/*
+ * mi355_int8.h — C ABI of libmi355_int8.so: the int8 inference hot path
+ * (block-Hadamard rotation + int8 quantizer, W8A8 GEMM / GEMV, GQA decode
+ * attention over an int8 KV cache, MoE top-k dispatch + grouped expert GEMM)
+ * as hand-written HIP kernels for gfx950 (MI355X), plus the two runtime
+ * pieces that stand in, on this path only, for the upstream NUMA arena and
+ * clone3 thread pool.
+ *
+ * Calling convention (what a Mojo `external_call` / `DLHandle` binding, a cgo
+ * stub or ctypes needs): every argument is a pointer, an int64_t or an
+ * int32_t — the "args are 8-byte trivials" rule of the upstream launch path
+ * (threading/linux_threading.mojo:106-112).  Errors are return values, never
+ * exceptions and never exit(): 0 on success, a negative errno-class code
+ * otherwise, the convention of the upstream syscall shim
+ * (threading/linux.mojo:229-230, :235-236); allocation failure is a null
+ * pointer (threading/numa_arena.mojo:46-52).
+ *
+ * Upstream has NO int8 kernels and no FFI (README.md:4, :10-13), so the
+ * kernel entry points below replace nothing upstream; each cites the
+ * workload element it implements.  The arena and stream-pool entry points do
+ * replace upstream code and cite it.
+ *
+ * All device pointers must come from one device; kernels are enqueued on the
+ * `stream` argument (a hipStream_t passed as void*, NULL = the null stream)
+ * and return without waiting.  Calls are thread-compatible: no hidden mutable
+ * globals, but one context / pool / arena must not be used from two threads
+ * at once (upstream issues every launch from one orchestrator thread,
+ * test_linux_threading.mojo:112-115).
+ */
+#ifndef MI355_INT8_H
+#define MI355_INT8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_API __attribute__((visibility("default")))
+
+/* ---- status codes (negative errno class) -------------------------------- */
+#define MI_OK        0
+#define MI_EIO      (-5)   /* a HIP runtime call failed; see mi_last_hip_error */
+#define MI_ENOMEM   (-12)  /* device or host allocation failed                 */
+#define MI_EBUSY    (-16)  /* no free slot / destroy while work is in flight   */
+#define MI_ENODEV   (-19)  /* no such device, or not a gfx950 device           */
+#define MI_EINVAL   (-22)  /* null pointer, bad shape, bad alignment           */
+#define MI_ENOSPC   (-28)  /* workspace too small                              */
+#define MI_ERANGE   (-34)  /* a size is beyond what the kernels support        */
+
+MI_API const char *mi_status_string(int32_t status);
+MI_API int32_t mi_last_hip_error(void);        /* hipError_t of the last MI_EIO on this thread */
+MI_API int32_t mi_abi_version(void);
+
+/* ---- context ------------------------------------------------------------- */
+typedef struct mi_ctx mi_ctx;
+MI_API int32_t mi_ctx_create(int32_t device, mi_ctx **out);
+MI_API int32_t mi_ctx_destroy(mi_ctx *ctx);
+MI_API int32_t mi_ctx_device(const mi_ctx *ctx);
+MI_API int32_t mi_ctx_compute_units(const mi_ctx *ctx);
+MI_API int64_t mi_ctx_memory_bytes(const mi_ctx *ctx);
+MI_API int32_t mi_ctx_arch_name(const mi_ctx *ctx, char *buf, int64_t buf_len);
+
+/* ---- device arena --------------------------------------------------------
+ * Replaces NumaArena (threading/numa_arena.mojo:5-87) on this path: one slab
+ * of device memory, bump allocation with an alignment, watermarks, a null
+ * pointer on exhaustion, no per-allocation free.  `alignment` is a power of
+ * two (numa_arena.mojo:139-140); the slab is zero-filled at creation the way
+ * fresh mmap pages are (upstream tests rely on it, test_linux_threading.mojo:431). */
+typedef struct mi_arena mi_arena;
+MI_API int32_t mi_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t alignment, mi_arena **out); /* numa_arena.mojo:20-30 */
+MI_API int32_t mi_arena_destroy(mi_arena *a);                  /* numa_arena.mojo:32-34 */
+MI_API void   *mi_arena_alloc(mi_arena *a, int64_t bytes);     /* numa_arena.mojo:40-55; NULL when exhausted */
+MI_API int64_t mi_arena_mark(const mi_arena *a);               /* numa_arena.mojo:57-59 */
+MI_API int32_t mi_arena_reset_to(mi_arena *a, int64_t mark);   /* numa_arena.mojo:61-66; ignored (MI_EINVAL) unless 0 <= mark <= used */
+MI_API int32_t mi_arena_reset(mi_arena *a);                    /* numa_arena.mojo:68-70 */
+MI_API int64_t mi_arena_remaining(const mi_arena *a);          /* numa_arena.mojo:72-74 */
+MI_API int64_t mi_arena_used(const mi_arena *a);               /* numa_arena.mojo:76-78 */
+MI_API int32_t mi_arena_verify_placement(const mi_arena *a);   /* numa_arena.mojo:80-87; 1 = slab lives on the context's device */
+
+/* ---- stream pool and gate ------------------------------------------------
+ * Replaces ThreadPool (threading/linux_threading.mojo:43-158) on this path:
+ * a fixed number of slots, each a hipStream plus a completion event.  A slot
+ * is "in use" from mi_stream_pool_end until its event has completed, as a
+ * thread slot is from clone3 until child_tid returns to 0
+ * (linux_threading.mojo:273-275).
+ *   launch(fn, args)  ==  slot = begin(); enqueue work on stream(slot); end(slot)
+ * begin never blocks and reports a full pool as MI_EBUSY, as launch returns
+ * False (linux_threading.mojo:103-121). */
+typedef struct mi_stream_pool mi_stream_pool;
+MI_API int32_t mi_stream_pool_create(mi_ctx *ctx, int32_t capacity, mi_stream_pool **out); /* linux_threading.mojo:56-66, :130-158 */
+MI_API int32_t mi_stream_pool_destroy(mi_stream_pool *p);      /* linux_threading.mojo:70-77: MI_EBUSY (pool kept) instead of abort() when work is in flight */
+MI_API int32_t mi_stream_pool_capacity(const mi_stream_pool *p);         /* linux_threading.mojo:85-86 */
+MI_API int32_t mi_stream_pool_begin(mi_stream_pool *p);        /* first free slot index, or MI_EBUSY; linux_threading.mojo:104-105 */
+MI_API void   *mi_stream_pool_stream(mi_stream_pool *p, int32_t slot);   /* hipStream_t of the slot, NULL if out of range */
+MI_API int32_t mi_stream_pool_end(mi_stream_pool *p, int32_t slot);      /* record the completion event: slot is now in use */
+MI_API int32_t mi_stream_pool_in_use(mi_stream_pool *p, int32_t slot);   /* 1 / 0; frees the slot when its event has completed */
+MI_API int32_t mi_stream_pool_wait_all(mi_stream_pool *p);     /* linux_threading.mojo:123-126 */
+MI_API int32_t mi_stream_pool_wait_any(mi_stream_pool *p);     /* linux_threading.mojo:128-129, :391-407: index of a slot that finished, -1 if none was in use */
+
+/* Replaces MutexGate (linux_threading.mojo:174-198): a one-shot token.
+ * release() records it on a stream; wait() makes later work on another stream
+ * wait for it, wait_host() makes the calling thread wait; waiting on a gate
+ * that was never released is MI_EINVAL instead of blocking forever. */
+typedef struct mi_gate mi_gate;
+MI_API int32_t mi_gate_create(mi_ctx *ctx, mi_gate **out);
+MI_API int32_t mi_gate_destroy(mi_gate *g);
+MI_API int32_t mi_gate_release(mi_gate *g, void *stream);      /* linux_threading.mojo:191-194 */
+MI_API int32_t mi_gate_wait(mi_gate *g, void *stream);         /* linux_threading.mojo:186-189: later work on `stream` waits */
+MI_API int32_t mi_gate_wait_host(mi_gate *g);                  /* the calling host thread waits */
+MI_API int32_t mi_gate_reset(mi_gate *g);                      /* linux_threading.mojo:196-198 */
+
+/* ---- copies, host staging, events ----------------------------------------- */
+MI_API int32_t mi_memcpy_h2d(void *dst_dev, const void *src_host, int64_t bytes, void *stream);
+MI_API int32_t mi_memcpy_d2h(void *dst_host, const void *src_dev, int64_t bytes, void *stream);
+MI_API int32_t mi_memcpy_d2d(void *dst_dev, const void *src_dev, int64_t bytes, void *stream);
+MI_API int32_t mi_fill_u32(void *dst_dev, uint32_t value, int64_t count, void *stream); /* a fill kernel, safe under graph capture */
+MI_API int32_t mi_stream_synchronize(void *stream);
+MI_API void   *mi_host_alloc(int64_t bytes);                   /* pinned host memory, NULL on failure */
+MI_API int32_t mi_host_free(void *p);
+typedef struct mi_event mi_event;
+MI_API int32_t mi_event_create(mi_event **out);
+MI_API int32_t mi_event_destroy(mi_event *e);
+MI_API int32_t mi_event_record(mi_event *e, void *stream);
+MI_API int32_t mi_event_synchronize(mi_event *e);
+MI_API int32_t mi_event_elapsed_ms(mi_event *start, mi_event *stop, float *ms);
+
+/* ---- a1 + a2 / a3 / a7: block Hadamard rotation fused with the row quantizer
+ * x fp32 [M,K] row-major -> q int8 [M,K], scale fp32 [M].
+ * Each row is rotated in blocks of `block` (128 or 256) along K with the
+ * normalized Sylvester Hadamard matrix, then quantized symmetrically with its
+ * own absmax: scale = a/127, code = clamp(rne(x' * (127/a)), -127, 127); an
+ * all-zero row gives scale 1 and codes 0.  The same call prepares activations
+ * (per token), weights [N,K] (per output channel) and KV-cache rows
+ * [B*Hkv*T, D] (per token-head, block = D).  K % block == 0, K <= 32768.
+ * Codes and scales are bit-exact against the CPU restatement. */
+MI_API int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale,
+                                    int64_t M, int64_t K, int32_t block, void *stream);
+/* a1 alone: out fp32 [M,K] = rotated rows (out may alias x). */
+MI_API int32_t mi_fwht_f32(const float *x, float *out, int64_t M, int64_t K,
+                           int32_t block, void *stream);
+
+/* ---- a4 / a5: W8A8 contraction, acc[m,n] = sum_k qx[m,k] * qw[n,k]
+ * qx int8 [M,K], qw int8 [N,K] (both K-contiguous), acc int32 [M,N].
+ * M <= 64 streams the weights once through a skinny MFMA kernel (decode
+ * GEMV); larger M uses the LDS-tiled v_mfma_i32_16x16x64_i8 kernel (prefill).
+ * K % 128 == 0, N % 16 == 0.  Exact integer arithmetic. */
+MI_API int32_t mi_w8a8_gemm_i32(const int8_t *qx, const int8_t *qw, int32_t *acc,
+                                int64_t M, int64_t N, int64_t K, void *stream);
+/* a4/a5 + a6 fused: y[m,n] = ((float)acc * sx[m]) * sw[n], fp32 [M,N]. */
+MI_API int32_t mi_w8a8_gemm_dequant_f32(const int8_t *qx, const float *sx,
+                                        const int8_t *qw, const float *sw, float *y,
+                                        int64_t M, int64_t N, int64_t K, void *stream);
+/* a6 alone. */
+MI_API int32_t mi_dequant_i32_f32(const int32_t *acc, const float *sx, const float *sw,
+                                  float *y, int64_t M, int64_t N, void *stream);
+/* The whole rotated W8A8 linear: x fp32 [M,K] -> y fp32 [M,N] with prepared
+ * weights (qw, sw).  workspace holds the activation codes and scales. */
+MI_API int64_t mi_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+MI_API int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const float *sw, float *y,
+                                  int64_t M, int64_t N, int64_t K, int32_t block,
+                                  void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- a8: grouped-query decode attention over an int8 KV cache
+ * q fp32 [B,Hq,D] (unrotated); kq,vq int8 [B,Hkv,T,D]; ks,vs fp32 [B,Hkv,T];
+ * o fp32 [B,Hq,D].  D == 128, Hq % Hkv == 0, Hq/Hkv <= 4, any T >= 1.
+ * The query head is rotated and quantized to int8, scores are int32 dots,
+ * softmax (scale 1/sqrt(D)) and the P.V sum accumulate in fp32.
+ * out_rotated != 0 leaves o in the rotated basis of V. */
+MI_API int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T);
+MI_API int32_t mi_gqa_decode_attn(const float *q, const int8_t *kq, const float *ks,
+                                  const int8_t *vq, const float *vs, float *o,
+                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T,
+                                  int32_t out_rotated, void *workspace, int64_t workspace_bytes,
+                                  void *stream);
+/* Gate helper: runs the same split kernel and also writes out the int8 query
+ * codes [B,Hq,D], their scales [B,Hq] and the raw int32 scores [B,Hq,T] it
+ * works from (no merge, no o). */
+MI_API int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const float *ks,
+                                        const int8_t *vq, const float *vs,
+                                        int8_t *qq, float *sq, int32_t *dots,
+                                        int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T,
+                                        void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- a9: MoE router: logits = x . wr^T in a fixed fp32 order, top-k on the
+ * logits (ties to the lower expert), weights = softmax over the k picks.
+ * x fp32 [T,H], wr fp32 [E,H] -> idx int32 [T,topk], w fp32 [T,topk].
+ * H % 256 == 0, E <= 256, topk <= 8. */
+MI_API int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, float *w,
+                            int64_t T, int64_t H, int64_t E, int32_t topk, void *stream);
+/* ---- a10: stable grouping of the T*topk (token,slot) pairs by expert.
+ * idx int32 [T,topk] -> perm int32 [T*topk] (perm[pos] = pair = token*topk+slot),
+ * seg_off int32 [E+1].  E * ceil(T/32) <= 16384. */
+MI_API int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off,
+                               int64_t T, int64_t E, int32_t topk, void *stream);
+/* ---- a11: grouped expert SwiGLU FFN over expert-sorted segments.
+ * x fp32 [T,H]; idx,w [T,topk]; wg,wu int8 [E,I,H] + sg,su fp32 [E,I];
+ * wd int8 [E,H,I] + sd fp32 [E,H]; y fp32 [T,H].
+ * H % 128 == 0 (input block 128), I % 256 == 0 (inner block 256). */
+MI_API int64_t mi_moe_ffn_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk);
+MI_API int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w,
+                          const int8_t *wg, const float *sg, const int8_t *wu, const float *su,
+                          const int8_t *wd, const float *sd, float *y,
+                          int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk,
+                          void *workspace, int64_t workspace_bytes, void *stream);
+/* Byte offsets into the mi_moe_ffn workspace, for gates that inspect the
+ * intermediates: which = 0 qx int8[T,H], 1 sx f32[T], 2 perm i32[T*topk],
+ * 3 seg_off i32[E+1], 4 h f32[T*topk,I] (sorted order), 5 hq int8[T*topk,I],
+ * 6 hs f32[T*topk], 7 out f32[T*topk,H] (pair order).  Negative on error. */
+MI_API int64_t mi_moe_ffn_workspace_offset(int32_t which, int64_t T, int64_t H, int64_t I,
+                                           int64_t E, int32_t topk);
+/* Router + dispatch + FFN in one call (routing results land in the workspace). */
+MI_API int32_t mi_moe_layer(const float *x, const float *wr,
+                            const int8_t *wg, const float *sg, const int8_t *wu, const float *su,
+                            const int8_t *wd, const float *sd, float *y,
+                            int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk,
+                            void *workspace, int64_t workspace_bytes, void *stream);
+MI_API int64_t mi_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_INT8_H */

@@ -1,0 +1,270 @@
+// Block Hadamard rotation fused with the symmetric int8 row quantizer
+// (workload elements a1 + a2, reused for weight prep a3 and KV-cache rows a7).
+//
+// Data layout.  A row of K floats is cut into chunks of 8 floats; chunk c of a
+// Hadamard block of size BLOCK is the two float4 at offsets 4c and
+// BLOCK/2 + 4c inside the block, so one thread owns the elements whose index
+// bits are {0,1} (inside a float4) and the top bit (lower / upper half), and
+// the BLOCK/8 consecutive lanes that share a block own the middle bits.  The
+// butterfly stages therefore run in the fixed order h = 1, 2 (in-lane),
+// h = 4 .. BLOCK/4 (lane xor 1, 2, 4, 8[, 16] through DPP / ds_swizzle),
+// h = BLOCK/2 (in-lane), each output being one fp32 add or subtract, followed
+// by one multiply by fp32(1/sqrt(BLOCK)).  That is the order the CPU
+// restatement uses, and since no FMA is formed (-ffp-contract=off) the codes
+// are bit-exact against it.
+//
+// Every load is a float4 and the BLOCK/8 neighbouring lanes of a block read
+// 2*BLOCK contiguous bytes (whole 128-byte lines); the codes leave as one
+// dword per float4.  The kernel reads 4 B and writes 1 B per element: HBM-bound.
+#include "common.h"
+
+namespace mi {
+
+// value held by lane (lane ^ MASK); MASK in {1,2,4,8,16}
+template <int MASK>
+__device__ __forceinline__ float xor_lane(float v)
+{
+    const int i = __float_as_int(v);
+    int r;
+    if constexpr (MASK == 1) {
+        r = __builtin_amdgcn_update_dpp(i, i, 0xB1, 0xf, 0xf, false);  // quad_perm [1,0,3,2]
+    } else if constexpr (MASK == 2) {
+        r = __builtin_amdgcn_update_dpp(i, i, 0x4E, 0xf, 0xf, false);  // quad_perm [2,3,0,1]
+    } else {
+        // ds_swizzle bit mode: lane' = ((lane & 0x1f) | 0) ^ MASK inside each half wave
+        r = __builtin_amdgcn_ds_swizzle(i, 0x1F | (MASK << 10));
+    }
+    return __int_as_float(r);
+}
+
+// one cross-lane butterfly stage on 8 values: the lane whose MASK bit is
+// clear holds x[i] and keeps x[i] + x[i+h]; its partner keeps x[i] - x[i+h]
+template <int MASK>
+__device__ __forceinline__ void cross_stage(float (&v)[8], unsigned negmask)
+{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float other = xor_lane<MASK>(v[e]);
+        const float mine = __int_as_float(__float_as_int(v[e]) ^ negmask);  // -v on the upper lane
+        v[e] = other + mine;
+    }
+}
+
+template <int BLOCK>
+__device__ __forceinline__ void fwht_chunk(float (&v)[8], int j)
+{
+    // h = 1, 2: inside each float4
+#pragma unroll
+    for (int b = 0; b < 8; b += 4) {
+        float a0 = v[b] + v[b + 1], a1 = v[b] - v[b + 1];
+        float a2 = v[b + 2] + v[b + 3], a3 = v[b + 2] - v[b + 3];
+        v[b] = a0 + a2; v[b + 2] = a0 - a2;
+        v[b + 1] = a1 + a3; v[b + 3] = a1 - a3;
+    }
+    // h = 4 .. BLOCK/4: across the lanes of the block
+    cross_stage<1>(v, (j & 1) ? 0x80000000u : 0u);
+    cross_stage<2>(v, (j & 2) ? 0x80000000u : 0u);
+    cross_stage<4>(v, (j & 4) ? 0x80000000u : 0u);
+    cross_stage<8>(v, (j & 8) ? 0x80000000u : 0u);
+    if constexpr (BLOCK == 256) cross_stage<16>(v, (j & 16) ? 0x80000000u : 0u);
+    // h = BLOCK/2: lower half against upper half
+    constexpr float S = (BLOCK == 128) ? 0.08838834764831845f : 0.0625f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float lo = v[e] + v[e + 4], hi = v[e] - v[e + 4];
+        v[e] = lo * S;
+        v[e + 4] = hi * S;
+    }
+}
+
+__device__ __forceinline__ float abs8(const float (&v)[8])
+{
+    float a = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a = fmaxf(a, fabsf(v[e]));
+    return a;
+}
+
+__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d, float inv)
+{
+    const int i0 = (int)fminf(fmaxf(rintf(a * inv), -127.0f), 127.0f);
+    const int i1 = (int)fminf(fmaxf(rintf(b * inv), -127.0f), 127.0f);
+    const int i2 = (int)fminf(fmaxf(rintf(c * inv), -127.0f), 127.0f);
+    const int i3 = (int)fminf(fmaxf(rintf(d * inv), -127.0f), 127.0f);
+    return (uint32_t)(i0 & 0xff) | ((uint32_t)(i1 & 0xff) << 8) | ((uint32_t)(i2 & 0xff) << 16) |
+           ((uint32_t)i3 << 24);
+}
+
+// One workgroup per row; thread t owns chunks t, t + T, ... (C of them).
+// QUANT: write int8 codes + scale; otherwise write the rotated fp32 row.
+template <int BLOCK, int C, bool QUANT>
+__global__ __launch_bounds__(1024) void k_fwht_rows(const float *x, int8_t *__restrict__ q,
+                                                    float *__restrict__ scale, float *xrot, int K)
+{
+    constexpr int LPB = BLOCK / 8;
+    const int t = threadIdx.x, T = blockDim.x;
+    const int j = t % LPB;
+    const int nchunk = K / 8;
+    const int64_t row = blockIdx.x;
+    const float *xr = x + row * (int64_t)K;
+
+    float v[C][8];
+    int base[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int c = t + i * T;
+        base[i] = (c / LPB) * BLOCK + 4 * j;
+        if (c < nchunk) {
+            const float4 lo = *reinterpret_cast<const float4 *>(xr + base[i]);
+            const float4 hi = *reinterpret_cast<const float4 *>(xr + base[i] + BLOCK / 2);
+            v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+            v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        fwht_chunk<BLOCK>(v[i], j);
+        amax = fmaxf(amax, abs8(v[i]));
+    }
+
+    if constexpr (!QUANT) {
+        float *orow = xrot + row * (int64_t)K;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (t + i * T < nchunk) {
+                *reinterpret_cast<float4 *>(orow + base[i]) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+                *reinterpret_cast<float4 *>(orow + base[i] + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+            }
+        }
+    } else {
+        // row absmax: wave butterfly, then across waves through LDS
+        __shared__ float s_max[16];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        const int wave = t >> 6, nwave = (T + 63) >> 6;
+        if ((t & 63) == 0) s_max[wave] = amax;
+        __syncthreads();
+        float a = s_max[0];
+        for (int w = 1; w < nwave; ++w) a = fmaxf(a, s_max[w]);
+        const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+        const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+        if (t == 0) scale[row] = sc;
+        int8_t *qrow = q + row * (int64_t)K;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (t + i * T < nchunk) {
+                *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                *reinterpret_cast<uint32_t *>(qrow + base[i] + BLOCK / 2) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+            }
+        }
+    }
+}
+
+// K == BLOCK (a row is one Hadamard block, e.g. attention heads and KV-cache
+// rows): BLOCK/8 lanes per row, 256*8/BLOCK rows per workgroup, the absmax is
+// reduced inside the lane group only.
+template <int BLOCK, bool QUANT>
+__global__ __launch_bounds__(256) void k_fwht_small(const float *x, int8_t *__restrict__ q,
+                                                    float *__restrict__ scale, float *xrot, int64_t M)
+{
+    constexpr int LPB = BLOCK / 8;
+    constexpr int ROWS = 256 / LPB;
+    const int t = threadIdx.x, j = t % LPB;
+    const int64_t row = (int64_t)blockIdx.x * ROWS + t / LPB;
+    const bool live = row < M;
+    const int64_t off = row * BLOCK + 4 * j;
+    float v[8];
+    if (live) {
+        const float4 lo = *reinterpret_cast<const float4 *>(x + off);
+        const float4 hi = *reinterpret_cast<const float4 *>(x + off + BLOCK / 2);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+        v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    }
+    fwht_chunk<BLOCK>(v, j);
+    if constexpr (!QUANT) {
+        if (live) {
+            *reinterpret_cast<float4 *>(xrot + off) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4 *>(xrot + off + BLOCK / 2) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+    } else {
+        float a = abs8(v);
+#pragma unroll
+        for (int m = LPB / 2; m >= 1; m >>= 1) a = fmaxf(a, __shfl_xor(a, m, 64));
+        const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+        const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+        if (live) {
+            if (j == 0) scale[row] = sc;
+            *reinterpret_cast<uint32_t *>(q + off) = quant4(v[0], v[1], v[2], v[3], inv);
+            *reinterpret_cast<uint32_t *>(q + off + BLOCK / 2) = quant4(v[4], v[5], v[6], v[7], inv);
+        }
+    }
+}
+
+template <int BLOCK, bool QUANT>
+static int32_t launch_rows(const float *x, int8_t *q, float *scale, float *xrot, int64_t M, int64_t K,
+                           hipStream_t s)
+{
+    if (K == BLOCK) {
+        constexpr int ROWS = 256 / (BLOCK / 8);
+        const int64_t grid = (M + ROWS - 1) / ROWS;
+        hipLaunchKernelGGL((k_fwht_small<BLOCK, QUANT>), dim3((unsigned)grid), dim3(256), 0, s, x, q, scale, xrot, M);
+        return launch_status();
+    }
+    const int nchunk = (int)(K / 8);
+    int T = nchunk >= 256 ? 256 : ((nchunk + 63) / 64) * 64;
+    const int C = (nchunk + T - 1) / T;
+    const dim3 grid((unsigned)M), blk((unsigned)T);
+#define MI_ROWS_CASE(CC)                                                                                   \
+    hipLaunchKernelGGL((k_fwht_rows<BLOCK, CC, QUANT>), grid, blk, 0, s, x, q, scale, xrot, (int)K)
+    if (C <= 1) MI_ROWS_CASE(1);
+    else if (C <= 2) MI_ROWS_CASE(2);
+    else if (C <= 4) MI_ROWS_CASE(4);
+    else if (C <= 7) MI_ROWS_CASE(7);
+    else if (C <= 8) MI_ROWS_CASE(8);
+    else if (C <= 16) MI_ROWS_CASE(16);
+    else return MI_ERANGE;
+#undef MI_ROWS_CASE
+    return launch_status();
+}
+
+static int32_t check_rows(const void *x, const void *out, int64_t M, int64_t K, int32_t block)
+{
+    if (!x || !out || M < 0 || K <= 0) return MI_EINVAL;
+    if (block != 128 && block != 256) return MI_EINVAL;
+    if (K % block) return MI_EINVAL;
+    if (K > 32768 || M > 0x7fffffffLL) return MI_ERANGE;
+    if (!aligned16(x)) return MI_EINVAL;
+    return MI_OK;
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale, int64_t M, int64_t K,
+                                        int32_t block, void *stream)
+{
+    int32_t rc = check_rows(x, q, M, K, block);
+    if (rc) return rc;
+    if (!scale || !aligned4(q) || !aligned4(scale)) return MI_EINVAL;
+    if (M == 0) return MI_OK;
+    return block == 128 ? launch_rows<128, true>(x, q, scale, nullptr, M, K, as_stream(stream))
+                        : launch_rows<256, true>(x, q, scale, nullptr, M, K, as_stream(stream));
+}
+
+extern "C" int32_t mi_fwht_f32(const float *x, float *out, int64_t M, int64_t K, int32_t block, void *stream)
+{
+    int32_t rc = check_rows(x, out, M, K, block);
+    if (rc) return rc;
+    if (!aligned16(out)) return MI_EINVAL;
+    if (M == 0) return MI_OK;
+    return block == 128 ? launch_rows<128, false>(x, nullptr, nullptr, out, M, K, as_stream(stream))
+                        : launch_rows<256, false>(x, nullptr, nullptr, out, M, K, as_stream(stream));
+}

@@ -1,0 +1,290 @@
+"""ctypes binding of libmi355_int8.so (the C ABI in include/mi355_int8.h).
+
+Host-side plumbing for tests, smoke and the benchmark: it owns no arithmetic.
+Device buffers come from the library's own arena (the device analog of the
+upstream NumaArena, threading/numa_arena.mojo:5-87), so a test reads like the
+upstream ones: make an arena, alloc, launch, wait, check
+(test_linux_threading.mojo:164-215).
+
+There is no CPU fallback: if the shared library is missing, import fails.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355_int8.so")
+
+OK, EIO, ENOMEM, EBUSY, ENODEV, EINVAL, ENOSPC, ERANGE = 0, -5, -12, -16, -19, -22, -28, -34
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libmi355_int8.so is not built (%s). Run `python -c 'import __graft_entry__ as g; g.build()'` "
+        "or `make -C mojo-linuxperiments_amd/csrc`; there is no CPU fallback." % LIB_PATH)
+
+lib = C.CDLL(LIB_PATH)
+
+i32, i64, vp, f32p = C.c_int32, C.c_int64, C.c_void_p, C.POINTER(C.c_float)
+
+# name -> (restype, argtypes); the same list drives the export check in tests
+SIGNATURES = {
+    "mi_status_string": (C.c_char_p, [i32]),
+    "mi_last_hip_error": (i32, []),
+    "mi_abi_version": (i32, []),
+    "mi_ctx_create": (i32, [i32, C.POINTER(vp)]),
+    "mi_ctx_destroy": (i32, [vp]),
+    "mi_ctx_device": (i32, [vp]),
+    "mi_ctx_compute_units": (i32, [vp]),
+    "mi_ctx_memory_bytes": (i64, [vp]),
+    "mi_ctx_arch_name": (i32, [vp, C.c_char_p, i64]),
+    "mi_arena_create": (i32, [vp, i64, i64, C.POINTER(vp)]),
+    "mi_arena_destroy": (i32, [vp]),
+    "mi_arena_alloc": (vp, [vp, i64]),
+    "mi_arena_mark": (i64, [vp]),
+    "mi_arena_reset_to": (i32, [vp, i64]),
+    "mi_arena_reset": (i32, [vp]),
+    "mi_arena_remaining": (i64, [vp]),
+    "mi_arena_used": (i64, [vp]),
+    "mi_arena_verify_placement": (i32, [vp]),
+    "mi_stream_pool_create": (i32, [vp, i32, C.POINTER(vp)]),
+    "mi_stream_pool_destroy": (i32, [vp]),
+    "mi_stream_pool_capacity": (i32, [vp]),
+    "mi_stream_pool_begin": (i32, [vp]),
+    "mi_stream_pool_stream": (vp, [vp, i32]),
+    "mi_stream_pool_end": (i32, [vp, i32]),
+    "mi_stream_pool_in_use": (i32, [vp, i32]),
+    "mi_stream_pool_wait_all": (i32, [vp]),
+    "mi_stream_pool_wait_any": (i32, [vp]),
+    "mi_gate_create": (i32, [vp, C.POINTER(vp)]),
+    "mi_gate_destroy": (i32, [vp]),
+    "mi_gate_release": (i32, [vp, vp]),
+    "mi_gate_wait": (i32, [vp, vp]),
+    "mi_gate_wait_host": (i32, [vp]),
+    "mi_gate_reset": (i32, [vp]),
+    "mi_memcpy_h2d": (i32, [vp, vp, i64, vp]),
+    "mi_memcpy_d2h": (i32, [vp, vp, i64, vp]),
+    "mi_memcpy_d2d": (i32, [vp, vp, i64, vp]),
+    "mi_fill_u32": (i32, [vp, C.c_uint32, i64, vp]),
+    "mi_stream_synchronize": (i32, [vp]),
+    "mi_host_alloc": (vp, [i64]),
+    "mi_host_free": (i32, [vp]),
+    "mi_event_create": (i32, [C.POINTER(vp)]),
+    "mi_event_destroy": (i32, [vp]),
+    "mi_event_record": (i32, [vp, vp]),
+    "mi_event_synchronize": (i32, [vp]),
+    "mi_event_elapsed_ms": (i32, [vp, vp, f32p]),
+    "mi_fwht_quant_f32_i8": (i32, [vp, vp, vp, i64, i64, i32, vp]),
+    "mi_fwht_f32": (i32, [vp, vp, i64, i64, i32, vp]),
+    "mi_w8a8_gemm_i32": (i32, [vp, vp, vp, i64, i64, i64, vp]),
+    "mi_w8a8_gemm_dequant_f32": (i32, [vp, vp, vp, vp, vp, i64, i64, i64, vp]),
+    "mi_dequant_i32_f32": (i32, [vp, vp, vp, vp, i64, i64, vp]),
+    "mi_w8a8_linear_workspace_bytes": (i64, [i64, i64, i64]),
+    "mi_w8a8_linear_f32": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
+    "mi_gqa_decode_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
+    "mi_gqa_decode_attn": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp]),
+    "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
+}
+
+_missing = []
+for _name, (_res, _args) in SIGNATURES.items():
+    try:
+        _fn = getattr(lib, _name)
+    except AttributeError:
+        _missing.append(_name)
+        continue
+    _fn.restype = _res
+    _fn.argtypes = _args
+if _missing:
+    raise ImportError("libmi355_int8.so lacks symbols: %s" % ", ".join(_missing))
+
+
+class MiError(RuntimeError):
+    def __init__(self, status, what=""):
+        self.status = status
+        msg = lib.mi_status_string(status).decode()
+        if status == EIO:
+            msg += " (hipError %d)" % lib.mi_last_hip_error()
+        super().__init__("%s: %s [%d]" % (what, msg, status))
+
+
+def check(status, what=""):
+    if status != OK:
+        raise MiError(status, what)
+
+
+class DevBuf:
+    """A typed view of arena memory: device pointer + shape + dtype."""
+
+    def __init__(self, ptr, shape, dtype):
+        self.ptr = ptr
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+
+    @property
+    def nbytes(self):
+        return int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+
+    def offset(self, nbytes, shape, dtype):
+        return DevBuf(self.ptr + int(nbytes), shape, dtype)
+
+
+class Device:
+    """Context + one device arena + upload / download helpers."""
+
+    def __init__(self, device=0, arena_bytes=1 << 30, alignment=256):
+        self.ctx = vp()
+        check(lib.mi_ctx_create(device, C.byref(self.ctx)), "mi_ctx_create")
+        self.arena = vp()
+        rc = lib.mi_arena_create(self.ctx, arena_bytes, alignment, C.byref(self.arena))
+        if rc != OK:
+            lib.mi_ctx_destroy(self.ctx)
+            raise MiError(rc, "mi_arena_create")
+
+    def close(self):
+        if self.arena:
+            lib.mi_arena_destroy(self.arena)
+            self.arena = None
+        if self.ctx:
+            lib.mi_ctx_destroy(self.ctx)
+            self.ctx = None
+
+    @property
+    def compute_units(self):
+        return lib.mi_ctx_compute_units(self.ctx)
+
+    @property
+    def arch(self):
+        buf = C.create_string_buffer(64)
+        check(lib.mi_ctx_arch_name(self.ctx, buf, 64))
+        return buf.value.decode()
+
+    def mark(self):
+        return lib.mi_arena_mark(self.arena)
+
+    def reset_to(self, mark):
+        check(lib.mi_arena_reset_to(self.arena, mark), "mi_arena_reset_to")
+
+    def empty(self, shape, dtype):
+        shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        nbytes = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
+        p = lib.mi_arena_alloc(self.arena, max(nbytes, 1))
+        if not p:
+            raise MiError(ENOMEM, "mi_arena_alloc(%d)" % nbytes)
+        return DevBuf(p, shape, dtype)
+
+    def upload(self, arr, stream=None):
+        arr = np.ascontiguousarray(arr)
+        b = self.empty(arr.shape, arr.dtype)
+        check(lib.mi_memcpy_h2d(b.ptr, arr.ctypes.data, arr.nbytes, stream), "mi_memcpy_h2d")
+        check(lib.mi_stream_synchronize(stream))
+        return b
+
+    def download(self, buf, stream=None):
+        out = np.empty(buf.shape, buf.dtype)
+        check(lib.mi_stream_synchronize(stream))
+        check(lib.mi_memcpy_d2h(out.ctypes.data, buf.ptr, out.nbytes, stream), "mi_memcpy_d2h")
+        check(lib.mi_stream_synchronize(stream))
+        return out
+
+    def sync(self, stream=None):
+        check(lib.mi_stream_synchronize(stream), "mi_stream_synchronize")
+
+
+class Event:
+    def __init__(self):
+        self.h = vp()
+        check(lib.mi_event_create(C.byref(self.h)), "mi_event_create")
+
+    def record(self, stream=None):
+        check(lib.mi_event_record(self.h, stream), "mi_event_record")
+
+    def synchronize(self):
+        check(lib.mi_event_synchronize(self.h), "mi_event_synchronize")
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float()
+        check(lib.mi_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "mi_event_elapsed_ms")
+        return float(ms.value)
+
+    def destroy(self):
+        if self.h:
+            lib.mi_event_destroy(self.h)
+            self.h = None
+
+
+# ---- thin checked wrappers over the kernel entry points (DevBuf in, status checked) ----
+
+def fwht_quant(x, q, scale, block, stream=None):
+    M, K = x.shape
+    check(lib.mi_fwht_quant_f32_i8(x.ptr, q.ptr, scale.ptr, M, K, block, stream), "mi_fwht_quant_f32_i8")
+
+
+def fwht(x, out, block, stream=None):
+    M, K = x.shape
+    check(lib.mi_fwht_f32(x.ptr, out.ptr, M, K, block, stream), "mi_fwht_f32")
+
+
+def gemm_i32(qx, qw, acc, stream=None):
+    M, K = qx.shape
+    N = qw.shape[0]
+    check(lib.mi_w8a8_gemm_i32(qx.ptr, qw.ptr, acc.ptr, M, N, K, stream), "mi_w8a8_gemm_i32")
+
+
+def gemm_dequant(qx, sx, qw, sw, y, stream=None):
+    M, K = qx.shape
+    N = qw.shape[0]
+    check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, y.ptr, M, N, K, stream),
+          "mi_w8a8_gemm_dequant_f32")
+
+
+def dequant(acc, sx, sw, y, stream=None):
+    M, N = acc.shape
+    check(lib.mi_dequant_i32_f32(acc.ptr, sx.ptr, sw.ptr, y.ptr, M, N, stream), "mi_dequant_i32_f32")
+
+
+def linear(x, qw, sw, y, block, ws, stream=None):
+    M, K = x.shape
+    N = qw.shape[0]
+    check(lib.mi_w8a8_linear_f32(x.ptr, qw.ptr, sw.ptr, y.ptr, M, N, K, block, ws.ptr, ws.nbytes, stream),
+          "mi_w8a8_linear_f32")
+
+
+def gqa_decode(q, kq, ks, vq, vs, o, out_rotated, ws, stream=None):
+    B, Hq, D = q.shape
+    _, Hkv, T, _ = kq.shape
+    check(lib.mi_gqa_decode_attn(q.ptr, kq.ptr, ks.ptr, vq.ptr, vs.ptr, o.ptr, B, Hq, Hkv, D, T,
+                                 1 if out_rotated else 0, ws.ptr, ws.nbytes, stream), "mi_gqa_decode_attn")
+
+
+def gqa_scores(q, kq, ks, vq, vs, qq, sq, dots, ws, stream=None):
+    B, Hq, D = q.shape
+    _, Hkv, T, _ = kq.shape
+    check(lib.mi_gqa_decode_scores_i32(q.ptr, kq.ptr, ks.ptr, vq.ptr, vs.ptr, qq.ptr, sq.ptr, dots.ptr,
+                                       B, Hq, Hkv, D, T, ws.ptr, ws.nbytes, stream), "mi_gqa_decode_scores_i32")
+
+
+def moe_route(x, wr, idx, w, topk, stream=None):
+    T, H = x.shape
+    E = wr.shape[0]
+    check(lib.mi_moe_route(x.ptr, wr.ptr, idx.ptr, w.ptr, T, H, E, topk, stream), "mi_moe_route")
+
+
+def moe_dispatch(idx, perm, seg, E, stream=None):
+    T, topk = idx.shape
+    check(lib.mi_moe_dispatch(idx.ptr, perm.ptr, seg.ptr, T, E, topk, stream), "mi_moe_dispatch")
+
+
+def moe_ffn(x, idx, w, wg, sg, wu, su, wd, sd, y, ws, stream=None):
+    T, H = x.shape
+    E, I, _ = wg.shape
+    topk = idx.shape[1]
+    check(lib.mi_moe_ffn(x.ptr, idx.ptr, w.ptr, wg.ptr, sg.ptr, wu.ptr, su.ptr, wd.ptr, sd.ptr, y.ptr,
+                         T, H, I, E, topk, ws.ptr, ws.nbytes, stream), "mi_moe_ffn")
+
+
+def moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=None):
+    T, H = x.shape
+    E, I, _ = wg.shape
+    check(lib.mi_moe_layer(x.ptr, wr.ptr, wg.ptr, sg.ptr, wu.ptr, su.ptr, wd.ptr, sd.ptr, y.ptr,
+                           T, H, I, E, topk, ws.ptr, ws.nbytes, stream), "mi_moe_layer")

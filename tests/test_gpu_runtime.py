@@ -1,0 +1,188 @@
+"""Device arena and stream pool: the behaviours the upstream tests pin for
+NumaArena / ThreadPool (test_linux_threading.mojo:56-102, :164-215, :304-398),
+restated for device memory and streams."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def ctx(mi):
+    h = C.c_void_p()
+    mi.check(mi.lib.mi_ctx_create(0, C.byref(h)))
+    yield h
+    mi.lib.mi_ctx_destroy(h)
+
+
+def test_context_reports_gfx950(mi, ctx):
+    buf = C.create_string_buffer(64)
+    mi.check(mi.lib.mi_ctx_arch_name(ctx, buf, 64))
+    assert buf.value.startswith(b"gfx950")
+    assert mi.lib.mi_ctx_compute_units(ctx) >= 64
+    assert mi.lib.mi_ctx_memory_bytes(ctx) > (64 << 30)
+    bad = C.c_void_p()
+    assert mi.lib.mi_ctx_create(99, C.byref(bad)) == mi.ENODEV
+
+
+def test_arena_bump_marks_and_exhaustion(mi, ctx):
+    lib = mi.lib
+    a = C.c_void_p()
+    mi.check(lib.mi_arena_create(ctx, 1 << 20, 256, C.byref(a)))
+    assert lib.mi_arena_used(a) == 0 and lib.mi_arena_remaining(a) == 1 << 20
+    assert lib.mi_arena_verify_placement(a) == 1          # nothing allocated: true
+    p1 = lib.mi_arena_alloc(a, 100)
+    p2 = lib.mi_arena_alloc(a, 100)
+    assert p1 and p2 and p2 - p1 == 256 and p1 % 256 == 0  # aligned bump
+    assert lib.mi_arena_used(a) == 256 + 100
+    mark = lib.mi_arena_mark(a)
+    p3 = lib.mi_arena_alloc(a, 4096)
+    assert lib.mi_arena_reset_to(a, mark + 1 << 30) == mi.EINVAL   # beyond used: ignored
+    assert lib.mi_arena_reset_to(a, -1) == mi.EINVAL
+    assert lib.mi_arena_reset_to(a, mark) == mi.OK
+    assert lib.mi_arena_alloc(a, 4096) == p3                       # watermark restored
+    assert lib.mi_arena_alloc(a, 2 << 20) is None                  # exhausted: null, no error
+    assert lib.mi_arena_verify_placement(a) == 1
+    # fresh arena memory reads as zero
+    host = np.ones(64, np.uint32)
+    mi.check(lib.mi_memcpy_d2h(host.ctypes.data, p1, host.nbytes, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    assert not host.any()
+    lib.mi_arena_reset(a)
+    assert lib.mi_arena_used(a) == 0
+    bad = C.c_void_p()
+    assert lib.mi_arena_create(ctx, 1 << 20, 48, C.byref(bad)) == mi.EINVAL   # alignment not a power of two
+    mi.check(lib.mi_arena_destroy(a))
+
+
+def test_stream_pool_launch_wait_all_and_reuse(mi, ctx):
+    """32 launches on a pool of 4 in batches, as test_thread_pool / test_pool_reuse."""
+    lib = mi.lib
+    pool, a = C.c_void_p(), C.c_void_p()
+    mi.check(lib.mi_stream_pool_create(ctx, 4, C.byref(pool)))
+    mi.check(lib.mi_arena_create(ctx, 1 << 20, 256, C.byref(a)))
+    assert lib.mi_stream_pool_capacity(pool) == 4
+    buf = lib.mi_arena_alloc(a, 32 * 4096)
+    for batch in range(8):
+        for i in range(4):
+            slot = lib.mi_stream_pool_begin(pool)
+            assert slot >= 0
+            k = batch * 4 + i
+            mi.check(lib.mi_fill_u32(buf + k * 4096, 2 * k * k, 1024, lib.mi_stream_pool_stream(pool, slot)))
+            mi.check(lib.mi_stream_pool_end(pool, slot))
+        mi.check(lib.mi_stream_pool_wait_all(pool))
+    host = np.empty(32 * 1024, np.uint32)
+    mi.check(lib.mi_memcpy_d2h(host.ctypes.data, buf, host.nbytes, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    assert np.array_equal(host.reshape(32, 1024)[:, 0], 2 * np.arange(32, dtype=np.uint32) ** 2)
+    assert lib.mi_stream_pool_wait_any(pool) == -1       # nothing in flight
+    mi.check(lib.mi_stream_pool_destroy(pool))
+    mi.check(lib.mi_arena_destroy(a))
+
+
+def test_stream_pool_full_wait_any_and_busy_destroy(mi, ctx):
+    lib = mi.lib
+    pool, a, gate = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    mi.check(lib.mi_stream_pool_create(ctx, 2, C.byref(pool)))
+    mi.check(lib.mi_arena_create(ctx, 64 << 20, 256, C.byref(a)))
+    mi.check(lib.mi_gate_create(ctx, C.byref(gate)))
+    assert lib.mi_gate_wait(gate, None) == mi.EINVAL      # never released
+    big = lib.mi_arena_alloc(a, 48 << 20)
+    done = []
+    launched = 0
+    for it in range(50):                                  # launch-all / wait-any / wait-all, as test_wait_any_reuse
+        while True:
+            slot = lib.mi_stream_pool_begin(pool)
+            if slot < 0:
+                assert slot == mi.EBUSY
+                break
+            s = lib.mi_stream_pool_stream(pool, slot)
+            mi.check(lib.mi_fill_u32(big, it, (48 << 20) // 4, s))
+            mi.check(lib.mi_stream_pool_end(pool, slot))
+            launched += 1
+            if launched % 2 == 0:
+                break
+        got = lib.mi_stream_pool_wait_any(pool)
+        assert got in (0, 1)
+        done.append(got)
+        mi.check(lib.mi_stream_pool_wait_all(pool))
+    assert launched == 100
+    # destroy while busy is refused, not fatal
+    slot = lib.mi_stream_pool_begin(pool)
+    s = lib.mi_stream_pool_stream(pool, slot)
+    for _ in range(20):
+        mi.check(lib.mi_fill_u32(big, 7, (48 << 20) // 4, s))
+    mi.check(lib.mi_gate_release(gate, s))
+    mi.check(lib.mi_stream_pool_end(pool, slot))
+    rc = lib.mi_stream_pool_destroy(pool)
+    assert rc in (mi.EBUSY, mi.OK)
+    if rc == mi.EBUSY:
+        mi.check(lib.mi_gate_wait_host(gate))
+        mi.check(lib.mi_stream_pool_wait_all(pool))
+        mi.check(lib.mi_stream_pool_destroy(pool))
+    mi.check(lib.mi_gate_reset(gate))
+    assert lib.mi_gate_wait_host(gate) == mi.EINVAL
+    mi.check(lib.mi_gate_destroy(gate))
+    mi.check(lib.mi_arena_destroy(a))
+
+
+def test_gate_orders_two_streams(mi, ctx):
+    """Chain reduce across streams: each stage waits on the previous stage's
+    gate, as the NUMA ring reduce waits on futex gates (test_linux_threading.mojo:400-476)."""
+    lib = mi.lib
+    n = 4
+    pool, a = C.c_void_p(), C.c_void_p()
+    mi.check(lib.mi_stream_pool_create(ctx, n, C.byref(pool)))
+    mi.check(lib.mi_arena_create(ctx, 1 << 20, 256, C.byref(a)))
+    gates = []
+    buf = lib.mi_arena_alloc(a, 4096)
+    stage = lib.mi_arena_alloc(a, 4096)
+    for i in range(n):
+        g = C.c_void_p()
+        mi.check(lib.mi_gate_create(ctx, C.byref(g)))
+        gates.append(g)
+    for i in range(n):
+        slot = lib.mi_stream_pool_begin(pool)
+        s = lib.mi_stream_pool_stream(pool, slot)
+        if i:
+            mi.check(lib.mi_gate_wait(gates[i - 1], s))
+        mi.check(lib.mi_fill_u32(stage, i + 1, 1024, s))        # each stage overwrites: order matters
+        mi.check(lib.mi_memcpy_d2d(buf, stage, 4096, s))
+        mi.check(lib.mi_gate_release(gates[i], s))
+        mi.check(lib.mi_stream_pool_end(pool, slot))
+    mi.check(lib.mi_stream_pool_wait_all(pool))
+    host = np.empty(1024, np.uint32)
+    mi.check(lib.mi_memcpy_d2h(host.ctypes.data, buf, 4096, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    assert np.all(host == n)
+    for g in gates:
+        lib.mi_gate_destroy(g)
+    mi.check(lib.mi_stream_pool_destroy(pool))
+    mi.check(lib.mi_arena_destroy(a))
+
+
+def test_pinned_host_staging_and_events(mi, ctx):
+    lib = mi.lib
+    p = lib.mi_host_alloc(1 << 20)
+    assert p
+    a = C.c_void_p()
+    mi.check(lib.mi_arena_create(ctx, 2 << 20, 256, C.byref(a)))
+    d = lib.mi_arena_alloc(a, 1 << 20)
+    src = (C.c_uint8 * (1 << 20)).from_address(p)
+    C.memset(p, 0x5a, 1 << 20)
+    e0, e1 = mi.Event(), mi.Event()
+    e0.record()
+    mi.check(lib.mi_memcpy_h2d(d, p, 1 << 20, None))
+    C.memset(p, 0, 0)
+    e1.record()
+    e1.synchronize()
+    assert e0.elapsed_ms(e1) >= 0.0
+    back = np.zeros(1 << 20, np.uint8)
+    mi.check(lib.mi_memcpy_d2h(back.ctypes.data, d, 1 << 20, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    assert np.all(back == 0x5a) and src[0] == 0x5a
+    e0.destroy(); e1.destroy()
+    mi.check(lib.mi_host_free(p))
+    mi.check(lib.mi_arena_destroy(a))
