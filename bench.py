@@ -1,0 +1,351 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 inference hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" = the prefill workload (cfg3): the four Llama-8B-style rotated W8A8
+linears at M = 2048 tokens (4096->6144, 4096->14336 twice, 14336->4096), each
+= block-128 Hadamard rotation + per-token int8 quantization of the fp32
+activations, int8 MFMA GEMM against pre-rotated pre-quantized weights, fp32
+dequant.  Inputs are resident in HBM before the timed region.  `value` is
+int8 TOPS over the whole step (rotate/quant prologue included).
+
+The same run also reports, under "sub_metrics": the GEMM kernels alone, the
+decode GEMV sweep (cfg1), decode attention (cfg2), the MoE layer (cfg4) and
+the small linear (cfg0), each against its own roofline, with weight / KV
+buffers rotated through more than 256 MB so that the Infinity Cache cannot
+stand in for HBM; and "cpu_baseline": the CPU oracle timed on the host cores
+(a reported baseline, not a target).  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "mojo-linuxperiments_amd"))
+
+PEAK_INT8_TOPS = 5000.0     # dense int8 MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+MALL_BYTES = 256 << 20
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def host_topology():
+    """Core and NUMA node counts from the sysfs files the upstream NumaInfo reads
+    (numa/numa.mojo:107-115)."""
+    nodes = 1
+    try:
+        txt = open("/sys/devices/system/node/online").read().strip()
+        nodes = 0
+        for part in txt.split(","):
+            lo, _, hi = part.partition("-")
+            nodes += int(hi or lo) - int(lo) + 1
+    except OSError:
+        pass
+    return {"cores": len(os.sched_getaffinity(0)), "numa_nodes": nodes}
+
+
+class Timer:
+    def __init__(self, mi, stream):
+        self.mi, self.stream = mi, stream
+        self.e0, self.e1 = mi.Event(), mi.Event()
+
+    def run(self, fn, reps):
+        """ms per call of fn(), timed with HIP events on the launch stream."""
+        self.mi.check(self.mi.lib.mi_stream_synchronize(self.stream))
+        self.e0.record(self.stream)
+        for _ in range(reps):
+            fn()
+        self.e1.record(self.stream)
+        self.e1.synchronize()
+        return self.e0.elapsed_ms(self.e1) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-sub", action="store_true", help="only the headline workload")
+    ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
+
+    import mi355_int8 as mi     # fails loudly when the HIP library is not built
+    import workload as wl
+
+    dev = mi.Device(arena_bytes=12 << 30)
+    pool = mi.StreamPool(dev, 1)
+    s = pool.stream(0)
+    timer = Timer(mi, s)
+    lib = mi.lib
+    M = wl.PREFILL_M
+
+    # ---- weights: one fp32 matrix per shape from the seed, prepared on the GPU,
+    # then replicated to distinct addresses so that reuse across calls misses the cache
+    log("preparing weights ...")
+    shapes = {}
+    for name, K, N in wl.PROJECTIONS:
+        if (K, N) in shapes:
+            continue
+        w = wl.weights(2025, N, K, stream=K + N)
+        mark = dev.mark()
+        dw = dev.upload(w)
+        q0, s0 = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+        mi.fwht_quant(dw, q0, s0, wl.HADAMARD_BLOCK)
+        dev.sync()
+        qh, sh = dev.download(q0), dev.download(s0)
+        dev.reset_to(mark)
+        copies = MALL_BYTES // (N * K) + 2
+        bufs = []
+        for _ in range(copies):
+            bufs.append((dev.upload(qh), dev.upload(sh)))
+        shapes[(K, N)] = bufs
+        del w
+    acts = {K: dev.upload(wl.activations(2025, M, K, stream=K)) for K in (4096, 14336)}
+    ybuf = dev.empty((M, 14336), np.float32)
+    lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(M, 14336, 14336), np.uint8)
+    dev.sync()
+
+    counters = {k: 0 for k in shapes}
+
+    def next_w(K, N):
+        bufs = shapes[(K, N)]
+        counters[(K, N)] = (counters[(K, N)] + 1) % len(bufs)
+        return bufs[counters[(K, N)]]
+
+    def prefill_step():
+        for name, K, N in wl.PROJECTIONS:
+            qw, sw = next_w(K, N)
+            mi.check(lib.mi_w8a8_linear_f32(acts[K].ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, wl.HADAMARD_BLOCK,
+                                            lin_ws.ptr, lin_ws.nbytes, s))
+
+    log("headline: prefill step x%d (+%d warm-up)" % (args.steps, args.warmup))
+    for _ in range(args.warmup):
+        prefill_step()
+    dev.sync(s)
+    t0 = time.perf_counter()
+    ms_step = timer.run(prefill_step, args.steps)
+    dev.sync(s)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    step_ops = sum(wl.gemm_ops(M, N, K) for _, K, N in wl.PROJECTIONS)
+    value = step_ops / (ms_step * 1e-3) / 1e12
+
+    # ---- the dominant kernel alone: the tiled MFMA GEMM on already-quantized activations
+    gemm_ms = {}
+    qx = {K: dev.empty((M, K), np.int8) for K in (4096, 14336)}
+    sx = {K: dev.empty(M, np.float32) for K in (4096, 14336)}
+    for K in qx:
+        mi.fwht_quant(acts[K], qx[K], sx[K], wl.HADAMARD_BLOCK, stream=s)
+    quant_ms = {K: timer.run(lambda K=K: mi.fwht_quant(acts[K], qx[K], sx[K], wl.HADAMARD_BLOCK, stream=s), 20)
+                for K in qx}
+    for name, K, N in wl.PROJECTIONS:
+        def one(K=K, N=N):
+            qw, sw = next_w(K, N)
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx[K].ptr, sx[K].ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, s))
+        timer.run(one, 5)
+        gemm_ms[name] = timer.run(one, max(10, args.steps))
+    gemm_total_ms = sum(gemm_ms.values())
+    gemm_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "k_w8a8_tiled (v_mfma_i32_16x16x64_i8), four cfg3 shapes, ops-weighted",
+        "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+        "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": None,
+        "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
+        "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
+                           for name, K, N in wl.PROJECTIONS},
+    }
+
+    out = {
+        "metric": "W8A8 GEMM int8 TOPS & decode GB/s (% roofline) @1 GPU; vs CPU host cores",
+        "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "cfg3 prefill: 4 rotated W8A8 linears (4096->6144, 4096->14336 x2, 14336->4096) "
+                               "at M=2048, Hadamard block 128, rotate+quant prologue included",
+                   "tokens": M, "ops_per_step": step_ops, "tokens_per_s": round(M / (ms_step * 1e-3), 1),
+                   "wall_ms_per_step": round(wall_ms, 4)},
+        "roofline": roofline,
+        "host": host_topology(),
+    }
+
+    sub = {"prefill_quant_prologue_us": {str(K): round(v * 1e3, 2) for K, v in quant_ms.items()}}
+    if not args.skip_sub:
+        sub.update(decode_gemv(mi, wl, dev, pool, s, timer, shapes, next_w))
+        sub.update(decode_attention(mi, wl, dev, s, timer))
+        sub.update(moe_layer(mi, wl, dev, s, timer))
+        sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
+    out["sub_metrics"] = sub
+    if not args.skip_cpu:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(out), flush=True)
+    pool.destroy()
+    dev.close()
+
+
+def graph_time(mi, dev, s, timer, calls, reps):
+    """Per-call ms of a list of closures recorded once into a graph and replayed
+    (decode kernels are a few microseconds: eager launches from Python would
+    measure the interpreter)."""
+    for c in calls:
+        c()
+    dev.sync(s)
+    with mi.Graph.capture(s) as g:
+        for c in calls:
+            c()
+    g.launch()
+    dev.sync(s)
+    ms = timer.run(lambda: g.launch(), reps) / len(calls)
+    g.destroy()
+    return ms
+
+
+def decode_gemv(mi, wl, dev, pool, s, timer, shapes, next_w):
+    """cfg1: M in {1,4,16} x the four projections; weights rotate through > 256 MB."""
+    lib = mi.lib
+    res = {}
+    layer_ms = {}
+    for Mb in wl.DECODE_BATCHES:
+        mark = dev.mark()
+        per = {}
+        for name, K, N in wl.PROJECTIONS:
+            x = wl.activations(77, Mb, K)
+            dx = dev.upload(x)
+            qx, sx = dev.empty((Mb, K), np.int8), dev.empty(Mb, np.float32)
+            y = dev.empty((Mb, N), np.float32)
+            mi.fwht_quant(dx, qx, sx, wl.HADAMARD_BLOCK, stream=s)
+            bufs = shapes[(K, N)]
+            calls = [(lambda b=b: mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, b[0].ptr, b[1].ptr, y.ptr,
+                                                                       Mb, N, K, s))) for b in bufs]
+            ms = graph_time(mi, dev, s, timer, calls, 20)
+            ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(Mb, N, K), np.uint8)
+            calls2 = [(lambda b=b: mi.check(lib.mi_w8a8_linear_f32(dx.ptr, b[0].ptr, b[1].ptr, y.ptr, Mb, N, K,
+                                                                  wl.HADAMARD_BLOCK, ws.ptr, ws.nbytes, s)))
+                      for b in bufs]
+            ms2 = graph_time(mi, dev, s, timer, calls2, 20)
+            nbytes = wl.linear_algorithmic_bytes(Mb, N, K)
+            per[name] = {"gemv_us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                         "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "TOPS": round(wl.gemm_ops(Mb, N, K) / (ms * 1e-3) / 1e12, 2),
+                         "linear_with_quant_us": round(ms2 * 1e3, 2)}
+        total_ms = sum(v["linear_with_quant_us"] for v in per.values()) * 1e-3
+        per["tokens_per_s_four_projections"] = round(Mb / (total_ms * 1e-3), 1)
+        res["M%d" % Mb] = per
+        dev.reset_to(mark)
+    return {"cfg1_decode_gemv": res}
+
+
+def decode_attention(mi, wl, dev, s, timer):
+    """cfg2: B=16, 32/8 heads, D=128, T=4096; three KV sets (402 MB) in rotation."""
+    lib = mi.lib
+    c = wl.ATTN
+    B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
+    mark = dev.mark()
+    rows = B * Hkv * T
+    sets = []
+    src = dev.upload(wl.normal(88, (rows, D), 0))
+    for i in range(3):
+        kq, ks = dev.empty((B, Hkv, T, D), np.int8), dev.empty((B, Hkv, T), np.float32)
+        vq, vs = dev.empty((B, Hkv, T, D), np.int8), dev.empty((B, Hkv, T), np.float32)
+        mi.check(lib.mi_fwht_quant_f32_i8(src.ptr, kq.ptr, ks.ptr, rows, D, D, s))
+        mi.check(lib.mi_fwht_quant_f32_i8(src.ptr, vq.ptr, vs.ptr, rows, D, D, s))
+        sets.append((kq, ks, vq, vs))
+    dq = dev.upload(wl.normal(88, (B, Hq, D), 1))
+    do = dev.empty((B, Hq, D), np.float32)
+    ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T), np.uint8)
+    calls = [(lambda k=k: mi.gqa_decode(dq, k[0], k[1], k[2], k[3], do, False, ws, stream=s)) for k in sets]
+    ms = graph_time(mi, dev, s, timer, calls, 20)
+    nbytes = wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
+    dev.reset_to(mark)
+    return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                      "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                      "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes}}
+
+
+def moe_layer(mi, wl, dev, s, timer):
+    """cfg4: 512 tokens, hidden 2048, 128 experts top-8, inner 768 (604 MB of expert weights)."""
+    lib = mi.lib
+    c = wl.MOE
+    T, H, E, topk, I = c["T"], c["H"], c["E"], c["topk"], c["I"]
+    mark = dev.mark()
+    x = dev.upload(wl.activations(99, T, H))
+    wr = dev.upload(wl.weights(99, E, H, 1))
+
+    def prep(n, k, b, stream):
+        w = dev.upload(wl.weights(99, E * n, k, stream))
+        q, sc = dev.empty((E, n, k), np.int8), dev.empty((E, n), np.float32)
+        mi.check(lib.mi_fwht_quant_f32_i8(w.ptr, q.ptr, sc.ptr, E * n, k, b, s))
+        return q, sc
+    wg, sg = prep(I, H, wl.HADAMARD_BLOCK, 2)
+    wu, su = prep(I, H, wl.HADAMARD_BLOCK, 3)
+    wd, sd = prep(H, I, wl.MOE_INNER_BLOCK, 4)
+    y = dev.empty((T, H), np.float32)
+    ws = dev.empty(lib.mi_moe_layer_workspace_bytes(T, H, I, E, topk), np.uint8)
+    call = lambda: mi.moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=s)
+    ms = graph_time(mi, dev, s, timer, [call], 20)
+    wbytes = wl.moe_weight_bytes(E, H, I)
+    ops = wl.moe_ops(T, topk, H, I)
+    dev.reset_to(mark)
+    return {"cfg4_moe_layer": {"us": round(ms * 1e3, 2), "GBps": round(wbytes / (ms * 1e-3) / 1e9, 1),
+                               "hbm_frac": round(wbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                               "TOPS": round(ops / (ms * 1e-3) / 1e12, 2),
+                               "tokens_per_s": round(T / (ms * 1e-3), 1), "weight_bytes": wbytes}}
+
+
+def cfg0_linear(mi, wl, dev, s, timer, shapes):
+    lib = mi.lib
+    c = wl.CFG0
+    M, K, N = c["M"], c["K"], c["N"]
+    mark = dev.mark()
+    w = dev.upload(wl.weights(5, N, K))
+    q0, s0 = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+    mi.fwht_quant(w, q0, s0, wl.HADAMARD_BLOCK, stream=s)
+    dev.sync(s)
+    qh, sh = dev.download(q0, s), dev.download(s0, s)
+    bufs = [(dev.upload(qh), dev.upload(sh)) for _ in range(MALL_BYTES // (N * K) + 2)]
+    dx = dev.upload(wl.activations(5, M, K))
+    y = dev.empty((M, N), np.float32)
+    ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(M, N, K), np.uint8)
+    calls = [(lambda b=b: mi.check(lib.mi_w8a8_linear_f32(dx.ptr, b[0].ptr, b[1].ptr, y.ptr, M, N, K,
+                                                         wl.HADAMARD_BLOCK, ws.ptr, ws.nbytes, s))) for b in bufs]
+    ms = graph_time(mi, dev, s, timer, calls, 20)
+    nbytes = wl.linear_algorithmic_bytes(M, N, K)
+    dev.reset_to(mark)
+    return {"cfg0_linear_m32": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                "TOPS": round(wl.gemm_ops(M, N, K) / (ms * 1e-3) / 1e12, 2)}}
+
+
+def cpu_baseline(wl):
+    """The CPU oracle (a builder-written port; upstream has no CPU kernels for
+    this path) on the host cores: rotate+quant of X [2048,4096] and the int8
+    GEMM against the first 1536 of the 6144 QKV output channels."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import cpu_oracle as orc
+    M, K, N = wl.PREFILL_M, 4096, 1536
+    x = wl.activations(1, M, K)
+    g = np.random.default_rng(3)
+    qw = g.integers(-127, 128, (N, K)).astype(np.int8)
+    sw = np.full(N, 0.001, np.float32)
+    orc.rotate_quant_rows(x[:64], 128)          # load the library, spin up the OpenMP team
+    t0 = time.perf_counter()
+    y, qx, sx, acc = orc.w8a8_linear(x, qw, sw, 128)
+    dt = time.perf_counter() - t0
+    ops = wl.gemm_ops(M, N, K)
+    topo = host_topology()
+    return {"value": round(ops / dt / 1e12, 4), "unit": "TOPS", "cores": orc.num_threads(), "kind": "port",
+            "numa_nodes": topo["numa_nodes"],
+            "sample": "cfg3 QKV linear, M=2048 K=4096, first 1536 of 6144 output channels "
+                      "(rotate+quant + int8 GEMM + dequant), %.2f s, OpenMP + auto-vectorized C" % dt}
+
+
+if __name__ == "__main__":
+    main()

@@ -110,6 +110,19 @@ MI_API int32_t mi_gate_wait(mi_gate *g, void *stream);         /* linux_threadin
 MI_API int32_t mi_gate_wait_host(mi_gate *g);                  /* the calling host thread waits */
 MI_API int32_t mi_gate_reset(mi_gate *g);                      /* linux_threading.mojo:196-198 */
 
+/* ---- graphs ------------------------------------------------------------------
+ * Decode-time chains of small kernels are launch-bound; a caller records the
+ * chain once on a pool stream and replays it.  Every kernel entry point of
+ * this library may be called between begin and end (none of them allocates,
+ * synchronizes or records a memset node); call each one once eagerly first so
+ * that one-time kernel attributes are already set.  No upstream counterpart:
+ * a thread pool has no launch cost to amortize. */
+typedef struct mi_graph mi_graph;
+MI_API int32_t mi_graph_capture_begin(void *stream);           /* stream must not be the null stream */
+MI_API int32_t mi_graph_capture_end(void *stream, mi_graph **out);
+MI_API int32_t mi_graph_launch(mi_graph *g, void *stream);
+MI_API int32_t mi_graph_destroy(mi_graph *g);
+
 /* ---- copies, host staging, events ----------------------------------------- */
 MI_API int32_t mi_memcpy_h2d(void *dst_dev, const void *src_host, int64_t bytes, void *stream);
 MI_API int32_t mi_memcpy_d2h(void *dst_host, const void *src_dev, int64_t bytes, void *stream);
@@ -185,12 +198,12 @@ MI_API int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const 
 /* ---- a9: MoE router: logits = x . wr^T in a fixed fp32 order, top-k on the
  * logits (ties to the lower expert), weights = softmax over the k picks.
  * x fp32 [T,H], wr fp32 [E,H] -> idx int32 [T,topk], w fp32 [T,topk].
- * H % 256 == 0, E <= 256, topk <= 8. */
+ * H % 256 == 0, E % 16 == 0, E <= 256, topk <= 8. */
 MI_API int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, float *w,
                             int64_t T, int64_t H, int64_t E, int32_t topk, void *stream);
 /* ---- a10: stable grouping of the T*topk (token,slot) pairs by expert.
  * idx int32 [T,topk] -> perm int32 [T*topk] (perm[pos] = pair = token*topk+slot),
- * seg_off int32 [E+1].  E * ceil(T/32) <= 16384. */
+ * seg_off int32 [E+1].  2 * E * ceil(T/32) + E + 1 <= 36864 (the bitmaps live in LDS). */
 MI_API int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off,
                                int64_t T, int64_t E, int32_t topk, void *stream);
 /* ---- a11: grouped expert SwiGLU FFN over expert-sorted segments.
@@ -206,7 +219,8 @@ MI_API int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w,
 /* Byte offsets into the mi_moe_ffn workspace, for gates that inspect the
  * intermediates: which = 0 qx int8[T,H], 1 sx f32[T], 2 perm i32[T*topk],
  * 3 seg_off i32[E+1], 4 h f32[T*topk,I] (sorted order), 5 hq int8[T*topk,I],
- * 6 hs f32[T*topk], 7 out f32[T*topk,H] (pair order).  Negative on error. */
+ * 6 hs f32[T*topk], 7 out f32[T*topk,H] (pair order), 8 idx i32[T,topk] and
+ * 9 w f32[T,topk] (filled by mi_moe_layer only).  Negative on error. */
 MI_API int64_t mi_moe_ffn_workspace_offset(int32_t which, int64_t T, int64_t H, int64_t I,
                                            int64_t E, int32_t topk);
 /* Router + dispatch + FFN in one call (routing results land in the workspace). */

@@ -72,6 +72,11 @@ struct mi_event {
     hipEvent_t ev;
 };
 
+struct mi_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
 extern "C" {
 
 const char *mi_status_string(int32_t s)
@@ -390,6 +395,48 @@ int32_t mi_gate_reset(mi_gate *g)
 {
     if (!g) return MI_EINVAL;
     g->released = false;
+    return MI_OK;
+}
+
+/* ---- graphs -------------------------------------------------------------------- */
+
+int32_t mi_graph_capture_begin(void *stream)
+{
+    if (!stream) return MI_EINVAL;
+    MI_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return MI_OK;
+}
+
+int32_t mi_graph_capture_end(void *stream, mi_graph **out)
+{
+    if (!out) return MI_EINVAL;
+    *out = nullptr;
+    if (!stream) return MI_EINVAL;
+    hipGraph_t graph = nullptr;
+    MI_HIP(hipStreamEndCapture(as_stream(stream), &graph));
+    if (!graph) return MI_EINVAL;
+    mi_graph *g = new (std::nothrow) mi_graph;
+    if (!g) { (void)hipGraphDestroy(graph); return MI_ENOMEM; }
+    g->graph = graph;
+    hipError_t e = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) { (void)hipGraphDestroy(graph); delete g; return hip_fail(e); }
+    *out = g;
+    return MI_OK;
+}
+
+int32_t mi_graph_launch(mi_graph *g, void *stream)
+{
+    if (!g) return MI_EINVAL;
+    MI_HIP(hipGraphLaunch(g->exec, as_stream(stream)));
+    return MI_OK;
+}
+
+int32_t mi_graph_destroy(mi_graph *g)
+{
+    if (!g) return MI_EINVAL;
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    delete g;
     return MI_OK;
 }
 

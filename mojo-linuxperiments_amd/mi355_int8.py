@@ -62,6 +62,10 @@ SIGNATURES = {
     "mi_gate_wait": (i32, [vp, vp]),
     "mi_gate_wait_host": (i32, [vp]),
     "mi_gate_reset": (i32, [vp]),
+    "mi_graph_capture_begin": (i32, [vp]),
+    "mi_graph_capture_end": (i32, [vp, C.POINTER(vp)]),
+    "mi_graph_launch": (i32, [vp, vp]),
+    "mi_graph_destroy": (i32, [vp]),
     "mi_memcpy_h2d": (i32, [vp, vp, i64, vp]),
     "mi_memcpy_d2h": (i32, [vp, vp, i64, vp]),
     "mi_memcpy_d2d": (i32, [vp, vp, i64, vp]),
@@ -84,6 +88,13 @@ SIGNATURES = {
     "mi_gqa_decode_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
     "mi_gqa_decode_attn": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
+    "mi_moe_route": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "mi_moe_dispatch": (i32, [vp, vp, vp, i64, i64, i32, vp]),
+    "mi_moe_ffn_workspace_bytes": (i64, [i64, i64, i64, i64, i32]),
+    "mi_moe_ffn": (i32, [vp] * 10 + [i64, i64, i64, i64, i32, vp, i64, vp]),
+    "mi_moe_ffn_workspace_offset": (i64, [i32, i64, i64, i64, i64, i32]),
+    "mi_moe_layer": (i32, [vp] * 9 + [i64, i64, i64, i64, i32, vp, i64, vp]),
+    "mi_moe_layer_workspace_bytes": (i64, [i64, i64, i64, i64, i32]),
 }
 
 _missing = []
@@ -210,6 +221,67 @@ class Event:
     def destroy(self):
         if self.h:
             lib.mi_event_destroy(self.h)
+            self.h = None
+
+
+class StreamPool:
+    """Fixed-capacity pool of streams; launch() mirrors ThreadPool.launch
+    (threading/linux_threading.mojo:103-121): first free slot or False."""
+
+    def __init__(self, dev, capacity):
+        self.h = vp()
+        check(lib.mi_stream_pool_create(dev.ctx, capacity, C.byref(self.h)), "mi_stream_pool_create")
+
+    def stream(self, slot):
+        return lib.mi_stream_pool_stream(self.h, slot)
+
+    def launch(self, fn, *args):
+        slot = lib.mi_stream_pool_begin(self.h)
+        if slot < 0:
+            return False
+        fn(*args, stream=self.stream(slot))
+        check(lib.mi_stream_pool_end(self.h, slot), "mi_stream_pool_end")
+        return True
+
+    def wait_all(self):
+        check(lib.mi_stream_pool_wait_all(self.h), "mi_stream_pool_wait_all")
+
+    def wait_any(self):
+        return lib.mi_stream_pool_wait_any(self.h)
+
+    def destroy(self):
+        if self.h:
+            check(lib.mi_stream_pool_destroy(self.h), "mi_stream_pool_destroy")
+            self.h = None
+
+
+class Graph:
+    """Record the calls made inside `with Graph.capture(stream) as g:` and replay them."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.h = vp()
+
+    @classmethod
+    def capture(cls, stream):
+        return cls(stream)
+
+    def __enter__(self):
+        check(lib.mi_graph_capture_begin(self.stream), "mi_graph_capture_begin")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = lib.mi_graph_capture_end(self.stream, C.byref(self.h))
+        if exc_type is None:
+            check(rc, "mi_graph_capture_end")
+        return False
+
+    def launch(self, stream=None):
+        check(lib.mi_graph_launch(self.h, stream if stream is not None else self.stream), "mi_graph_launch")
+
+    def destroy(self):
+        if self.h:
+            lib.mi_graph_destroy(self.h)
             self.h = None
 
 

@@ -186,3 +186,40 @@ def test_pinned_host_staging_and_events(mi, ctx):
     e0.destroy(); e1.destroy()
     mi.check(lib.mi_host_free(p))
     mi.check(lib.mi_arena_destroy(a))
+
+
+def test_graph_replays_match_eager(mi, dev, orc):
+    """A captured rotate+quant -> GEMM -> dequant chain replayed four times with
+    new inputs between replays; every replay must equal the eager result."""
+    import workload
+    M, K, N = 16, 1024, 256
+    mark = dev.mark()
+    pool = mi.StreamPool(dev, 1)
+    s = pool.stream(0)
+    w = workload.weights(71, N, K)
+    dqw, dsw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+    mi.fwht_quant(dev.upload(w), dqw, dsw, 128)
+    dev.sync()                       # pool streams do not order against the null stream
+    dx = dev.upload(workload.activations(72, M, K))
+    ws = dev.empty(mi.lib.mi_w8a8_linear_workspace_bytes(M, N, K), np.uint8)
+    dy, dy_eager = dev.empty((M, N), np.float32), dev.empty((M, N), np.float32)
+    mi.linear(dx, dqw, dsw, dy_eager, 128, ws, stream=s)      # eager warm-up sets kernel attributes
+    dev.sync(s)
+    with mi.Graph.capture(s) as g:
+        mi.linear(dx, dqw, dsw, dy, 128, ws, stream=s)
+    for rep in range(4):
+        x = workload.activations(100 + rep, M, K)
+        mi.check(mi.lib.mi_memcpy_h2d(dx.ptr, x.ctypes.data, x.nbytes, s))
+        dev.sync(s)
+        mi.linear(dx, dqw, dsw, dy_eager, 128, ws, stream=s)
+        dev.sync(s)
+        want = dev.download(dy_eager, s)
+        mi.check(mi.lib.mi_fill_u32(dy.ptr, 0x7fc00000, M * N, s))     # poison the output
+        g.launch()
+        dev.sync(s)
+        got = dev.download(dy, s)
+        assert np.array_equal(got, want), rep
+    g.destroy()
+    pool.destroy()
+    assert mi.lib.mi_graph_capture_begin(None) == mi.EINVAL
+    dev.reset_to(mark)
