@@ -1,0 +1,199 @@
+// C++ host layer over the C ABI (include/mi355_int8.h).
+//
+// The upstream library is Mojo and its host types are move-only RAII structs
+// that report failure through `__bool__`, null pointers and Bool returns
+// (threading/numa_arena.mojo:6, :32-38, :46-52; threading/linux_threading.mojo:43,
+// :70-80, :103-121).  No Mojo toolchain exists where this is built, so the same
+// surface is written in C++: DeviceArena mirrors NumaArena, StreamPool mirrors
+// ThreadPool, Gate mirrors MutexGate, and QuantLinear / DecodeAttention /
+// MoeFfn are the quantize / linear / attention / MoE call surface that a Mojo
+// host would hold as structs over the same handles.  Nothing here throws.
+#pragma once
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <utility>
+
+#include "../../include/mi355_int8.h"
+
+namespace mi355 {
+
+class Context {
+public:
+    explicit Context(int device = 0) { if (mi_ctx_create(device, &h_) != MI_OK) h_ = nullptr; }
+    ~Context() { if (h_) mi_ctx_destroy(h_); }
+    Context(Context &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    explicit operator bool() const { return h_ != nullptr; }
+    mi_ctx *handle() const { return h_; }
+    int compute_units() const { return h_ ? mi_ctx_compute_units(h_) : 0; }
+
+private:
+    mi_ctx *h_ = nullptr;
+};
+
+// NumaArena[alignment] -> DeviceArena<Alignment> (numa_arena.mojo:5-87)
+template <int64_t Alignment = 256>
+class DeviceArena {
+public:
+    DeviceArena(const Context &ctx, int64_t size) : size_(size)
+    {
+        if (!ctx || mi_arena_create(ctx.handle(), size, Alignment, &h_) != MI_OK) { h_ = nullptr; size_ = 0; }
+    }
+    ~DeviceArena() { if (h_) mi_arena_destroy(h_); }
+    DeviceArena(DeviceArena &&o) noexcept : h_(o.h_), size_(o.size_) { o.h_ = nullptr; o.size_ = 0; }
+    DeviceArena(const DeviceArena &) = delete;
+    DeviceArena &operator=(const DeviceArena &) = delete;
+    explicit operator bool() const { return h_ != nullptr; }
+
+    // Pointer to uninitialized device memory, or nullptr if the arena is exhausted.
+    template <typename T>
+    T *alloc(int64_t count = 1) { return h_ ? static_cast<T *>(mi_arena_alloc(h_, count * (int64_t)sizeof(T))) : nullptr; }
+    int64_t mark() const { return h_ ? mi_arena_mark(h_) : 0; }
+    void reset_to(int64_t watermark) { if (h_) (void)mi_arena_reset_to(h_, watermark); }
+    void reset() { if (h_) (void)mi_arena_reset(h_); }
+    int64_t remaining() const { return h_ ? mi_arena_remaining(h_) : 0; }
+    int64_t used() const { return h_ ? mi_arena_used(h_) : 0; }
+    bool verify_placement() const { return !h_ || mi_arena_verify_placement(h_) == 1; }
+
+private:
+    mi_arena *h_ = nullptr;
+    int64_t size_ = 0;
+};
+
+// MutexGate (linux_threading.mojo:174-198): trivially copyable token over a handle.
+struct Gate {
+    mi_gate *h = nullptr;
+    static Gate create(const Context &ctx) { Gate g; if (mi_gate_create(ctx.handle(), &g.h) != MI_OK) g.h = nullptr; return g; }
+    void destroy() { if (h) mi_gate_destroy(h); h = nullptr; }
+    bool release(void *stream) const { return mi_gate_release(h, stream) == MI_OK; }
+    bool wait(void *stream) const { return mi_gate_wait(h, stream) == MI_OK; }
+    bool wait_host() const { return mi_gate_wait_host(h) == MI_OK; }
+    void reset() const { (void)mi_gate_reset(h); }
+};
+
+// ThreadPool (linux_threading.mojo:43-158): launch / wait_all / wait_any over streams.
+class StreamPool {
+public:
+    StreamPool(const Context &ctx, int capacity)
+    {
+        if (!ctx || mi_stream_pool_create(ctx.handle(), capacity, &h_) != MI_OK) h_ = nullptr;
+    }
+    ~StreamPool()
+    {
+        if (!h_) return;
+        if (mi_stream_pool_destroy(h_) == MI_EBUSY) {
+            // linux_threading.mojo:70-77: destroying a pool with live work is fatal
+            std::fputs("FATAL: StreamPool destroyed with work in flight\n", stderr);
+            std::abort();
+        }
+    }
+    StreamPool(StreamPool &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    StreamPool(const StreamPool &) = delete;
+    StreamPool &operator=(const StreamPool &) = delete;
+    explicit operator bool() const { return h_ != nullptr; }
+    int size() const { return h_ ? mi_stream_pool_capacity(h_) : 0; }
+
+    // func(stream, args...) is enqueued on the first free slot; false when the
+    // pool is full or func reports a status other than MI_OK.  Never blocks.
+    template <typename F, typename... Args>
+    bool launch(F &&func, Args &&...args)
+    {
+        if (!h_) return false;
+        const int32_t slot = mi_stream_pool_begin(h_);
+        if (slot < 0) return false;
+        const int32_t rc = func(mi_stream_pool_stream(h_, slot), std::forward<Args>(args)...);
+        return mi_stream_pool_end(h_, slot) == MI_OK && rc == MI_OK;
+    }
+    void wait_all() { if (h_) (void)mi_stream_pool_wait_all(h_); }
+    int wait_any() { return h_ ? mi_stream_pool_wait_any(h_) : -1; }
+    void *stream(int slot) const { return h_ ? mi_stream_pool_stream(h_, slot) : nullptr; }
+
+private:
+    mi_stream_pool *h_ = nullptr;
+};
+
+// A Hadamard-rotated W8A8 linear layer with weights prepared once on the device.
+template <int Block = 128>
+struct QuantLinear {
+    int8_t *qw = nullptr;
+    float *sw = nullptr;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+    int64_t N = 0, K = 0, max_tokens = 0;
+
+    // w_dev: fp32 [N,K] in device memory.  false if the arena is exhausted.
+    template <typename Arena>
+    bool prepare(Arena &arena, const float *w_dev, int64_t n, int64_t k, int64_t max_m, void *stream)
+    {
+        N = n; K = k; max_tokens = max_m;
+        qw = arena.template alloc<int8_t>(n * k);
+        sw = arena.template alloc<float>(n);
+        workspace_bytes = mi_w8a8_linear_workspace_bytes(max_m, n, k);
+        workspace = workspace_bytes > 0 ? arena.template alloc<uint8_t>(workspace_bytes) : nullptr;
+        if (!qw || !sw || !workspace) return false;
+        return mi_fwht_quant_f32_i8(w_dev, qw, sw, n, k, Block, stream) == MI_OK;
+    }
+    // x fp32 [M,K] -> y fp32 [M,N]; status as in the C ABI
+    int32_t forward(const float *x, float *y, int64_t M, void *stream) const
+    {
+        if (M > max_tokens) return MI_ERANGE;
+        return mi_w8a8_linear_f32(x, qw, sw, y, M, N, K, Block, workspace, workspace_bytes, stream);
+    }
+};
+
+// Decode attention over an int8 KV cache held by the caller.
+struct DecodeAttention {
+    int64_t B = 0, Hq = 0, Hkv = 0, D = 128, T = 0;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t)
+    {
+        B = b; Hq = hq; Hkv = hkv; T = t;
+        workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T);
+        if (workspace_bytes <= 0) return false;
+        workspace = arena.template alloc<uint8_t>(workspace_bytes);
+        return workspace != nullptr;
+    }
+    // appends nothing: quantizes `rows` fp32 rows [rows,128] into cache codes + scales
+    static int32_t quantize_rows(const float *kv, int8_t *codes, float *scales, int64_t rows, void *stream)
+    {
+        return mi_fwht_quant_f32_i8(kv, codes, scales, rows, 128, 128, stream);
+    }
+    int32_t forward(const float *q, const int8_t *kq, const float *ks, const int8_t *vq, const float *vs, float *o,
+                    bool out_rotated, void *stream) const
+    {
+        return mi_gqa_decode_attn(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T, out_rotated ? 1 : 0, workspace,
+                                  workspace_bytes, stream);
+    }
+};
+
+// Router + top-k dispatch + grouped expert SwiGLU FFN.
+struct MoeFfn {
+    int64_t T = 0, H = 0, I = 0, E = 0;
+    int32_t topk = 0;
+    const float *wr = nullptr;
+    const int8_t *wg = nullptr, *wu = nullptr, *wd = nullptr;
+    const float *sg = nullptr, *su = nullptr, *sd = nullptr;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t t, int64_t h, int64_t i, int64_t e, int32_t k)
+    {
+        T = t; H = h; I = i; E = e; topk = k;
+        workspace_bytes = mi_moe_layer_workspace_bytes(T, H, I, E, topk);
+        if (workspace_bytes <= 0) return false;
+        workspace = arena.template alloc<uint8_t>(workspace_bytes);
+        return workspace != nullptr;
+    }
+    int32_t forward(const float *x, float *y, void *stream) const
+    {
+        return mi_moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream);
+    }
+};
+
+}  // namespace mi355

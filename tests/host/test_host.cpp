@@ -1,0 +1,195 @@
+// Parity harness for the C++ host layer, one binary in the style of the
+// upstream test program (test_linux_threading.mojo:11-16, :555-570): each test
+// prints [PASS]/[FAIL]; unlike upstream, a failure also sets the exit status.
+// The CPU oracle (oracle/oracle.c) is linked here as the checker only.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../mojo-linuxperiments_amd/host/mi355_host.hpp"
+
+extern "C" {
+int orc_rotate_quant_rows(const float *, int64_t, int64_t, int, int8_t *, float *, float *);
+int orc_w8a8_linear(const float *, const int8_t *, const float *, float *, int64_t, int64_t, int64_t, int, int8_t *,
+                    float *, int32_t *);
+int orc_gqa_decode(const float *, const int8_t *, const float *, const int8_t *, const float *, float *, int64_t,
+                   int64_t, int64_t, int64_t, int64_t, int, int8_t *, float *, int32_t *);
+}
+
+using namespace mi355;
+
+static int g_failed = 0;
+static void report(const char *name, bool passed, const std::string &detail = "")
+{
+    std::printf("[%s] %s%s%s\n", passed ? "PASS" : "FAIL", name, detail.empty() ? "" : ": ", detail.c_str());
+    if (!passed) ++g_failed;
+}
+
+// splitmix64 -> uniform -> Box-Muller: host-only synthetic inputs
+struct Rng {
+    uint64_t s;
+    uint64_t next() { uint64_t z = (s += 0x9e3779b97f4a7c15ull); z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull; z = (z ^ (z >> 27)) * 0x94d049bb133111ebull; return z ^ (z >> 31); }
+    double uni() { return ((next() >> 11) + 0.5) / 9007199254740992.0; }
+    float normal() { return (float)(std::sqrt(-2.0 * std::log(uni())) * std::cos(6.283185307179586 * uni())); }
+};
+
+template <typename T>
+static std::vector<T> download(const T *dev, size_t n)
+{
+    std::vector<T> h(n);
+    mi_stream_synchronize(nullptr);
+    mi_memcpy_d2h(h.data(), dev, (int64_t)(n * sizeof(T)), nullptr);
+    mi_stream_synchronize(nullptr);
+    return h;
+}
+
+template <typename T, typename Arena>
+static T *upload(Arena &a, const std::vector<T> &h)
+{
+    T *d = a.template alloc<T>((int64_t)h.size());
+    if (!d) return nullptr;
+    mi_memcpy_h2d(d, h.data(), (int64_t)(h.size() * sizeof(T)), nullptr);
+    mi_stream_synchronize(nullptr);
+    return d;
+}
+
+static void test_arena(const Context &ctx)
+{
+    DeviceArena<256> arena(ctx, 1 << 20);
+    bool ok = (bool)arena && arena.used() == 0 && arena.remaining() == (1 << 20) && arena.verify_placement();
+    int *a = arena.alloc<int>(10);
+    int *b = arena.alloc<int>(10);
+    ok = ok && a && b && (reinterpret_cast<uintptr_t>(b) - reinterpret_cast<uintptr_t>(a)) == 256;
+    const int64_t w = arena.mark();
+    double *c = arena.alloc<double>(1000);
+    arena.reset_to(w + 999999);  // beyond used: ignored
+    ok = ok && arena.used() == w + 8000 + (256 - w % 256) % 256;
+    arena.reset_to(w);
+    ok = ok && arena.alloc<double>(1000) == c;
+    ok = ok && arena.alloc<char>(2 << 20) == nullptr;  // exhausted: null pointer
+    DeviceArena<256> moved(std::move(arena));
+    ok = ok && (bool)moved && !(bool)arena && moved.verify_placement();
+    moved.reset();
+    ok = ok && moved.used() == 0;
+    report("device_arena", ok);
+}
+
+static int32_t fill_op(void *stream, uint32_t *dst, uint32_t value, int64_t count)
+{
+    return mi_fill_u32(dst, value, count, stream);
+}
+
+static void test_stream_pool(const Context &ctx)
+{
+    DeviceArena<256> arena(ctx, 64 << 20);
+    StreamPool pool(ctx, 4);
+    bool ok = (bool)pool && pool.size() == 4;
+    uint32_t *out = arena.alloc<uint32_t>(32 * 1024);
+    for (int batch = 0; batch < 8 && ok; ++batch) {  // 32 launches in 8 batches of 4, output[i] == 2*i*i
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t k = batch * 4 + i;
+            ok = ok && pool.launch(fill_op, out + k * 1024, 2 * k * k, (int64_t)1024);
+        }
+        pool.wait_all();
+    }
+    std::vector<uint32_t> h = download(out, 32 * 1024);
+    for (uint32_t k = 0; k < 32; ++k) ok = ok && h[k * 1024] == 2 * k * k && h[k * 1024 + 1023] == 2 * k * k;
+    report("stream_pool_launch_wait_all", ok);
+
+    // pool full -> launch returns false; wait_any frees a slot; nothing in flight -> -1
+    uint32_t *big = arena.alloc<uint32_t>(8 << 20);
+    int launched = 0;
+    bool saw_full = false;
+    for (int i = 0; i < 64; ++i) {
+        if (pool.launch(fill_op, big, 7u, (int64_t)(8 << 20))) ++launched;
+        else { saw_full = true; break; }
+    }
+    int completed = 0;
+    while (pool.wait_any() >= 0) ++completed;
+    report("stream_pool_full_and_wait_any", saw_full && launched == 4 && completed == 4 && pool.wait_any() == -1,
+           "launched " + std::to_string(launched) + " completed " + std::to_string(completed));
+
+    Gate gate = Gate::create(ctx);
+    bool gok = gate.h && !gate.wait(pool.stream(0));  // never released
+    gok = gok && pool.launch([&](void *s) { int32_t rc = mi_fill_u32(big, 9u, 1 << 20, s); gate.release(s); return rc; });
+    gok = gok && pool.launch([&](void *s) { gate.wait(s); return mi_fill_u32(big, 11u, 1 << 20, s); });
+    pool.wait_all();
+    gok = gok && download(big, 16)[3] == 11u;
+    gate.reset();
+    gok = gok && !gate.wait_host();
+    gate.destroy();
+    report("gate_orders_streams", gok);
+}
+
+static void test_quant_linear(const Context &ctx)
+{
+    const int64_t M = 48, K = 1024, N = 256;
+    DeviceArena<256> arena(ctx, 64 << 20);
+    Rng rng{42};
+    std::vector<float> x(M * K), w(N * K);
+    for (auto &v : x) v = rng.normal();
+    for (int64_t m = 0; m < M; ++m) x[m * K + 17] *= 20.0f;  // an outlier channel
+    for (auto &v : w) v = 0.02f * rng.normal();
+    float *dx = upload(arena, x), *dw = upload(arena, w);
+    float *dy = arena.alloc<float>(M * N);
+    QuantLinear<128> lin;
+    bool ok = dx && dw && dy && lin.prepare(arena, dw, N, K, M, nullptr);
+    ok = ok && lin.forward(dx, dy, M, nullptr) == MI_OK;
+    ok = ok && lin.forward(dx, dy, M + 1, nullptr) == MI_ERANGE;
+    std::vector<int8_t> qw = download(lin.qw, N * K), qw_ref(N * K), qx_ref(M * K);
+    std::vector<float> sw = download(lin.sw, N), sw_ref(N), sx_ref(M), y = download(dy, M * N), y_ref(M * N);
+    std::vector<int32_t> acc_ref(M * N);
+    orc_rotate_quant_rows(w.data(), N, K, 128, qw_ref.data(), sw_ref.data(), nullptr);
+    orc_w8a8_linear(x.data(), qw_ref.data(), sw_ref.data(), y_ref.data(), M, N, K, 128, qx_ref.data(), sx_ref.data(),
+                    acc_ref.data());
+    ok = ok && qw == qw_ref && sw == sw_ref;
+    std::vector<int8_t> qx = download(static_cast<int8_t *>(lin.workspace), M * K);
+    ok = ok && qx == qx_ref;
+    double num = 0, den = 0;
+    for (int64_t i = 0; i < M * N; ++i) { num += (double)(y[i] - y_ref[i]) * (y[i] - y_ref[i]); den += (double)y_ref[i] * y_ref[i]; }
+    const double rel = std::sqrt(num / den);
+    report("quant_linear_vs_oracle", ok && rel <= 1e-3, "rel-L2 " + std::to_string(rel));
+}
+
+static void test_decode_attention(const Context &ctx)
+{
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 128, T = 200;
+    DeviceArena<256> arena(ctx, 64 << 20);
+    Rng rng{7};
+    std::vector<float> q(B * Hq * D), k(B * Hkv * T * D), v(B * Hkv * T * D);
+    for (auto &e : q) e = rng.normal();
+    for (auto &e : k) e = rng.normal();
+    for (auto &e : v) e = rng.normal();
+    float *dq = upload(arena, q), *dk = upload(arena, k), *dv = upload(arena, v);
+    int8_t *kq = arena.alloc<int8_t>(B * Hkv * T * D), *vq = arena.alloc<int8_t>(B * Hkv * T * D);
+    float *ks = arena.alloc<float>(B * Hkv * T), *vs = arena.alloc<float>(B * Hkv * T), *o = arena.alloc<float>(B * Hq * D);
+    DecodeAttention att;
+    bool ok = att.prepare(arena, B, Hq, Hkv, T);
+    ok = ok && DecodeAttention::quantize_rows(dk, kq, ks, B * Hkv * T, nullptr) == MI_OK;
+    ok = ok && DecodeAttention::quantize_rows(dv, vq, vs, B * Hkv * T, nullptr) == MI_OK;
+    ok = ok && att.forward(dq, kq, ks, vq, vs, o, false, nullptr) == MI_OK;
+    std::vector<int8_t> hkq = download(kq, B * Hkv * T * D), hvq = download(vq, B * Hkv * T * D);
+    std::vector<float> hks = download(ks, B * Hkv * T), hvs = download(vs, B * Hkv * T), ho = download(o, B * Hq * D);
+    std::vector<float> o_ref(B * Hq * D);
+    orc_gqa_decode(q.data(), hkq.data(), hks.data(), hvq.data(), hvs.data(), o_ref.data(), B, Hq, Hkv, D, T, 0, nullptr,
+                   nullptr, nullptr);
+    float err = 0;
+    for (size_t i = 0; i < ho.size(); ++i) err = std::fmax(err, std::fabs(ho[i] - o_ref[i]));
+    report("decode_attention_vs_oracle", ok && err <= 2e-3f, "max-abs " + std::to_string(err));
+}
+
+int main()
+{
+    Context ctx(0);
+    report("context", (bool)ctx, ctx ? "CUs " + std::to_string(ctx.compute_units()) : "no gfx950 device");
+    if (!ctx) return 1;
+    test_arena(ctx);
+    test_stream_pool(ctx);
+    test_quant_linear(ctx);
+    test_decode_attention(ctx);
+    std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");
+    return g_failed ? 1 : 0;
+}
