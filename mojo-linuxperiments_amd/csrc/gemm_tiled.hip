@@ -2,30 +2,54 @@
 //   acc[m,n] = sum_k qx[m,k] * qw[n,k],   y = ((float)acc * sx[m]) * sw[n]
 //
 // Tiling.  A workgroup of four waves (2 x 2) owns a (32*TM) x (32*TN) output
-// tile; each wave owns (16*TM) x (16*TN) of it as TM*TN MFMA accumulators
-// (256 registers at TM = TN = 8, which is why a SIMD holds one wave).  K is
-// walked in stages of 128 bytes, double buffered in LDS.
+// tile; each wave owns (16*TM) x (16*TN) of it as TM*TN MFMA accumulators held
+// in AccVGPRs (192 registers at 8 x 6, so a SIMD holds one wave).  K is walked
+// in stages of 128 bytes, double buffered in LDS.
 //
-// LDS layout = MFMA operand order.  A "fragment" is 16 rows x 64 K-bytes,
-// stored as 1024 contiguous bytes in which lane l's 16 bytes sit at offset
-// 16*l (row l%16, K-bytes 16*(l/16)..+15).  A fragment is filled by ONE
-// direct-to-LDS load per wave (global_load_lds_dwordx4: every lane supplies
-// its global address, the hardware writes lane l's 16 bytes at LDS base +
-// 16*l) and consumed by ONE ds_read_b128 per lane with no bank conflict, no
-// staging registers and no ds_write.  Both halves of a 128-byte line are
-// fetched in the same stage, so every L2 line is requested once per tile.
+// Global -> LDS.  Every transfer is a direct-to-LDS load
+// (global_load_lds_dwordx4): one wave instruction moves 8 rows x 128 bytes,
+// lane l = 8*rho + c fetching the 16-byte chunk kappa = c ^ sigma of row rho,
+// and the hardware writes lane l's bytes at LDS base + 16*l.  Eight lanes per
+// row means each quarter wave touches two whole 128-byte lines: measured
+// 13-28 TB/s aggregate against 7-8 TB/s for the 16-rows-x-64-bytes shape that
+// an MFMA fragment would suggest.  No staging registers, no ds_write.
+//
+// LDS -> MFMA.  A fragment (16 rows x 64 K-bytes; lane l wants row l%16, chunk
+// 4*kk + l/16) is read with one ds_read_b128 per lane from two of those 1 KB
+// blocks.  The XOR sigma(rho, block parity) = (rho & 6) | ((rho ^ parity) & 1)
+// spreads the 16 lanes that share a chunk index over 16 distinct 16-byte bank
+// groups, whichever of 8 or 16 lanes the LDS serves per cycle.
+//
+// Stage loop.  The MFMAs of a stage form 2*TN groups of TM instructions that
+// share one weight fragment.  Fragments are fetched two groups ahead with
+// explicit ds_read_b128 / s_waitcnt lgkmcnt(n) (inline asm: the compiler would
+// wait for lgkmcnt(0) and expose the LDS latency in every group).  The single
+// barrier of a stage sits before the last two groups: by then every wave has
+// issued and drained its reads of the current buffer and its share of the next
+// stage has landed (vmcnt 0), so after the barrier the next stage is visible,
+// the current buffer is free, the loads of stage +2 go out at once and the
+// first fragments of the next stage are fetched under the last two groups.
+//
+// MFMA accumulators are tied (destination == source, AccVGPR) through inline
+// asm; with the builtin the register allocator rotates all accumulators
+// through v_accvgpr moves in every stage.  The compiler cannot see inside the
+// asm, so the one software-managed hazard that remains (VALU read of a fresh
+// MFMA result) is covered by explicit wait states before the epilogue.
 //
 // Operand roles: the weight fragment is MFMA operand A and the activation
-// fragment operand B, so a lane ends up with four consecutive output channels
-// of one token (registers e = 0..3 -> n = 16*tile + 4*(l/16) + e, token
-// l%16) and the epilogue stores float4.
+// fragment operand B, so a lane holds four consecutive output channels of one
+// token.  The epilogue pairs neighbouring channel tiles and swaps halves
+// between lanes r and r ^ 8 (DPP row_ror:8) so that one store instruction
+// writes 8 rows x 128 contiguous bytes.
 //
 // Workgroup -> tile mapping is XCD-aware: hardware deals workgroup ids round
-// robin over the 8 XCDs, each with a private L2, so the tile grid is cut into
-// 8 rectangular parts (pm x pn) and XCD x only ever touches the rows and
-// columns of part x.
+// robin over the 8 XCDs (measured), each with a private L2, so the tile grid
+// is cut into 8 rectangular parts (pm x pn) and XCD x only ever touches the
+// rows and columns of part x.
 //
 // Bound: int8 MFMA (2*M*N*K ops).  Exact integer arithmetic.
+#include <utility>
+
 #include "common.h"
 
 namespace mi {
@@ -33,10 +57,60 @@ namespace mi {
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
+__device__ __forceinline__ void mfma_i8(v4i &acc, const v4i &a, const v4i &b)
+{
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm()
+{
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void ds_read128(v4i &dst, unsigned addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>)
+{
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
+}
+// how many second-half activation fragments are fetched during group g of the first half
+template <int TM, int TN>
+constexpr int xb1_count(int g)
+{
+    int c = 0;
+    for (int i = 0; i < TM; ++i)
+        if (i * TN / TM == g) ++c;
+    return c;
+}
+__device__ __forceinline__ int ror8(int v) { return __builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false); }
+
 struct GemmGrid {
     int tiles_m, tiles_n;
     int pm, pn;  // XCD partition; pm == 0 -> plain row-major tile order
 };
+
+template <bool DEQ>
+__device__ __forceinline__ void store4(float *y, int32_t *acc_out, int64_t idx, const v4i &v, float sxm, const float4 &s4)
+{
+    if constexpr (DEQ) {
+        float4 o;
+        o.x = ((float)v[0] * sxm) * s4.x;
+        o.y = ((float)v[1] * sxm) * s4.y;
+        o.z = ((float)v[2] * sxm) * s4.z;
+        o.w = ((float)v[3] * sxm) * s4.w;
+        *reinterpret_cast<float4 *>(y + idx) = o;
+    } else {
+        *reinterpret_cast<v4i *>(acc_out + idx) = v;
+    }
+}
 
 template <int TM, int TN, bool DEQ>
 __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
@@ -45,13 +119,13 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
                                                     int N, int K, GemmGrid gg)
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
-    constexpr int NFX = BM / 16 * 2;  // activation fragments per stage
-    constexpr int NFW = BN / 16 * 2;  // weight fragments per stage
-    constexpr int STAGE = (NFX + NFW) * 1024;
+    constexpr int NBX = BM / 8, NBW = BN / 8;  // 1 KB blocks (8 rows x 128 B) per stage
+    constexpr int STAGE = (NBX + NBW) * 1024;
+    constexpr int G = 2 * TN;                  // MFMA groups per stage
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     int tile_m, tile_n;
     {
@@ -59,7 +133,6 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
         if (gg.pm) {
             const int x = w & 7, li = w >> 3;
             const int sub_m = gg.tiles_m / gg.pm, sub_n = gg.tiles_n / gg.pn;
-            (void)sub_m;
             tile_m = (x / gg.pn) * sub_m + li / sub_n;
             tile_n = (x % gg.pn) * sub_n + li % sub_n;
         } else {
@@ -69,25 +142,29 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // this wave fills fragments f = wave, wave+4, ...: row tile f/2, K half f%2
-    constexpr int LX = NFX / 4, LW = NFW / 4;
+    // load side: this wave fills blocks b = wave, wave+4, ...
+    constexpr int LX = NBX / 4, LW = NBW / 4;
     const int8_t *xsrc[LX];
     const int8_t *wsrc[LW];
+    {
+        const int rho = lane >> 3, c = lane & 7;
 #pragma unroll
-    for (int i = 0; i < LX; ++i) {
-        const int f = wave + 4 * i;
-        int row = m0 + (f >> 1) * 16 + r;
-        if (row > M - 1) row = M - 1;
-        xsrc[i] = qx + (int64_t)row * K + (f & 1) * 64 + g * 16;
-    }
+        for (int i = 0; i < LX; ++i) {
+            const int b = wave + 4 * i;
+            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            int row = m0 + b * 8 + rho;
+            if (row > M - 1) row = M - 1;  // rows past the edge are computed from a valid row and never stored
+            xsrc[i] = qx + (int64_t)row * K + ((c ^ sigma) << 4);
+        }
 #pragma unroll
-    for (int i = 0; i < LW; ++i) {
-        const int f = wave + 4 * i;
-        int row = n0 + (f >> 1) * 16 + r;
-        if (row > N - 1) row = N - 1;
-        wsrc[i] = qw + (int64_t)row * K + (f & 1) * 64 + g * 16;
+        for (int i = 0; i < LW; ++i) {
+            const int b = wave + 4 * i;
+            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            int row = n0 + b * 8 + rho;
+            if (row > N - 1) row = N - 1;
+            wsrc[i] = qw + (int64_t)row * K + ((c ^ sigma) << 4);
+        }
     }
-
     auto issue = [&](int stage, int kt) {
         char *sb = smem + stage * STAGE;
         const int64_t koff = (int64_t)kt * 128;
@@ -96,65 +173,128 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
             __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + koff), (lptr_t)(sb + (wave + 4 * i) * 1024), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < LW; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + koff), (lptr_t)(sb + (NFX + wave + 4 * i) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + koff), (lptr_t)(sb + (NBX + wave + 4 * i) * 1024), 16, 0, 0);
     };
+
+    // read side
+    const int r = lane & 15, g_ = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    unsigned roff0, roff1;
+    {
+        const int rho = r & 7, bpar = r >> 3;
+        const int sigma = (rho & 6) | ((rho ^ bpar) & 1);
+        roff0 = bpar * 1024 + ((8 * rho + ((0 + g_) ^ sigma)) << 4);
+        roff1 = bpar * 1024 + ((8 * rho + ((4 + g_) ^ sigma)) << 4);
+    }
+    const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
+    const unsigned xo = lds_base + wm * TM * 2048, wo = lds_base + NBX * 1024 + wn * TN * 2048;
 
     v4i acc[TN][TM];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int i = 0; i < TM; ++i) acc[j][i] = (v4i){0, 0, 0, 0};
+    v4i xb0[TM], xb1[TM], wa[3];
 
-    const int wm = wave >> 1, wn = wave & 1;
     const int nk = K >> 7;
     issue(0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) issue(cur ^ 1, kt + 1);
-        const char *sb = smem + cur * STAGE;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            v4i xb[TM];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                xb[i] = *reinterpret_cast<const v4i *>(sb + (((wm * TM + i) * 2 + kk) * 1024) + lane * 16);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const v4i wa = *reinterpret_cast<const v4i *>(sb + ((NFX + (wn * TN + j) * 2 + kk) * 1024) + lane * 16);
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa, xb[i], acc[j][i], 0, 0, 0);
-            }
-        }
-        // the next stage has landed in LDS (this wave's share: vmcnt 0; the other
-        // waves' shares: barrier) and every wave is done reading this stage
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+    if (nk > 1) issue(1, 1);
+    {   // first fragments of stage 0
+        const unsigned ax0 = xo + roff0, aw0 = wo + roff0;
+        static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb0[decltype(I)::value], ax0); });
+        ds_read128<0>(wa[0], aw0);
+        ds_read128<2048>(wa[1], aw0);
     }
+    for (int kt = 0; kt < nk; ++kt) {
+        const unsigned cb = (kt & 1) * STAGE, nb = ((kt & 1) ^ 1) * STAGE;
+        const unsigned ax1 = xo + cb + roff1, aw0 = wo + cb + roff0, aw1 = wo + cb + roff1;
+        const unsigned nax0 = xo + nb + roff0, naw0 = wo + nb + roff0;
+        static_for<G>([&](auto GG) {
+            constexpr int g = decltype(GG)::value;
+            constexpr int kk = g / TN, j = g % TN;
+            if constexpr (g == G - 2) {
+                // all reads of the current buffer have been issued: drain them and this wave's
+                // share of the next stage, then the one barrier of the stage
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (kt + 2 < nk) issue(kt & 1, kt + 2);
+                static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb0[decltype(I)::value], nax0); });
+                ds_read128<0>(wa[G % 3], naw0);
+            } else if constexpr (g == G - 1) {
+                ds_read128<2048>(wa[(G + 1) % 3], naw0);
+            } else {
+                if constexpr (kk == 0) {
+                    static_for<TM>([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        if constexpr (i * TN / TM == j) ds_read128<i * 2048>(xb1[i], ax1);
+                    });
+                }
+                constexpr int g2 = g + 2;  // <= G - 1
+                ds_read128<(g2 % TN) * 2048>(wa[g2 % 3], (g2 / TN) ? aw1 : aw0);
+                // LDS returns in order: allow the reads issued after wa[g % 3] to stay in flight
+                constexpr int c_prev = (kk == 0 && g >= 1) ? xb1_count<TM, TN>(g - 1) : 0;
+                constexpr int c_cur = (kk == 0) ? xb1_count<TM, TN>(g) : 0;
+                wait_lgkm<2 + c_prev + c_cur>();
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) mfma_i8(acc[j][i], wa[g % 3], kk ? xb1[i] : xb0[i]);
+        });
+        // the next stage numbers its groups from 0 again
+        if constexpr (G % 3 != 0) {
+            wait_lgkm<0>();
+            const v4i t0 = wa[G % 3], t1 = wa[(G + 1) % 3];
+            wa[0] = t0;
+            wa[1] = t1;
+        }
+    }
+    // drain the trailing fragment reads; 2 x 16 wait states cover the longest MFMA-result -> VALU-read hazard
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
 
-    // epilogue: lane holds n = nb + 4*g + e (e = 0..3) for token mb + r
+    // epilogue: lane holds channels nb + 4*g_ .. +3 of token mrow + r for each (i, j)
+    const bool lo = r < 8;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int m = m0 + (wm * TM + i) * 16 + r;
-        if (m >= M) continue;
-        float sxm = 0.0f;
-        if constexpr (DEQ) sxm = sx[m];
+        const int mrow = m0 + (wm * TM + i) * 16;
+        const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7);
+        float sxA = 0.0f, sxB = 0.0f;
+        if constexpr (DEQ) {
+            sxA = sx[mA < M ? mA : M - 1];
+            sxB = sx[mB < M ? mB : M - 1];
+        }
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + (wn * TN + j) * 16 + 4 * g;
-            if (n >= N) continue;
-            if constexpr (DEQ) {
-                const float4 s4 = *reinterpret_cast<const float4 *>(sw + n);
-                float4 o;
-                o.x = ((float)acc[j][i][0] * sxm) * s4.x;
-                o.y = ((float)acc[j][i][1] * sxm) * s4.y;
-                o.z = ((float)acc[j][i][2] * sxm) * s4.z;
-                o.w = ((float)acc[j][i][3] * sxm) * s4.w;
-                *reinterpret_cast<float4 *>(y + (int64_t)m * N + n) = o;
-            } else {
-                *reinterpret_cast<v4i *>(acc_out + (int64_t)m * N + n) = acc[j][i];
+        for (int j = 0; j + 1 < TN; j += 2) {
+            const int nb0 = n0 + (wn * TN + j) * 16;
+            const v4i a0 = acc[j][i], a1 = acc[j + 1][i];
+            v4i t0, t1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                t0[e] = ror8(a0[e]);
+                t1[e] = ror8(a1[e]);
+            }
+            const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
+            const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
+            const int n = nb0 + (lo ? 0 : 16) + 4 * g_;
+            if (n < N) {
+                float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if constexpr (DEQ) s4 = *reinterpret_cast<const float4 *>(sw + n);
+                if (mA < M) store4<DEQ>(y, acc_out, (int64_t)mA * N + n, vA, sxA, s4);
+                if (mB < M) store4<DEQ>(y, acc_out, (int64_t)mB * N + n, vB, sxB, s4);
+            }
+        }
+        if constexpr (TN & 1) {
+            constexpr int j = TN - 1;
+            const int m = mrow + r;
+            const int n = n0 + (wn * TN + j) * 16 + 4 * g_;
+            if (m < M && n < N) {
+                float sxm = 0.0f;
+                float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if constexpr (DEQ) {
+                    sxm = sx[m];
+                    s4 = *reinterpret_cast<const float4 *>(sw + n);
+                }
+                store4<DEQ>(y, acc_out, (int64_t)m * N + n, acc[j][i], sxm, s4);
             }
         }
     }
@@ -169,7 +309,7 @@ static int32_t launch_shape(const int8_t *qx, const float *sx, const int8_t *qw,
                             float *y, int M, int N, int K, hipStream_t s)
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
-    constexpr int LDS = 2 * (BM / 16 * 2 + BN / 16 * 2) * 1024;
+    constexpr int LDS = 2 * (BM / 8 + BN / 8) * 1024;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_w8a8_tiled<TM, TN, DEQ>),
