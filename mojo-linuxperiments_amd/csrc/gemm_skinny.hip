@@ -1,117 +1,452 @@
 // W8A8 contraction for skinny activations (decode GEMV, M <= 64):
 //   acc[m,n] = sum_k qx[m,k] * qw[n,k],   y = ((float)acc * sx[m]) * sw[n]
-//
-// The weights [N,K] are read from HBM exactly once with 128-bit loads; the
-// activation codes (at most 64 x K bytes) stay in L2.  One workgroup owns 16
-// consecutive weight rows and its waves split K; a wave feeds
-// v_mfma_i32_16x16x64_i8 with a 16-row x 64-byte weight fragment as the A
-// operand (lane l: row l%16, bytes 16*(l/16)..+15 of the 64-byte K step) and
-// the matching fragment of up to 16 tokens as the B operand.  Both operands
-// use the same lane -> K mapping, and an integer dot product does not depend
-// on the order of its terms, so the int32 accumulators are exact.  The waves'
-// partial accumulators meet in LDS; the epilogue applies the two scales.
-//
+// The weights [N,K] are read from HBM exactly once; everything else is small.
 // Bound: HBM.  Algorithmic bytes per call = N*K (weights) + M*K (codes)
 // + 4*M*N (output) + 4*(M+N) (scales).
+//
+// Two kernels, chosen by M:
+//
+//  k_gemv_dot4 (M <= 4).  One workgroup per compute unit owns a contiguous span
+//  of weight rows; the activation codes (M*K bytes) sit in LDS.  A wave streams
+//  one weight row at a time with 128-bit loads, 1 KB contiguous per wave
+//  instruction (eight whole 128-byte lines), double buffered in registers, and
+//  each lane feeds its 16 bytes to v_dot4_i32_i8 against the matching 16 bytes
+//  of every token.  The 64 partial int32 sums of a row meet in a DPP / swizzle
+//  wave reduction.  Exact: integer sums are order independent.
+//
+//  k_skinny_ring (4 < M <= 64).  v_mfma_i32_16x16x64_i8 wants 16 rows x 64
+//  bytes per operand, but a load shaped like that touches 16 different lines
+//  per quarter wave and runs at a third of the bandwidth of a load that takes
+//  8 rows x 128 bytes.  So every wave owns a private ring of LDS stages, fills
+//  it with direct-to-LDS loads of the good shape (weights and activation codes
+//  alike, XOR-swizzled so that the fragment reads are conflict free) and reads
+//  MFMA fragments back out.  The ring is private to the wave: no barrier in
+//  the main loop, only vmcnt / lgkmcnt waits, and several stages stay in
+//  flight per wave.  Waves of a workgroup split K; their partial accumulators
+//  meet in LDS at the end.
 #include "common.h"
 
 namespace mi {
 
-template <int MT, bool DEQ>
-__global__ __launch_bounds__(1024) void k_w8a8_skinny(const int8_t *__restrict__ qx,
-                                                      const int8_t *__restrict__ qw,
-                                                      const float *__restrict__ sx,
-                                                      const float *__restrict__ sw,
-                                                      int32_t *__restrict__ acc_out, float *__restrict__ y,
-                                                      int M, int N, int K)
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// ------------------------------------------------------------------ M <= 4
+__device__ __forceinline__ int wave_sum(int v)
 {
-    extern __shared__ int s_part[];  // [nwave][MT][4][64]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwave = blockDim.x >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const int steps = K >> 6;
-    const int s0 = (int)((int64_t)steps * wave / nwave), s1 = (int)((int64_t)steps * (wave + 1) / nwave);
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, true);  // row_ror:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, true);  // row_ror:8
+    v += __builtin_amdgcn_ds_swizzle(v, 0x401F);                    // lane ^ 16
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
 
-    const int8_t *wp = qw + (int64_t)(n0 + r) * K + g * 16;
-    const int8_t *xp[MT];
+// Transposed butterfly: `p` holds V (a power of two <= 64) per-lane partial sums; after the call lane l holds
+// the wave-wide total of value  l >> (6 - log2 V)  (lanes that share those top bits hold the same total).
+// Each round hands half of the values to the partner lane, so V values cost V - 1 shuffles + log-many, not 6 V.
+template <int V, int OFF>
+__device__ __forceinline__ void fold_sum(int (&p)[V], int lane)
+{
+    if constexpr (V > 1) {
+        const bool hi = (lane & OFF) != 0;
+        int q[V / 2];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        int m = mt * 16 + r;
-        if (m > M - 1) m = M - 1;  // rows past M are computed from a valid row and never stored
-        xp[mt] = qx + (int64_t)m * K + g * 16;
+        for (int i = 0; i < V / 2; ++i) {
+            const int keep = hi ? p[i + V / 2] : p[i];
+            const int send = hi ? p[i] : p[i + V / 2];
+            q[i] = keep + __shfl_xor(send, OFF, 64);
+        }
+        fold_sum<V / 2, OFF / 2>(q, lane);
+#pragma unroll
+        for (int i = 0; i < V / 2; ++i) p[i] = q[i];
+    } else {
+#pragma unroll
+        for (int off = OFF; off >= 1; off >>= 1) p[0] += __shfl_xor(p[0], off, 64);
     }
-    v4i acc[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (v4i){0, 0, 0, 0};
+}
 
-    constexpr int U = 4;
-    int s = s0;
-    for (; s + U <= s1; s += U) {
-        v4i a[U];
+constexpr int pow2_ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
+
+// k_gemv_reg (M <= 4, K = 1024 * CW * QW up to a ragged last chunk): lane l always works on the same byte
+// offsets of a row (16*l + 1024*c for the wave's CW chunks), so its share of the activation codes lives in
+// registers for the whole kernel: no LDS, no barrier in the streaming part.  A wave issues all the loads of
+// its R rows at once (R*CW <= 16 x 1 KB in flight per wave), runs v_dot4_i32_i8 on them and reduces its
+// R*MB per-lane sums with one transposed butterfly.  QW waves that split a row add their totals in LDS.
+template <int MB, int CW, bool DEQ>
+__global__ __launch_bounds__(256) void k_gemv_reg(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                                  const float *__restrict__ sx, const float *__restrict__ sw,
+                                                  int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
+                                                  int N, int K, int QW)
+{
+    constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);   // rows per wave
+    constexpr int V = pow2_ceil(R * MB);
+    __shared__ int s_red[4][V];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = wave % QW;                  // which CW-chunk slice of the row
+    const int rows_per_wg = (4 / QW) * R;
+    const int row0 = blockIdx.x * rows_per_wg + (wave / QW) * R;
+    const int kbase = q * CW * 1024 + lane * 16;
+
+    v4i w[R][CW];
 #pragma unroll
-        for (int u = 0; u < U; ++u) a[u] = *reinterpret_cast<const v4i *>(wp + (int64_t)(s + u) * 64);
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int c = 0; c < CW; ++c) {
+            const int off = kbase + c * 1024;
+            w[r][c] = (row0 + r < N && off < K) ? *reinterpret_cast<const v4i *>(qw + (int64_t)(row0 + r) * K + off)
+                                                : (v4i){0, 0, 0, 0};
+        }
+    v4i xr[MB][CW];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < CW; ++c) {
+            const int off = kbase + c * 1024;
+            const int ms = m < M ? m : M - 1;
+            xr[m][c] = off < K ? *reinterpret_cast<const v4i *>(qx + (int64_t)ms * K + off) : (v4i){0, 0, 0, 0};
+        }
+    int p[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) p[i] = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            int a = 0;
+#pragma unroll
+            for (int c = 0; c < CW; ++c) {
+                a = __builtin_amdgcn_sdot4(w[r][c][0], xr[m][c][0], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][1], xr[m][c][1], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][2], xr[m][c][2], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][3], xr[m][c][3], a, false);
+            }
+            p[r * MB + m] = a;
+        }
+    fold_sum<V, 32>(p, lane);
+    // lane l holds value v = l >> SH; the first lane of each group of 64/V lanes speaks for it
+    constexpr int SH = 6 - __builtin_ctz(V);
+    const int v = lane >> SH;
+    const bool speaker = (lane & ((1 << SH) - 1)) == 0;
+    int total = p[0];
+    if (QW > 1) {
+        if (speaker) s_red[wave][v] = total;
+        __syncthreads();
+        if (q == 0 && speaker) {
+            for (int o = 1; o < QW; ++o) total += s_red[wave + o][v];
+        }
+    }
+    if (q == 0 && speaker && v < R * MB) {
+        const int r = v / MB, m = v % MB, n = row0 + r;
+        if (n < N && m < M) {
+            if constexpr (DEQ) y[(int64_t)m * N + n] = ((float)total * sx[m]) * sw[n];
+            else acc_out[(int64_t)m * N + n] = total;
+        }
+    }
+}
+
+template <int MB, bool DEQ>
+__global__ __launch_bounds__(512) void k_gemv_dot4(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                                   const float *__restrict__ sx, const float *__restrict__ sw,
+                                                   int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
+                                                   int N, int K)
+{
+    extern __shared__ __attribute__((aligned(16))) char s_x[];  // [MB][K] activation codes
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwave = blockDim.x >> 6;
+    const int n_lo = (int)((int64_t)N * blockIdx.x / gridDim.x), n_hi = (int)((int64_t)N * (blockIdx.x + 1) / gridDim.x);
+    const int nchunk = (K + 1023) >> 10;   // 1 KB chunks per row; K % 128 == 0 so a chunk is whole for lane*16 < K - c*1024
+    constexpr int U = 4;                   // loads in flight per buffer
+
+    auto load_chunks = [&](v4i (&buf)[U], int row, int c0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const v4i b = *reinterpret_cast<const v4i *>(xp[mt] + (int64_t)(s + u) * 64);
-                acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u], b, acc[mt], 0, 0, 0);
-            }
+            const int off = (c0 + u) * 1024 + lane * 16;
+            buf[u] = (row < n_hi && off < K) ? *reinterpret_cast<const v4i *>(qw + (int64_t)row * K + off) : (v4i){0, 0, 0, 0};
         }
-    }
-    for (; s < s1; ++s) {
-        const v4i a = *reinterpret_cast<const v4i *>(wp + (int64_t)s * 64);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const v4i b = *reinterpret_cast<const v4i *>(xp[mt] + (int64_t)s * 64);
-            acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[mt], 0, 0, 0);
-        }
-    }
+    };
+    // first weight loads go out before the activation codes are staged
+    v4i buf[2][U];
+    int row = n_lo + wave, c0 = 0;
+    load_chunks(buf[0], row, 0);
 
-    // accumulator layout: lane l, register e  <->  weight row 4*(l/16)+e, token l%16
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s_part[((wave * MT + mt) * 4 + e) * 64 + lane] = acc[mt][e];
+    for (int i = tid * 16; i < MB * K; i += blockDim.x * 16) {
+        const int m = i / K, k = i - m * K;
+        const int ms = m < M ? m : M - 1;   // rows past M repeat the last token and are never stored
+        *reinterpret_cast<v4i *>(s_x + i) = *reinterpret_cast<const v4i *>(qx + (int64_t)ms * K + k);
+    }
     __syncthreads();
 
-    for (int o = tid; o < 256 * MT; o += blockDim.x) {
-        const int nl = o & 15, m = o >> 4;
-        if (m >= M) continue;
-        const int mt = m >> 4, src_lane = (nl >> 2) * 16 + (m & 15), e = nl & 3;
-        int sum = 0;
-        for (int w = 0; w < nwave; ++w) sum += s_part[((w * MT + mt) * 4 + e) * 64 + src_lane];
+    int acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0;
+    int cur = 0;
+    while (row < n_hi) {
+        // next batch of this row, or the first batch of the wave's next row
+        int nrow = row, nc0 = c0 + U;
+        if (nc0 >= nchunk) { nrow = row + nwave; nc0 = 0; }
+        load_chunks(buf[cur ^ 1], nrow, nc0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int off = (c0 + u) * 1024 + lane * 16;
+            if (off < K) {
+                const v4i w = buf[cur][u];
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    const v4i xv = *reinterpret_cast<const v4i *>(s_x + m * K + off);
+                    int a = acc[m];
+                    a = __builtin_amdgcn_sdot4(w[0], xv[0], a, false);
+                    a = __builtin_amdgcn_sdot4(w[1], xv[1], a, false);
+                    a = __builtin_amdgcn_sdot4(w[2], xv[2], a, false);
+                    a = __builtin_amdgcn_sdot4(w[3], xv[3], a, false);
+                    acc[m] = a;
+                }
+            }
+        }
+        if (nrow != row) {
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const int sum = wave_sum(acc[m]);
+                if (lane == 0 && m < M) {
+                    if constexpr (DEQ) y[(int64_t)m * N + row] = ((float)sum * sx[m]) * sw[row];
+                    else acc_out[(int64_t)m * N + row] = sum;
+                }
+                acc[m] = 0;
+            }
+        }
+        row = nrow;
+        c0 = nc0;
+        cur ^= 1;
+    }
+}
+
+// --------------------------------------------------------------- 4 < M <= 64
+template <int N>
+__device__ __forceinline__ void wait_vm()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// NG groups of 16 weight rows per workgroup, MT groups of 16 tokens, ring of D stages per wave.
+// A stage = one 128-byte K step of (16*NG weight rows + 16*MT token rows) as 1 KB blocks of 8 rows.
+template <int NG, int MT, int D, bool DEQ>
+__global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                                     const float *__restrict__ sx, const float *__restrict__ sw,
+                                                     int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
+                                                     int N, int K)
+{
+    constexpr int BLK = 2 * (NG + MT);       // 1 KB blocks (= load instructions) per stage
+    constexpr int STAGE = BLK * 1024;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = blockDim.x >> 6;
+    char *ring = smem + wave * (D * STAGE);
+    const int n0 = blockIdx.x * 16 * NG;
+
+    // load side: lane l = 8*rho + c fetches chunk c ^ sigma of row rho of the block
+    const int8_t *src[BLK];
+    {
+        const int rho = lane >> 3, c = lane & 7;
+#pragma unroll
+        for (int b = 0; b < BLK; ++b) {
+            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            const int8_t *base;
+            if (b < 2 * NG) {
+                int rowi = n0 + b * 8 + rho;
+                if (rowi > N - 1) rowi = N - 1;
+                base = qw + (int64_t)rowi * K;
+            } else {
+                int tok = (b - 2 * NG) * 8 + rho;
+                if (tok > M - 1) tok = M - 1;   // tokens past M repeat the last one and are never stored
+                base = qx + (int64_t)tok * K;
+            }
+            src[b] = base + ((c ^ sigma) << 4);
+        }
+    }
+    const int steps = K >> 7;
+    const int s0 = (int)((int64_t)steps * wave / nwave), s1 = (int)((int64_t)steps * (wave + 1) / nwave);
+    auto issue = [&](int slot, int s) {
+        const int sc = s < s1 ? s : s1 - 1;   // past the slice: re-fetch the last step (keeps the vmcnt arithmetic uniform)
+        char *sb = ring + slot * STAGE;
+        const int64_t koff = (int64_t)sc * 128;
+#pragma unroll
+        for (int b = 0; b < BLK; ++b)
+            __builtin_amdgcn_global_load_lds((gptr_t)(src[b] + koff), (lptr_t)(sb + b * 1024), 16, 0, 0);
+    };
+
+    // read side: fragment (16-row group t, K half kk): lane (r = l%16, g = l/16) reads row r, chunk 4*kk + g
+    const int r = lane & 15, g_ = lane >> 4;
+    int roff[2];
+    {
+        const int rho = r & 7, bpar = r >> 3;
+        const int sigma = (rho & 6) | ((rho ^ bpar) & 1);
+        roff[0] = bpar * 1024 + ((8 * rho + ((0 + g_) ^ sigma)) << 4);
+        roff[1] = bpar * 1024 + ((8 * rho + ((4 + g_) ^ sigma)) << 4);
+    }
+    v4i acc[NG][MT];
+#pragma unroll
+    for (int a = 0; a < NG; ++a)
+#pragma unroll
+        for (int b = 0; b < MT; ++b) acc[a][b] = (v4i){0, 0, 0, 0};
+
+    if (s1 > s0) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) issue(d, s0 + d);
+        int slot = 0;
+        for (int s = s0; s < s1; ++s) {
+            wait_vm<(D - 1) * BLK>();   // the oldest stage in flight has landed
+            const char *sb = ring + slot * STAGE;
+            v4i wf[NG][2], xf[MT][2];
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                for (int a = 0; a < NG; ++a) wf[a][kk] = *reinterpret_cast<const v4i *>(sb + a * 2048 + roff[kk]);
+#pragma unroll
+                for (int b = 0; b < MT; ++b) xf[b][kk] = *reinterpret_cast<const v4i *>(sb + (NG + b) * 2048 + roff[kk]);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot may be refilled
+            issue(slot, s + D);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int a = 0; a < NG; ++a)
+#pragma unroll
+                    for (int b = 0; b < MT; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[a][kk], xf[b][kk], acc[a][b], 0, 0, 0);
+            slot = slot + 1 == D ? 0 : slot + 1;
+        }
+        wait_vm<0>();   // nothing of this wave may still be writing LDS when the ring is reused below
+    }
+    __syncthreads();
+
+    // partial accumulators of all waves -> LDS (the rings are idle now)
+    int *s_part = reinterpret_cast<int *>(smem);   // [nwave][NG][MT][4][64]
+#pragma unroll
+    for (int a = 0; a < NG; ++a)
+#pragma unroll
+        for (int b = 0; b < MT; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s_part[(((wave * NG + a) * MT + b) * 4 + e) * 64 + lane] = acc[a][b][e];
+    __syncthreads();
+    // accumulator layout: lane l, register e  <->  weight row 4*(l/16)+e, token l%16
+    for (int o = tid; o < 256 * NG * MT; o += blockDim.x) {
+        const int nl = o % (16 * NG), m = o / (16 * NG);
         const int n = n0 + nl;
+        if (m >= M || n >= N) continue;
+        const int a = nl >> 4, nn = nl & 15, b = m >> 4;
+        const int src_lane = (nn >> 2) * 16 + (m & 15), e = nn & 3;
+        int sum = 0;
+        for (int w = 0; w < nwave; ++w) sum += s_part[(((w * NG + a) * MT + b) * 4 + e) * 64 + src_lane];
         if constexpr (DEQ) y[(int64_t)m * N + n] = ((float)sum * sx[m]) * sw[n];
         else acc_out[(int64_t)m * N + n] = sum;
     }
 }
 
+template <int MB, bool DEQ>
+static int32_t launch_dot4(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
+                           float *y, int M, int N, int K, hipStream_t s)
+{
+    const size_t lds = (size_t)MB * K;
+    static bool attr_set = false;  // idempotent; a race only repeats the call
+    if (!attr_set) {
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_dot4<MB, DEQ>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+    }
+    const int cus = compute_units();
+    // one or two workgroups per compute unit, each with a contiguous span of at least 8 rows
+    int grid = lds <= 64 * 1024 ? 2 * cus : cus;
+    if (grid > (N + 7) / 8) grid = (N + 7) / 8;
+    hipLaunchKernelGGL((k_gemv_dot4<MB, DEQ>), dim3((unsigned)grid), dim3(512), lds, s, qx, qw, sx, sw, acc, y, M, N, K);
+    return launch_status();
+}
+
+template <int MB, int CW, bool DEQ>
+static int32_t launch_reg(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
+                          float *y, int M, int N, int K, int QW, hipStream_t s)
+{
+    constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);
+    const int rows_per_wg = (4 / QW) * R;
+    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL((k_gemv_reg<MB, CW, DEQ>), dim3(grid), dim3(256), 0, s, qx, qw, sx, sw, acc, y, M, N, K, QW);
+    return launch_status();
+}
+
+template <int MB, bool DEQ>
+static int32_t launch_reg_cw(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
+                             float *y, int M, int N, int K, int CW, int QW, hipStream_t s)
+{
+    switch (CW) {
+    case 1: return launch_reg<MB, 1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    case 2: return launch_reg<MB, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    case 3: return launch_reg<MB, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    case 4: return launch_reg<MB, 4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    case 5: return launch_reg<MB, 5, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    case 6: return launch_reg<MB, 6, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    default: return launch_reg<MB, 7, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, QW, s);
+    }
+}
+
+template <int NG, int MT, int D, bool DEQ>
+static int32_t launch_ring(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
+                           float *y, int M, int N, int K, int nwave, hipStream_t s)
+{
+    constexpr int STAGE = 2 * (NG + MT) * 1024;
+    size_t lds = (size_t)nwave * D * STAGE;
+    const size_t part = (size_t)nwave * NG * MT * 4 * 64 * sizeof(int);
+    if (part > lds) lds = part;
+    static bool attr_set = false;  // idempotent; a race only repeats the call
+    if (!attr_set) {
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_skinny_ring<NG, MT, D, DEQ>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+    }
+    const unsigned grid = (unsigned)((N + 16 * NG - 1) / (16 * NG));
+    hipLaunchKernelGGL((k_skinny_ring<NG, MT, D, DEQ>), dim3(grid), dim3((unsigned)(64 * nwave)), lds, s, qx, qw, sx,
+                       sw, acc, y, M, N, K);
+    return launch_status();
+}
+
 template <bool DEQ>
 int32_t launch_skinny(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
-                      float *y, int64_t M, int64_t N, int64_t K, hipStream_t s)
+                      float *y, int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
 {
-    const int64_t groups = N / 16;
+    const int M = (int)M64, N = (int)N64, K = (int)K64;
+    if (M <= 4) {
+        // K = 1024 * CW * QW (last chunk may be ragged) with CW <= 7 chunks per wave and QW in {1, 2, 4} waves per row
+        const int nchunk = (K + 1023) >> 10;
+        for (int QW = 1; QW <= 4; QW <<= 1) {
+            if (nchunk % QW || nchunk / QW > 7) continue;
+            const int CW = nchunk / QW;
+            if (M == 1) return launch_reg_cw<1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, CW, QW, s);
+            if (M == 2) return launch_reg_cw<2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, CW, QW, s);
+            return launch_reg_cw<4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, CW, QW, s);
+        }
+    }
+    if (M <= 4 && (int64_t)4 * K <= 152 * 1024) {
+        if (M == 1) return launch_dot4<1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
+        if (M == 2) return launch_dot4<2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
+        return launch_dot4<4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
+    }
     const int cus = compute_units();
-    // enough waves per compute unit to keep tens of KB of weight loads in flight
-    int nwave = groups <= 2 * (int64_t)cus ? 16 : 8;
-    const int64_t steps = K / 64;
+    const int steps = K >> 7;
+    const int MT = (M + 15) / 16;
+    // Two 16-row groups per workgroup halve the activation traffic when there are rows enough to fill the
+    // chip.  Four waves (a 64-72 KB ring set, so two workgroups share a compute unit and overlap their
+    // prologues and epilogues) when there are workgroups enough, else eight waves to keep bytes in flight.
+    const bool two = MT == 1 && N / 32 >= cus + cus / 2;
+    const int wgs = two ? (N + 31) / 32 : (N + 15) / 16;
+    int nwave = wgs >= cus + cus / 2 ? 4 : 8;
     while (nwave > 1 && nwave > steps) nwave >>= 1;
-    const int MT = (int)((M + 15) / 16);
-    if (MT > 2 && nwave > 8) nwave = 8;  // keeps the partial sums within 32 KB of LDS
-    const size_t lds = (size_t)nwave * MT * 4 * 64 * sizeof(int);
-    const dim3 grid((unsigned)groups), blk((unsigned)(64 * nwave));
-#define MI_SKINNY(MTT)                                                                                     \
-    hipLaunchKernelGGL((k_w8a8_skinny<MTT, DEQ>), grid, blk, lds, s, qx, qw, sx, sw, acc, y, (int)M, (int)N, (int)K)
     switch (MT) {
-    case 1: MI_SKINNY(1); break;
-    case 2: MI_SKINNY(2); break;
-    case 3: MI_SKINNY(3); break;
-    case 4: MI_SKINNY(4); break;
+    case 1:
+        return two ? launch_ring<2, 1, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s)
+                   : launch_ring<1, 1, 4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
+    case 2: return launch_ring<1, 2, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
+    case 3:
+    case 4: return launch_ring<1, 4, 1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
     default: return MI_ERANGE;
     }
-#undef MI_SKINNY
-    return launch_status();
 }
 
 template int32_t launch_skinny<true>(const int8_t *, const float *, const int8_t *, const float *, int32_t *,
