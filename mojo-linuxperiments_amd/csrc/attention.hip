@@ -10,15 +10,14 @@
 // tokens of one KV head once and serves the G = Hq/Hkv <= 4 query heads that
 // share it.  A second small kernel merges the splits.
 //
-// Pass 1 (scores).  A 16-token x 128-byte K tile is two MFMA A-fragments
-// (lane l: token l%16, bytes 16*(l/16)..+15 of each 64-byte half); the query
-// codes of the G heads are the B operand (heads beyond G are zero columns), so
-// v_mfma_i32_16x16x64_i8 leaves dot(token 4*(l/16)+e, head l%16) in register
-// e.  Scores (already in log2 units) go to LDS, the running max stays in
-// registers.
-// Pass 2 (P.V).  V is loaded 16 bytes per lane in token-major order (lane l:
-// token l/8 of an 8-token group, bytes 16*(l%8)..+15), i.e. 1 KB contiguous
-// per wave instruction.  v_mfma_f32_4x4x1_16B_f32 treats each aligned group of
+// Both passes load 16 bytes per lane in token-major order (lane l: token l/8
+// of an 8-token group, bytes 16*(l%8)..+15), i.e. 1 KB contiguous per wave
+// instruction, eight instructions in flight per wave.
+// Pass 1 (scores).  Each lane runs v_dot4_i32_i8 of its 16 key bytes against
+// the matching 16 query-code bytes of the G heads; the 8 lanes of a token add
+// their int32 partial sums (lane xor 1, 2, 4).  Scores (already in log2 units)
+// go to LDS, the running max stays in registers.
+// Pass 2 (P.V).  v_mfma_f32_4x4x1_16B_f32 treats each aligned group of
 // four lanes as one 4x4 outer product: the four lanes share a token, lane
 // l%4 = i supplies p(token, head i) * vs(token) as the A value and one V
 // element as the B value, so register i of the accumulator is head i.  Sixteen
@@ -36,7 +35,6 @@ namespace mi {
 namespace attn {
 
 constexpr int D = 128;
-constexpr int MAX_TS = 1024;  // tokens per split (LDS score buffer: 16 B per token)
 
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float v)
@@ -104,10 +102,36 @@ struct Params {
     float score_scale;    // log2(e) / sqrt(D)
 };
 
+// value of lane (lane ^ OFF) for OFF in {8, 16, 32}
+template <int OFF>
+__device__ __forceinline__ float slot_xor(float v)
+{
+    const int i = __float_as_int(v);
+    int r;
+    if constexpr (OFF == 8) r = __builtin_amdgcn_update_dpp(0, i, 0x128, 0xf, 0xf, true);   // row_ror:8
+    else if constexpr (OFF == 16) r = __builtin_amdgcn_ds_swizzle(i, 0x401F);
+    else r = __shfl_xor(i, 32, 64);
+    return __int_as_float(r);
+}
+// one round of the transposed butterfly over token slots: keep the half of the values whose index bit
+// matches this lane's OFF bit, hand the other half to lane ^ OFF
+template <int V, int OFF>
+__device__ __forceinline__ void fold_slots(float (&p)[64], int lane)
+{
+    const bool hi = (lane & OFF) != 0;
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) {
+        const float keep = hi ? p[i + V / 2] : p[i];
+        const float send = hi ? p[i] : p[i + V / 2];
+        p[i] = keep + slot_xor<OFF>(send);
+    }
+}
+
+constexpr int WAVE_GROUPS = 16;   // 8-token groups per wave: a workgroup covers at most 4 * 16 * 8 = 512 tokens
+
 template <bool DUMP>
 __global__ __launch_bounds__(256) void k_gqa_split(Params p)
 {
-    __shared__ float s_sc[MAX_TS * 4];
     __shared__ __attribute__((aligned(16))) int8_t s_q[4][4][D];
     __shared__ float s_sq[4][4];
     __shared__ float s_red[4][4][D];
@@ -120,8 +144,33 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     const int ntiles = (T + 15) >> 4;
     const int tile_lo = split * p.tiles_per_split;
     const int tile_hi = min(tile_lo + p.tiles_per_split, ntiles);
+    // lane layout of both passes: token slot = l/8 of an 8-token group, 16-byte chunk = l%8; head = l%4
+    const int hh = lane & 3, slot = lane >> 3, chunk = lane & 7;
+    const int t_lo = tile_lo << 4;
+    const int ngroups = max(0, min(tile_hi << 4, T) - t_lo + 7) >> 3;   // 8-token groups of this split
+    const int8_t *kbase = p.kq + (int64_t)bkv * T * D + 16 * chunk;
+    const int8_t *vbase = p.vq + (int64_t)bkv * T * D + 16 * chunk;
+    const float *ksb = p.ks + (int64_t)bkv * T;
+    const float *vsb = p.vs + (int64_t)bkv * T;
 
-    // ---- query heads of this group: rotate, quantize, lay out as the MFMA B operand
+    // ---- every K byte of this wave and the first half of its V bytes are requested before anything else:
+    // one load = 8 tokens x 128 B contiguous; wave w takes groups w, w+4, ...
+    v4i kv[WAVE_GROUPS], va[WAVE_GROUPS / 2];
+    float ksv[WAVE_GROUPS], vsa[WAVE_GROUPS / 2];
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS; ++u) {
+        const int tk = min(t_lo + (wave + 4 * u) * 8 + slot, T - 1);
+        kv[u] = *reinterpret_cast<const v4i *>(kbase + (int64_t)tk * D);
+        ksv[u] = ksb[tk];
+    }
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS / 2; ++u) {
+        const int tk = min(t_lo + (wave + 4 * u) * 8 + slot, T - 1);
+        va[u] = *reinterpret_cast<const v4i *>(vbase + (int64_t)tk * D);
+        vsa[u] = vsb[tk];
+    }
+
+    // ---- query heads of this group: rotate, quantize, park the codes in LDS
     {
         const int hr = lane >> 4, jj = lane & 15;
         const int head = kvh * G + min(hr, G - 1);
@@ -153,103 +202,97 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
         }
     }
     __syncthreads();
-
-    const int r = lane & 15, g = lane >> 4;
-    v4i qb0 = {0, 0, 0, 0}, qb1 = {0, 0, 0, 0};
-    float cq = 0.0f;  // per-head factor of the score, log2 units
-    if (r < G) {
-        qb0 = *reinterpret_cast<const v4i *>(&s_q[wave][r][16 * g]);
-        qb1 = *reinterpret_cast<const v4i *>(&s_q[wave][r][64 + 16 * g]);
-        cq = s_sq[wave][r] * p.score_scale;
-    }
-
-    const int8_t *kbase = p.kq + (int64_t)bkv * T * D;
-    const int8_t *vbase = p.vq + (int64_t)bkv * T * D;
-    const float *ksb = p.ks + (int64_t)bkv * T;
-    const float *vsb = p.vs + (int64_t)bkv * T;
-
-    // ---- pass 1: int32 scores of this wave's tiles -> LDS, running max in registers
-    float mx = -INFINITY;
-#pragma unroll 2
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += 4) {
-        const int t0 = tile << 4;
-        const int tk = min(t0 + r, T - 1);
-        const v4i k0 = *reinterpret_cast<const v4i *>(kbase + (int64_t)tk * D + 16 * g);
-        const v4i k1 = *reinterpret_cast<const v4i *>(kbase + (int64_t)tk * D + 64 + 16 * g);
-        v4i dot = {0, 0, 0, 0};
-        dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(k0, qb0, dot, 0, 0, 0);
-        dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(k1, qb1, dot, 0, 0, 0);
-        if (r < 4) {
-            const int tl = (tile - tile_lo) << 4;
+    v4i qd[4];       // query codes of the 4 heads for this lane's chunk
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int t = t0 + 4 * g + e;
-                float s = -INFINITY;
-                if (t < T) {
-                    s = (float)dot[e] * (ksb[t] * cq);
-                    if constexpr (DUMP) {
-                        if (r < G) p.dump_dots[((int64_t)b * p.Hq + kvh * G + r) * T + t] = dot[e];
-                    }
-                }
-                s_sc[(tl + 4 * g + e) * 4 + r] = s;
-                mx = fmaxf(mx, s);
-            }
+    for (int h = 0; h < 4; ++h)
+        qd[h] = h < G ? *reinterpret_cast<const v4i *>(&s_q[wave][h][16 * chunk]) : (v4i){0, 0, 0, 0};
+    const float cq = hh < G ? s_sq[wave][hh] * p.score_scale : 0.0f;   // per-head factor of the score, log2 units
+
+    // ---- pass 1: scores.  v_dot4_i32_i8 against the 4 heads, then the 8 lanes of a token add up
+    // (xor 1, 2, 4).  The score of (token l/8, head l%4) stays in a register, in log2 units.
+    float sc[WAVE_GROUPS];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS; ++u) {
+        const int gi = wave + 4 * u;
+        const int tt = t_lo + gi * 8 + slot;
+        int d[4];
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            int a = __builtin_amdgcn_sdot4(kv[u][0], qd[h][0], 0, false);
+            a = __builtin_amdgcn_sdot4(kv[u][1], qd[h][1], a, false);
+            a = __builtin_amdgcn_sdot4(kv[u][2], qd[h][2], a, false);
+            a = __builtin_amdgcn_sdot4(kv[u][3], qd[h][3], a, false);
+            a += __builtin_amdgcn_update_dpp(0, a, 0xB1, 0xf, 0xf, true);   // lane ^ 1
+            a += __builtin_amdgcn_update_dpp(0, a, 0x4E, 0xf, 0xf, true);   // lane ^ 2
+            a += __builtin_amdgcn_ds_swizzle(a, 0x101F);                    // lane ^ 4
+            d[h] = a;
         }
+        const int mine = hh == 0 ? d[0] : hh == 1 ? d[1] : hh == 2 ? d[2] : d[3];
+        const bool live = gi < ngroups && tt < T;
+        sc[u] = live ? (float)mine * (ksv[u] * cq) : -INFINITY;
+        if constexpr (DUMP) {
+            if (live && hh < G && chunk < 4) p.dump_dots[((int64_t)b * p.Hq + kvh * G + hh) * T + tt] = mine;
+        }
+        mx = fmaxf(mx, sc[u]);
     }
-    // lanes r = h (h < 4) of the four 16-lane rows hold partial maxima of head h
-    mx = fmaxf(mx, lane_xor<16>(mx));
-    mx = fmaxf(mx, lane_xor<32>(mx));
+    // the key registers are free: request the second half of V
+    v4i vb[WAVE_GROUPS / 2];
+    float vsb2[WAVE_GROUPS / 2];
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS / 2; ++u) {
+        const int tk = min(t_lo + (wave + 4 * (u + WAVE_GROUPS / 2)) * 8 + slot, T - 1);
+        vb[u] = *reinterpret_cast<const v4i *>(vbase + (int64_t)tk * D);
+        vsb2[u] = vsb[tk];
+    }
+    // lanes that share l%4 hold partial maxima of head l%4
+    mx = fmaxf(mx, slot_xor<8>(mx));
+    mx = fmaxf(mx, slot_xor<16>(mx));
+    mx = fmaxf(mx, slot_xor<32>(mx));
     if (lane < 4) s_m[wave][lane] = mx;
     __syncthreads();
 
     // ---- pass 2: P.V on the fp32 matrix pipe
-    const int hh = lane & 3, slot = lane >> 3, chunk = lane & 7;
     const float m_h = fmaxf(fmaxf(s_m[0][hh], s_m[1][hh]), fmaxf(s_m[2][hh], s_m[3][hh]));
     const bool counts = (lane & 4) == 0;  // each (token, head) is held by two lanes; one of them counts
     v4f acc[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = (v4f){0.f, 0.f, 0.f, 0.f};
     float lsum = 0.0f, csum = 0.0f;
-#pragma unroll 2
-    for (int tile = tile_lo + wave; tile < tile_hi; tile += 4) {
-        const int t0 = tile << 4;
-        const int tl = (tile - tile_lo) << 4;
+    auto pv = [&](const v4i &vv, float vscale, float score) {
+        const float pe = __builtin_amdgcn_exp2f(score - m_h);   // masked tokens: exp2(-inf) = 0
+        const float a = pe * vscale;
+        if (counts) { lsum += pe; csum += a; }
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int tt = t0 + 8 * u + slot;
-            const int tk = min(tt, T - 1);
-            const v4i vv = *reinterpret_cast<const v4i *>(vbase + (int64_t)tk * D + 16 * chunk);
-            const float pe = __builtin_amdgcn_exp2f(s_sc[(tl + 8 * u + slot) * 4 + hh] - m_h);
-            const float a = pe * vsb[tk];
-            if (counts) { lsum += pe; csum += a; }
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const uint32_t x = (uint32_t)vv[w] ^ 0x80808080u;
-                acc[4 * w + 0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x & 0xffu), acc[4 * w + 0], 0, 0, 0);
-                acc[4 * w + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 8) & 0xffu), acc[4 * w + 1], 0, 0, 0);
-                acc[4 * w + 2] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 16) & 0xffu), acc[4 * w + 2], 0, 0, 0);
-                acc[4 * w + 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x >> 24), acc[4 * w + 3], 0, 0, 0);
-            }
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t x = (uint32_t)vv[w] ^ 0x80808080u;
+            acc[4 * w + 0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x & 0xffu), acc[4 * w + 0], 0, 0, 0);
+            acc[4 * w + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 8) & 0xffu), acc[4 * w + 1], 0, 0, 0);
+            acc[4 * w + 2] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 16) & 0xffu), acc[4 * w + 2], 0, 0, 0);
+            acc[4 * w + 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x >> 24), acc[4 * w + 3], 0, 0, 0);
         }
-    }
-    // sum the 8 token slots (lanes that share l%8), and l / c over lanes that share l%4
+    };
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS / 2; ++u) pv(va[u], vsa[u], sc[u]);
+#pragma unroll
+    for (int u = 0; u < WAVE_GROUPS / 2; ++u) pv(vb[u], vsb2[u], sc[u + WAVE_GROUPS / 2]);
+
+    // sum the 8 token slots (lanes that share l%8): transposed butterfly over lane bits 5, 4, 3, after which
+    // lane l holds the 8 totals with flat index 8*(l/8) .. +7, flat = 4*e + head  (56 shuffles, not 192)
+    float flat[64];
 #pragma unroll
     for (int e = 0; e < 16; ++e)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float x = acc[e][i];
-            x += lane_xor<8>(x);
-            x += lane_xor<16>(x);
-            x += lane_xor<32>(x);
-            acc[e][i] = x;
-        }
-    lsum += lane_xor<8>(lsum); lsum += lane_xor<16>(lsum); lsum += lane_xor<32>(lsum);
-    csum += lane_xor<8>(csum); csum += lane_xor<16>(csum); csum += lane_xor<32>(csum);
-    if (lane < 8) {
+        for (int i = 0; i < 4; ++i) flat[4 * e + i] = acc[e][i];
+    fold_slots<64, 32>(flat, lane);
+    fold_slots<32, 16>(flat, lane);
+    fold_slots<16, 8>(flat, lane);
+    lsum += slot_xor<8>(lsum); lsum += slot_xor<16>(lsum); lsum += slot_xor<32>(lsum);
+    csum += slot_xor<8>(csum); csum += slot_xor<16>(csum); csum += slot_xor<32>(csum);
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) s_red[wave][i][16 * chunk + e] = acc[e][i];
+    for (int j = 0; j < 8; ++j) {
+        const int fl = 8 * slot + j;   // = 4*e + head
+        s_red[wave][fl & 3][16 * chunk + (fl >> 2)] = flat[j];
     }
     if (lane < 4) { s_l[wave][lane] = lsum; s_c[wave][lane] = csum; }
     __syncthreads();
@@ -309,10 +352,10 @@ static int pick_splits(int64_t B, int64_t Hkv, int64_t T)
 {
     const int ntiles = (int)((T + 15) / 16);
     const int cus = compute_units();
-    // enough workgroups for ~4 per compute unit, at least 16 tiles (256 tokens) each
-    int splits = 1;
-    while (splits < 64 && B * Hkv * splits < 4LL * cus && ntiles / (splits * 2) >= 16) splits *= 2;
-    while ((ntiles + splits - 1) / splits * 16 > MAX_TS) splits *= 2;
+    constexpr int MAX_TILES = 4 * WAVE_GROUPS / 2;   // 16-token tiles one workgroup can hold in registers
+    int splits = (ntiles + MAX_TILES - 1) / MAX_TILES;
+    // short caches / few heads: more, shorter splits until there are about two workgroups per compute unit
+    while (B * Hkv * splits < 2LL * cus && (ntiles + splits - 1) / splits > 8) splits *= 2;
     if (splits > ntiles) splits = ntiles;
     return splits;
 }
