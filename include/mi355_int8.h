@@ -199,8 +199,10 @@ MI_API int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const 
  * logits (ties to the lower expert), weights = softmax over the k picks.
  * x fp32 [T,H], wr fp32 [E,H] -> idx int32 [T,topk], w fp32 [T,topk].
  * H % 256 == 0, E % 16 == 0, E <= 256, topk <= 8. */
+MI_API int64_t mi_moe_route_workspace_bytes(int64_t T, int64_t E);   /* the fp32 logits [T,E] */
 MI_API int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, float *w,
-                            int64_t T, int64_t H, int64_t E, int32_t topk, void *stream);
+                            int64_t T, int64_t H, int64_t E, int32_t topk,
+                            void *workspace, int64_t workspace_bytes, void *stream);
 /* ---- a10: stable grouping of the T*topk (token,slot) pairs by expert.
  * idx int32 [T,topk] -> perm int32 [T*topk] (perm[pos] = pair = token*topk+slot),
  * seg_off int32 [E+1].  2 * E * ceil(T/32) + E + 1 <= 36864 (the bitmaps live in LDS). */
@@ -219,8 +221,8 @@ MI_API int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w,
 /* Byte offsets into the mi_moe_ffn workspace, for gates that inspect the
  * intermediates: which = 0 qx int8[T,H], 1 sx f32[T], 2 perm i32[T*topk],
  * 3 seg_off i32[E+1], 4 h f32[T*topk,I] (sorted order), 5 hq int8[T*topk,I],
- * 6 hs f32[T*topk], 7 out f32[T*topk,H] (pair order), 8 idx i32[T,topk] and
- * 9 w f32[T,topk] (filled by mi_moe_layer only).  Negative on error. */
+ * 6 hs f32[T*topk], 7 out f32[T*topk,H] (pair order), 8 idx i32[T,topk],
+ * 9 w f32[T,topk] and 10 router logits f32[T,E] (8-10 filled by mi_moe_layer only).  Negative on error. */
 MI_API int64_t mi_moe_ffn_workspace_offset(int32_t which, int64_t T, int64_t H, int64_t I,
                                            int64_t E, int32_t topk);
 /* Router + dispatch + FFN in one call (routing results land in the workspace). */

@@ -10,10 +10,10 @@
 //              y[token] = sum_slot w[token,slot] * out[pair]    (fixed order, no atomics)
 //
 // The expert GEMMs are weight-streaming bound (each expert sees ~32 rows): a
-// workgroup owns 16 gate + 16 up rows (or 64 down rows) of one expert, reads
-// them from HBM once with 128-bit loads as MFMA A-fragments, and walks the
-// expert's tokens 32 at a time with the gathered activation codes as B
-// fragments.  Waves split K; partial accumulators meet in LDS.
+// workgroup owns 16 gate + 16 up rows (or 32 down rows) of one expert, streams
+// them from HBM once through wave-private LDS rings, and walks the expert's
+// tokens 32 at a time with the gathered activation codes as MFMA B fragments.
+// Waves split K; partial accumulators meet in LDS.
 //
 // Bound: HBM on the int8 expert weights, E * 3 * H * I bytes per layer call.
 #include "common.h"
@@ -22,6 +22,7 @@ namespace mi {
 namespace moe {
 
 constexpr int MAX_TOPK = 8;
+static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 constexpr int64_t DISPATCH_MAX_WORDS = 36864;  // 144 KB of the 160 KB LDS
 
 __device__ __forceinline__ float shfl_xor_f(float v, int m) { return __shfl_xor(v, m, 64); }
@@ -49,16 +50,14 @@ __device__ __forceinline__ void fold(float (&p)[64], int lane)
     }
 }
 
-template <int MAX_THREADS>
-__global__ __launch_bounds__(MAX_THREADS) void k_moe_route(const float *__restrict__ x,
-                                                           const float *__restrict__ wr, int32_t *__restrict__ idx,
-                                                           float *__restrict__ w, int T, int H, int E, int topk)
+// grid = (T/16, E/16): a workgroup of 4 waves covers 16 tokens x 16 experts, so the router weights are read
+// T/16 times and the activations E/16 times in all (both from L2), and every compute unit gets work.
+__global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x, const float *__restrict__ wr,
+                                                    float *__restrict__ logits, int T, int H, int E)
 {
-    __shared__ float s_logit[4][256];
-    __shared__ float s_top[4][MAX_TOPK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int t0 = blockIdx.x * 4;
-    const int e0 = wave * 16;
+    const int t0 = blockIdx.x * 16 + wave * 4;
+    const int e0 = blockIdx.y * 16;
 
     float p[64];
 #pragma unroll
@@ -67,8 +66,7 @@ __global__ __launch_bounds__(MAX_THREADS) void k_moe_route(const float *__restri
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) xr[tt] = x + (int64_t)min(t0 + tt, T - 1) * H + 4 * lane;
     const float *wp = wr + (int64_t)e0 * H + 4 * lane;
-    const int nj = e0 < E ? H / 256 : 0;  // waves past the last expert group only help with top-k
-    for (int j = 0; j < nj; ++j) {
+    for (int j = 0; j < H / 256; ++j) {
         float4 xv[4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * j);
@@ -94,44 +92,55 @@ __global__ __launch_bounds__(MAX_THREADS) void k_moe_route(const float *__restri
     fold<2, 2>(p, lane);
     fold<1, 1>(p, lane);
     // lane l now holds pair l: token l/16, expert e0 + l%16
-    if (e0 < E) s_logit[lane >> 4][e0 + (lane & 15)] = p[0];
-    __syncthreads();
+    const int t = t0 + (lane >> 4);
+    if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
+}
 
-    // top-k by rank counting: rank(i) = #{j : l_j > l_i or (l_j == l_i and j < i)}
-    if (wave < 4 && t0 + wave < T) {
-        const int t = t0 + wave;
-        const float *lg = s_logit[wave];
-        float mine[4];
-        int rank[4];
+// one wave per token: k rounds of (wave-wide max, lowest index among the lanes that hold it); lane l holds
+// experts l, l+64, l+128, l+192.  Ties go to the lower expert index; picks come out by descending logit.
+__global__ __launch_bounds__(256) void k_moe_topk(const float *__restrict__ logits, int32_t *__restrict__ idx,
+                                                  float *__restrict__ w, int T, int E, int topk)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;   // whole wave
+    float mine[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = lane + 64 * u;
-            mine[u] = i < E ? lg[i] : -INFINITY;
-            rank[u] = 0;
-        }
-        for (int j = 0; j < E; ++j) {
-            const float v = lg[j];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int i = lane + 64 * u;
-                rank[u] += (v > mine[u] || (v == mine[u] && j < i)) ? 1 : 0;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = lane + 64 * u;
-            if (i < E && rank[u] < topk) {
-                idx[(int64_t)t * topk + rank[u]] = i;
-                s_top[wave][rank[u]] = mine[u];
-            }
-        }
+    for (int u = 0; u < 4; ++u) {
+        const int i = lane + 64 * u;
+        mine[u] = i < E ? logits[(int64_t)t * E + i] : -INFINITY;
     }
-    __syncthreads();
-    if (wave < 4 && t0 + wave < T && lane < topk) {
-        const float *tp = s_top[wave];
+    float top[MAX_TOPK];
+    int pick_lane = 0;       // lane s keeps pick s
+    for (int s = 0; s < topk; ++s) {
+        float v = fmaxf(fmaxf(mine[0], mine[1]), fmaxf(mine[2], mine[3]));
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+        // lowest expert index holding v: experts of slot u are 64u .. 64u+63, so the first non-empty ballot wins
+        int win = -1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned long long bal = __ballot(mine[u] == v);
+            if (win < 0 && bal) {
+                const int wl = __ffsll((long long)bal) - 1;
+                win = wl + 64 * u;
+                if (lane == wl) mine[u] = -INFINITY;   // taken
+            }
+        }
+        if (lane == s) pick_lane = win;
+#pragma unroll
+        for (int q = 0; q < MAX_TOPK; ++q)
+            if (q == s) top[q] = v;
+    }
+    if (lane < topk) {
+        idx[(int64_t)t * topk + lane] = pick_lane;
         float sum = 0.0f;
-        for (int s = 0; s < topk; ++s) sum = sum + expf(tp[s] - tp[0]);
-        w[(int64_t)(t0 + wave) * topk + lane] = expf(tp[lane] - tp[0]) / sum;
+        for (int s = 0; s < topk; ++s) sum = sum + expf(top[s] - top[0]);
+        float mine_top = top[0];
+#pragma unroll
+        for (int q = 1; q < MAX_TOPK; ++q)
+            if (q == lane) mine_top = top[q];
+        w[(int64_t)t * topk + lane] = expf(mine_top - top[0]) / sum;
     }
 }
 
@@ -181,140 +190,184 @@ __global__ __launch_bounds__(1024) void k_moe_dispatch(const int32_t *__restrict
 }
 
 // ------------------------------------------------------- a11 grouped GEMMs
-// Shared shape: a workgroup of 4 waves owns NG groups of 16 weight rows of one
-// expert; wave w owns K steps [steps*w/4, steps*(w+1)/4).  Tokens of the expert
-// are walked 32 at a time (two MFMA B-fragments).
-constexpr int MT = 2;  // 16-token fragments per pass
-
-// gate/up + SwiGLU.  Weight rows: 16 of wg and the same 16 of wu (NG = 2).
-__global__ __launch_bounds__(256) void k_moe_gate_up(const int8_t *__restrict__ qx, const float *__restrict__ sx,
-                                                     const int32_t *__restrict__ perm,
-                                                     const int32_t *__restrict__ seg_off,
-                                                     const int8_t *__restrict__ wg, const float *__restrict__ sg,
-                                                     const int8_t *__restrict__ wu, const float *__restrict__ su,
-                                                     float *__restrict__ h, int H, int I, int topk)
+// One kernel for both expert contractions.  A workgroup of 4 waves owns two groups of 16 weight rows of one
+// expert (gate/up: rows n0.. of wg and the same rows of wu, so SwiGLU happens in the epilogue; down: rows
+// n0.. and n0+16.. of wd) and walks the expert's tokens 32 at a time.  Waves split K.  Every wave streams
+// its K slice through a private ring of LDS stages filled by direct-to-LDS loads of 8 rows x 128 bytes
+// (weights and gathered activation rows alike; a load shaped like an MFMA fragment, 16 rows x 64 bytes, runs
+// at a third of the bandwidth), XOR-swizzled so that the v_mfma_i32_16x16x64_i8 fragment reads are conflict
+// free.  No barrier inside the stream; partial accumulators of the four waves meet in LDS.
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+template <int N>
+__device__ __forceinline__ void wait_vm()
 {
-    __shared__ int s_part[4][2][MT][4][64];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int e = blockIdx.y, n0 = blockIdx.x * 16;
-    const int seg0 = seg_off[e], count = seg_off[e + 1] - seg0;
-    if (count <= 0) return;
-    const int steps = H >> 6;
-    const int s0 = steps * wave / 4, s1 = steps * (wave + 1) / 4;
-    const int8_t *gp = wg + ((int64_t)e * I + n0 + r) * H + g * 16;
-    const int8_t *up = wu + ((int64_t)e * I + n0 + r) * H + g * 16;
-
-    for (int base = 0; base < count; base += 16 * MT) {
-        const int8_t *xp[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int row = min(base + mt * 16 + r, count - 1);
-            const int tok = perm[seg0 + row] / topk;
-            xp[mt] = qx + (int64_t)tok * H + g * 16;
-        }
-        v4i ag[MT], au[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) { ag[mt] = (v4i){0, 0, 0, 0}; au[mt] = (v4i){0, 0, 0, 0}; }
-#pragma unroll 4
-        for (int s = s0; s < s1; ++s) {
-            const v4i a_g = *reinterpret_cast<const v4i *>(gp + (int64_t)s * 64);
-            const v4i a_u = *reinterpret_cast<const v4i *>(up + (int64_t)s * 64);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const v4i b = *reinterpret_cast<const v4i *>(xp[mt] + (int64_t)s * 64);
-                ag[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_g, b, ag[mt], 0, 0, 0);
-                au[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_u, b, au[mt], 0, 0, 0);
-            }
-        }
-        __syncthreads();  // previous pass has finished reading s_part
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                s_part[wave][0][mt][c][lane] = ag[mt][c];
-                s_part[wave][1][mt][c][lane] = au[mt][c];
-            }
-        __syncthreads();
-        // 32 tokens x 16 channels: thread -> (token row, channel), channel fastest
-        for (int o = tid; o < 16 * MT * 16; o += 256) {
-            const int nl = o & 15, row = o >> 4;
-            if (base + row >= count) continue;
-            const int mt = row >> 4, src = (nl >> 2) * 16 + (row & 15), c = nl & 3;
-            int sg_i = 0, su_i = 0;
-#pragma unroll
-            for (int wv = 0; wv < 4; ++wv) { sg_i += s_part[wv][0][mt][c][src]; su_i += s_part[wv][1][mt][c][src]; }
-            const int pos = seg0 + base + row;
-            const int tok = perm[pos] / topk;
-            const float sxt = sx[tok];
-            const float gv = ((float)sg_i * sxt) * sg[(int64_t)e * I + n0 + nl];
-            const float uv = ((float)su_i * sxt) * su[(int64_t)e * I + n0 + nl];
-            h[(int64_t)pos * I + n0 + nl] = (gv / (1.0f + expf(-gv))) * uv;
-        }
-    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// down projection.  NG = 4 groups of 16 rows of wd per workgroup.
-constexpr int NGD = 4;
-__global__ __launch_bounds__(256) void k_moe_down(const int8_t *__restrict__ hq, const float *__restrict__ hs,
-                                                  const int32_t *__restrict__ perm,
-                                                  const int32_t *__restrict__ seg_off,
-                                                  const int8_t *__restrict__ wd, const float *__restrict__ sd,
-                                                  float *__restrict__ out, int H, int I)
+constexpr int MT = 2;             // 16-token fragments per pass
+constexpr int NGRP = 2;           // 16-row weight groups per workgroup
+constexpr int RING = 2;           // stages per wave
+constexpr int BLK = 2 * (NGRP + MT);
+constexpr int STAGE_BYTES = BLK * 1024;
+constexpr int RING_BYTES = 4 * RING * STAGE_BYTES;
+constexpr int EXPERT_LDS = RING_BYTES + 4 * NGRP * MT * 4 * 64 * 4;
+
+template <bool DOWN>
+__global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restrict__ act,
+                                                         const float *__restrict__ act_scale,
+                                                         const int32_t *__restrict__ perm,
+                                                         const int32_t *__restrict__ seg_off,
+                                                         const int8_t *__restrict__ w0, const float *__restrict__ sc0,
+                                                         const int8_t *__restrict__ w1, const float *__restrict__ sc1,
+                                                         float *__restrict__ out, int Kdim, int Nrows, int Hout,
+                                                         int topk, int nch)
 {
-    __shared__ int s_part[4][NGD][MT][4][64];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int e = blockIdx.y, n0 = blockIdx.x * 16 * NGD;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int e = blockIdx.y;
     const int seg0 = seg_off[e], count = seg_off[e + 1] - seg0;
     if (count <= 0) return;
-    const int steps = I >> 6;
-    const int s0 = steps * wave / 4, s1 = steps * (wave + 1) / 4;
-    const int8_t *wp[NGD];
+    // gate/up: the 4 waves split K (2048 bytes = 16 steps).  down: K is short (768 bytes = 6 steps), so each
+    // wave takes its own 32 rows over the whole of K and nothing has to be added across waves
+    // A workgroup walks `nch` consecutive row chunks (16 rows for gate/up, 128 for down) as ONE stream: the
+    // loads of the next chunk are already in flight while the partial sums of this one are added and stored,
+    // and the segment / permutation lookups are paid once per workgroup.
+    constexpr int CHUNK_ROWS = DOWN ? 128 : 16;
+    const int n0 = DOWN ? blockIdx.x * nch * 128 + wave * 32 : blockIdx.x * nch * 16;
+    char *ring = smem + wave * (RING * STAGE_BYTES);
+    int *s_part = reinterpret_cast<int *>(smem + RING_BYTES);   // [4 waves][NGRP][MT][4][64]
+
+    // load side: lane l = 8*rho + c fetches chunk c ^ sigma(rho, block parity) of row rho of the block
+    const int rho = lane >> 3, c8 = lane & 7;
+    const int8_t *wsrc[2 * NGRP];
 #pragma unroll
-    for (int ng = 0; ng < NGD; ++ng) wp[ng] = wd + ((int64_t)e * H + min(n0 + ng * 16 + r, H - 1)) * I + g * 16;
+    for (int b = 0; b < 2 * NGRP; ++b) {
+        const int sigma = (rho & 6) | ((rho ^ b) & 1);
+        const int grp = b >> 1;
+        int rowi = n0 + (DOWN ? grp * 16 : 0) + (b & 1) * 8 + rho;
+        if (rowi > Nrows - 1) rowi = Nrows - 1;
+        const int8_t *base = (DOWN || grp == 0) ? w0 : w1;
+        wsrc[b] = base + ((int64_t)e * Nrows + rowi) * Kdim + ((c8 ^ sigma) << 4);
+    }
+    const int steps = Kdim >> 7;
+    const int s0 = DOWN ? 0 : steps * wave / 4, s1 = DOWN ? steps : steps * (wave + 1) / 4;
+
+    // read side: fragment (16-row group, K half kk): lane (r = l%16, g = l/16) reads row r, chunk 4*kk + g
+    const int r = lane & 15, g_ = lane >> 4;
+    int roff[2];
+    {
+        const int rr = r & 7, bpar = r >> 3;
+        const int sigma = (rr & 6) | ((rr ^ bpar) & 1);
+        roff[0] = bpar * 1024 + ((8 * rr + ((0 + g_) ^ sigma)) << 4);
+        roff[1] = bpar * 1024 + ((8 * rr + ((4 + g_) ^ sigma)) << 4);
+    }
 
     for (int base = 0; base < count; base += 16 * MT) {
-        const int8_t *xp[MT];
+        // gathered activation rows of this pass (rows past the segment repeat its last row and are never stored)
+        const int8_t *xsrc[2 * MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xp[mt] = hq + (int64_t)(seg0 + min(base + mt * 16 + r, count - 1)) * I + g * 16;
-        v4i acc[NGD][MT];
-#pragma unroll
-        for (int ng = 0; ng < NGD; ++ng)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[ng][mt] = (v4i){0, 0, 0, 0};
-#pragma unroll 3
-        for (int s = s0; s < s1; ++s) {
-            v4i b[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) b[mt] = *reinterpret_cast<const v4i *>(xp[mt] + (int64_t)s * 64);
-#pragma unroll
-            for (int ng = 0; ng < NGD; ++ng) {
-                const v4i a = *reinterpret_cast<const v4i *>(wp[ng] + (int64_t)s * 64);
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[ng][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[mt], acc[ng][mt], 0, 0, 0);
-            }
+        for (int b = 0; b < 2 * MT; ++b) {
+            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            const int pos = seg0 + min(base + b * 8 + rho, count - 1);
+            const int64_t arow = DOWN ? (int64_t)pos : (int64_t)(perm[pos] / topk);
+            xsrc[b] = act + arow * Kdim + ((c8 ^ sigma) << 4);
         }
+        const int nsw = s1 - s0;            // K steps of this wave per chunk
+        const int total_f = nch * nsw;      // flattened (chunk, step) stages of this wave
+        auto issue = [&](int slot, int f) {
+            const int fc = f < total_f ? f : total_f - 1;   // past the end: re-fetch the last stage (uniform vmcnt arithmetic)
+            const int ch = fc / nsw, st = s0 + (fc - ch * nsw);
+            char *sb = ring + slot * STAGE_BYTES;
+            const int64_t koff = (int64_t)st * 128;
+            const int64_t woff = (int64_t)ch * CHUNK_ROWS * Kdim + koff;
+#pragma unroll
+            for (int b = 0; b < 2 * NGRP; ++b)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[b] + woff), (lptr_t)(sb + b * 1024), 16, 0, 0);
+#pragma unroll
+            for (int b = 0; b < 2 * MT; ++b)
+                __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[b] + koff), (lptr_t)(sb + (2 * NGRP + b) * 1024), 16, 0, 0);
+        };
+        if (nsw > 0) {
+#pragma unroll
+            for (int d = 0; d < RING; ++d) issue(d, d);
+        }
+        int slot = 0, f = 0;
+        for (int ch = 0; ch < nch; ++ch) {
+        const int nc0 = n0 + ch * CHUNK_ROWS;
+        v4i acc[NGRP][MT];
+#pragma unroll
+        for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+            for (int b = 0; b < MT; ++b) acc[a][b] = (v4i){0, 0, 0, 0};
+        for (int i = 0; i < nsw; ++i, ++f) {
+            wait_vm<(RING - 1) * BLK>();   // the oldest stage in flight has landed
+            const char *sb = ring + slot * STAGE_BYTES;
+            v4i wf[NGRP][2], xf[MT][2];
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                for (int a = 0; a < NGRP; ++a) wf[a][kk] = *reinterpret_cast<const v4i *>(sb + a * 2048 + roff[kk]);
+#pragma unroll
+                for (int b = 0; b < MT; ++b) xf[b][kk] = *reinterpret_cast<const v4i *>(sb + (NGRP + b) * 2048 + roff[kk]);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot may be refilled
+            issue(slot, f + RING);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+                    for (int b = 0; b < MT; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[a][kk], xf[b][kk], acc[a][b], 0, 0, 0);
+            slot = slot + 1 == RING ? 0 : slot + 1;
+        }
+        __syncthreads();   // the previous chunk's epilogue has finished reading s_part
+#pragma unroll
+        for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+            for (int b = 0; b < MT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) s_part[(((wave * NGRP + a) * MT + b) * 4 + q) * 64 + lane] = acc[a][b][q];
         __syncthreads();
-#pragma unroll
-        for (int ng = 0; ng < NGD; ++ng)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int c = 0; c < 4; ++c) s_part[wave][ng][mt][c][lane] = acc[ng][mt][c];
-        __syncthreads();
-        for (int o = tid; o < 16 * MT * 16 * NGD; o += 256) {
-            const int nl = o & (16 * NGD - 1), row = o / (16 * NGD);
-            if (base + row >= count || n0 + nl >= H) continue;
-            const int ng = nl >> 4, nn = nl & 15;
-            const int mt = row >> 4, src = (nn >> 2) * 16 + (row & 15), c = nn & 3;
+        // accumulator layout: lane l, register q  <->  weight row 4*(l/16)+q, token l%16
+        auto total = [&](int a, int row, int nn) {
+            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
             int sum = 0;
 #pragma unroll
-            for (int wv = 0; wv < 4; ++wv) sum += s_part[wv][ng][mt][c][src];
-            const int pos = seg0 + base + row;
-            const int pair = perm[pos];
-            out[(int64_t)pair * H + n0 + nl] = ((float)sum * hs[pos]) * sd[(int64_t)e * H + n0 + nl];
+            for (int wv = 0; wv < 4; ++wv) sum += s_part[(((wv * NGRP + a) * MT + b) * 4 + q) * 64 + src];
+            return sum;
+        };
+        auto own = [&](int wv, int a, int row, int nn) {   // down: one wave's accumulator is already the total
+            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
+            return s_part[(((wv * NGRP + a) * MT + b) * 4 + q) * 64 + src];
+        };
+        if constexpr (!DOWN) {
+            // 32 tokens x 16 channels, channel fastest; h = silu(g) * u in sorted-pair order
+            for (int o = tid; o < 16 * MT * 16; o += 256) {
+                const int nl = o & 15, row = o >> 4;
+                if (base + row >= count || nc0 + nl >= Nrows) continue;
+                const int pos = seg0 + base + row;
+                const float sxt = act_scale[perm[pos] / topk];
+                const float gv = ((float)total(0, row, nl) * sxt) * sc0[(int64_t)e * Nrows + nc0 + nl];
+                const float uv = ((float)total(1, row, nl) * sxt) * sc1[(int64_t)e * Nrows + nc0 + nl];
+                out[(int64_t)pos * Nrows + nc0 + nl] = (gv / (1.0f + expf(-gv))) * uv;
+            }
+        } else {
+            // 32 tokens x 128 channels (32 per wave); out[pair] in pair order, channel fastest
+            const int nbase = (blockIdx.x * nch + ch) * 128;
+            for (int o = tid; o < 16 * MT * 128; o += 256) {
+                const int nl = o & 127, row = o >> 7;
+                if (base + row >= count || nbase + nl >= Nrows) continue;
+                const int pos = seg0 + base + row;
+                const int sum = own(nl >> 5, (nl >> 4) & 1, row, nl & 15);
+                out[(int64_t)perm[pos] * Hout + nbase + nl] =
+                    ((float)sum * act_scale[pos]) * sc0[(int64_t)e * Nrows + nbase + nl];
+            }
         }
+        }   // chunks
+        wait_vm<0>();   // trailing re-fetches must not write LDS after the workgroup has gone
     }
 }
 
@@ -334,20 +387,18 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ o
     *reinterpret_cast<float4 *>(y + i) = a;
 }
 
-static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
-
 struct Layout {
-    int64_t off[10];
+    int64_t off[11];
     int64_t total;
 };
 
 static Layout layout(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk)
 {
     const int64_t P = T * topk;
-    const int64_t sz[10] = {T * H, T * 4, P * 4, (E + 1) * 4, P * I * 4, P * I, P * 4, P * H * 4, P * 4, P * 4};
+    const int64_t sz[11] = {T * H, T * 4, P * 4, (E + 1) * 4, P * I * 4, P * I, P * 4, P * H * 4, P * 4, P * 4, T * E * 4};
     Layout L;
     int64_t o = 0;
-    for (int i = 0; i < 10; ++i) { L.off[i] = o; o += align_up(sz[i], 256); }
+    for (int i = 0; i < 11; ++i) { L.off[i] = o; o += align_up(sz[i], 256); }
     L.total = o;
     return L;
 }
@@ -366,22 +417,29 @@ static int32_t check_shapes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t 
 
 using namespace mi;
 
+extern "C" int64_t mi_moe_route_workspace_bytes(int64_t T, int64_t E)
+{
+    if (T < 0 || E <= 0) return MI_EINVAL;
+    return moe::align_up(T * E * 4, 256);
+}
+
 extern "C" int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, float *w, int64_t T, int64_t H,
-                                int64_t E, int32_t topk, void *stream)
+                                int64_t E, int32_t topk, void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!x || !wr || !idx || !w || T < 0 || H <= 0 || E <= 0 || topk <= 0) return MI_EINVAL;
     if (H % 256 || E % 16 || topk > moe::MAX_TOPK || topk > E) return MI_EINVAL;
     if (E > 256 || T > (1LL << 24)) return MI_ERANGE;
     if (!aligned16(x) || !aligned16(wr) || !aligned4(idx) || !aligned4(w)) return MI_EINVAL;
+    if (!workspace || !aligned16(workspace)) return MI_EINVAL;
+    if (workspace_bytes < mi_moe_route_workspace_bytes(T, E)) return MI_ENOSPC;
     if (T == 0) return MI_OK;
-    const int waves = (int)(E / 16) < 4 ? 4 : (int)(E / 16);  // the top-k phase uses waves 0..3
-    const dim3 grid((unsigned)((T + 3) / 4)), blk((unsigned)(64 * waves));
-    if (waves <= 8)   // up to 128 experts: 512 threads, so a lane may keep 256 registers
-        hipLaunchKernelGGL(moe::k_moe_route<512>, grid, blk, 0, as_stream(stream), x, wr, idx, w, (int)T, (int)H,
-                           (int)E, (int)topk);
-    else
-        hipLaunchKernelGGL(moe::k_moe_route<1024>, grid, blk, 0, as_stream(stream), x, wr, idx, w, (int)T, (int)H,
-                           (int)E, (int)topk);
+    float *logits = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(moe::k_moe_logits, dim3((unsigned)((T + 15) / 16), (unsigned)(E / 16)), dim3(256), 0,
+                       as_stream(stream), x, wr, logits, (int)T, (int)H, (int)E);
+    int32_t rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe::k_moe_topk, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, as_stream(stream), logits, idx, w,
+                       (int)T, (int)E, (int)topk);
     return launch_status();
 }
 
@@ -420,7 +478,7 @@ extern "C" int64_t mi_moe_ffn_workspace_offset(int32_t which, int64_t T, int64_t
 {
     int32_t rc = moe::check_shapes(T, H, I, E, topk);
     if (rc) return rc;
-    if (which < 0 || which > 9) return MI_EINVAL;
+    if (which < 0 || which > 10) return MI_EINVAL;
     return moe::layout(T, H, I, E, topk).off[which];
 }
 
@@ -452,14 +510,27 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     if (rc) return rc;
     rc = mi_fwht_quant_f32_i8(x, qx, sx, T, H, 128, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_gate_up, dim3((unsigned)(I / 16), (unsigned)E), dim3(256), 0, s, qx, sx, perm, seg,
-                       wg, sg, wu, su, h, (int)H, (int)I, (int)topk);
+    static bool attr_set = false;  // idempotent; a race only repeats the calls
+    if (!attr_set) {
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_gemm<false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, moe::EXPERT_LDS));
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_gemm<true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, moe::EXPERT_LDS));
+        attr_set = true;
+    }
+    // Row chunks per workgroup.  Walking several chunks as one stream measured no faster than one chunk per
+    // workgroup (the activation rows are re-fetched per chunk either way), so one it is.
+    const int nch_gu = 1, nch_dn = 1;
+    hipLaunchKernelGGL(moe::k_moe_expert_gemm<false>, dim3((unsigned)(I / 16 / nch_gu), (unsigned)E), dim3(256),
+                       moe::EXPERT_LDS, s, qx, sx, perm, seg, wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk,
+                       nch_gu);
     rc = launch_status();
     if (rc) return rc;
     rc = mi_fwht_quant_f32_i8(h, hq, hs, P, I, 256, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_down, dim3((unsigned)((H + 16 * moe::NGD - 1) / (16 * moe::NGD)), (unsigned)E),
-                       dim3(256), 0, s, hq, hs, perm, seg, wd, sd, out, (int)H, (int)I);
+    hipLaunchKernelGGL(moe::k_moe_expert_gemm<true>, dim3((unsigned)((H + 128 * nch_dn - 1) / (128 * nch_dn)), (unsigned)E),
+                       dim3(256), moe::EXPERT_LDS, s, hq, hs, perm, seg, wd, sd, (const int8_t *)nullptr,
+                       (const float *)nullptr, out, (int)I, (int)H, (int)H, (int)topk, nch_dn);
     rc = launch_status();
     if (rc) return rc;
     hipLaunchKernelGGL(moe::k_moe_combine, dim3((unsigned)((T * H / 4 + 255) / 256)), dim3(256), 0, s, out, w, y,
@@ -480,7 +551,7 @@ extern "C" int32_t mi_moe_layer(const float *x, const float *wr, const int8_t *w
     char *ws = static_cast<char *>(workspace);
     int32_t *idx = reinterpret_cast<int32_t *>(ws + L.off[8]);
     float *w = reinterpret_cast<float *>(ws + L.off[9]);
-    rc = mi_moe_route(x, wr, idx, w, T, H, E, topk, stream);
+    rc = mi_moe_route(x, wr, idx, w, T, H, E, topk, ws + L.off[10], mi_moe_route_workspace_bytes(T, E), stream);
     if (rc) return rc;
     return mi_moe_ffn(x, idx, w, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream);
 }

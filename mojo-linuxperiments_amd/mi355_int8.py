@@ -88,7 +88,8 @@ SIGNATURES = {
     "mi_gqa_decode_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
     "mi_gqa_decode_attn": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
-    "mi_moe_route": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "mi_moe_route_workspace_bytes": (i64, [i64, i64]),
+    "mi_moe_route": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
     "mi_moe_dispatch": (i32, [vp, vp, vp, i64, i64, i32, vp]),
     "mi_moe_ffn_workspace_bytes": (i64, [i64, i64, i64, i64, i32]),
     "mi_moe_ffn": (i32, [vp] * 10 + [i64, i64, i64, i64, i32, vp, i64, vp]),
@@ -336,10 +337,10 @@ def gqa_scores(q, kq, ks, vq, vs, qq, sq, dots, ws, stream=None):
                                        B, Hq, Hkv, D, T, ws.ptr, ws.nbytes, stream), "mi_gqa_decode_scores_i32")
 
 
-def moe_route(x, wr, idx, w, topk, stream=None):
+def moe_route(x, wr, idx, w, topk, ws, stream=None):
     T, H = x.shape
     E = wr.shape[0]
-    check(lib.mi_moe_route(x.ptr, wr.ptr, idx.ptr, w.ptr, T, H, E, topk, stream), "mi_moe_route")
+    check(lib.mi_moe_route(x.ptr, wr.ptr, idx.ptr, w.ptr, T, H, E, topk, ws.ptr, ws.nbytes, stream), "mi_moe_route")
 
 
 def moe_dispatch(idx, perm, seg, E, stream=None):

@@ -21,7 +21,8 @@ def gpu_route(mi, dev, x, wr, topk):
     mark = dev.mark()
     T = x.shape[0]
     didx, dw = dev.empty((T, topk), np.int32), dev.empty((T, topk), np.float32)
-    mi.moe_route(dev.upload(x), dev.upload(wr), didx, dw, topk)
+    ws = dev.empty(mi.lib.mi_moe_route_workspace_bytes(T, wr.shape[0]), np.uint8)
+    mi.moe_route(dev.upload(x), dev.upload(wr), didx, dw, topk, ws)
     idx, w = dev.download(didx), dev.download(dw)
     dev.reset_to(mark)
     return idx, w
@@ -185,10 +186,12 @@ def test_argument_errors(mi, dev):
     lib = mi.lib
     mark = dev.mark()
     b = dev.empty(1 << 16, np.uint8)
-    assert lib.mi_moe_route(b.ptr, b.ptr, b.ptr, b.ptr, 4, 100, 16, 2, None) == mi.EINVAL    # H % 256
-    assert lib.mi_moe_route(b.ptr, b.ptr, b.ptr, b.ptr, 4, 256, 24, 2, None) == mi.EINVAL    # E % 16
-    assert lib.mi_moe_route(b.ptr, b.ptr, b.ptr, b.ptr, 4, 256, 16, 9, None) == mi.EINVAL    # topk > 8
-    assert lib.mi_moe_route(b.ptr, b.ptr, b.ptr, b.ptr, 4, 256, 512, 2, None) == mi.ERANGE   # E > 256
+    rargs = (b.ptr, b.ptr, b.ptr, b.ptr)
+    assert lib.mi_moe_route(*rargs, 4, 100, 16, 2, b.ptr, b.nbytes, None) == mi.EINVAL    # H % 256
+    assert lib.mi_moe_route(*rargs, 4, 256, 24, 2, b.ptr, b.nbytes, None) == mi.EINVAL    # E % 16
+    assert lib.mi_moe_route(*rargs, 4, 256, 16, 9, b.ptr, b.nbytes, None) == mi.EINVAL    # topk > 8
+    assert lib.mi_moe_route(*rargs, 4, 256, 512, 2, b.ptr, b.nbytes, None) == mi.ERANGE   # E > 256
+    assert lib.mi_moe_route(*rargs, 4, 256, 16, 2, b.ptr, 16, None) == mi.ENOSPC          # logits do not fit
     assert lib.mi_moe_dispatch(b.ptr, b.ptr, b.ptr, 1 << 20, 128, 8, None) == mi.ERANGE      # bitmap too large
     assert lib.mi_moe_ffn_workspace_bytes(8, 200, 256, 16, 2) == mi.EINVAL                   # H % 128
     assert lib.mi_moe_ffn_workspace_bytes(8, 256, 300, 16, 2) == mi.EINVAL                   # I % 256
