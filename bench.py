@@ -75,12 +75,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-sub", action="store_true", help="only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
+                         "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
 
     import mi355_int8 as mi     # fails loudly when the HIP library is not built
     import workload as wl
+
+    if args.pmc_probe:
+        return pmc_probe(mi, wl)
 
     dev = mi.Device(arena_bytes=12 << 30)
     pool = mi.StreamPool(dev, 1)
@@ -191,6 +197,38 @@ def main():
     dev.close()
 
 
+def pmc_probe(mi, wl):
+    """Three launches each of: the rotation-only kernel on fp32 [2048,14336] (reads and writes exactly
+    117,440,512 B: the calibration for the FETCH_SIZE / WRITE_SIZE counters), the tiled GEMM on the four cfg3
+    shapes, the decode GEMV (M=1, 4096->14336), decode attention (cfg2) and the MoE layer (cfg4)."""
+    lib = mi.lib
+    dev = mi.Device(arena_bytes=8 << 30)
+    M = wl.PREFILL_M
+    g = np.random.default_rng(0)
+    a = dev.upload(g.standard_normal((M, 14336), dtype=np.float32))
+    b = dev.empty((M, 14336), np.float32)
+    for _ in range(3):
+        mi.fwht(a, b, 128)
+    dev.sync()
+    y = dev.empty((M, 14336), np.float32)
+    for name, K, N in wl.PROJECTIONS:
+        if name == "up":
+            continue
+        qx = dev.upload(g.integers(-127, 128, (M, K)).astype(np.int8))
+        qw = dev.upload(g.integers(-127, 128, (N, K)).astype(np.int8))
+        sx, sw = dev.upload(np.ones(M, np.float32)), dev.upload(np.ones(N, np.float32))
+        for _ in range(3):
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, y.ptr, M, N, K, None))
+        if name == "gate":
+            for _ in range(3):
+                mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, y.ptr, 1, N, K, None))
+        dev.sync()
+    timer = Timer(mi, None)
+    print(json.dumps({"probe": "done", "attention": decode_attention(mi, wl, dev, None, timer, reps=1, graph=False),
+                      "moe": moe_layer(mi, wl, dev, None, timer, reps=1, graph=False)}), flush=True)
+    dev.close()
+
+
 def graph_time(mi, dev, s, timer, calls, reps):
     """Per-call ms of a list of closures recorded once into a graph and replayed
     (decode kernels are a few microseconds: eager launches from Python would
@@ -243,7 +281,7 @@ def decode_gemv(mi, wl, dev, pool, s, timer, shapes, next_w):
     return {"cfg1_decode_gemv": res}
 
 
-def decode_attention(mi, wl, dev, s, timer):
+def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
     """cfg2: B=16, 32/8 heads, D=128, T=4096; three KV sets (402 MB) in rotation."""
     lib = mi.lib
     c = wl.ATTN
@@ -262,7 +300,7 @@ def decode_attention(mi, wl, dev, s, timer):
     do = dev.empty((B, Hq, D), np.float32)
     ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T), np.uint8)
     calls = [(lambda k=k: mi.gqa_decode(dq, k[0], k[1], k[2], k[3], do, False, ws, stream=s)) for k in sets]
-    ms = graph_time(mi, dev, s, timer, calls, 20)
+    ms = graph_time(mi, dev, s, timer, calls, reps) if graph else eager_time(dev, s, timer, calls)
     nbytes = wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
     dev.reset_to(mark)
     return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
@@ -270,7 +308,14 @@ def decode_attention(mi, wl, dev, s, timer):
                                       "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes}}
 
 
-def moe_layer(mi, wl, dev, s, timer):
+def eager_time(dev, s, timer, calls):
+    for c in calls:
+        c()
+    dev.sync(s)
+    return timer.run(lambda: [c() for c in calls], 1) / len(calls)
+
+
+def moe_layer(mi, wl, dev, s, timer, reps=20, graph=True):
     """cfg4: 512 tokens, hidden 2048, 128 experts top-8, inner 768 (604 MB of expert weights)."""
     lib = mi.lib
     c = wl.MOE
@@ -290,7 +335,7 @@ def moe_layer(mi, wl, dev, s, timer):
     y = dev.empty((T, H), np.float32)
     ws = dev.empty(lib.mi_moe_layer_workspace_bytes(T, H, I, E, topk), np.uint8)
     call = lambda: mi.moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=s)
-    ms = graph_time(mi, dev, s, timer, [call], 20)
+    ms = graph_time(mi, dev, s, timer, [call], reps) if graph else eager_time(dev, s, timer, [call])
     wbytes = wl.moe_weight_bytes(E, H, I)
     ops = wl.moe_ops(T, topk, H, I)
     dev.reset_to(mark)

@@ -71,6 +71,14 @@ __device__ __forceinline__ void ds_read128(v4i &dst, unsigned addr)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
+// direct-to-LDS load of 16 bytes per lane: global address = sbase + voff, LDS address = ldsaddr + 16 * lane
+__device__ __forceinline__ void dma16(const int8_t *sbase, unsigned voff, unsigned ldsaddr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(ldsaddr)
+                 : "memory", "m0");
+}
 template <typename F, int... Is>
 __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>)
 {
@@ -112,6 +120,15 @@ __device__ __forceinline__ void store4(float *y, int32_t *acc_out, int64_t idx, 
     }
 }
 
+// LDS budget: two activation buffers and, where 160 KB allow it, three weight buffers (a small tile keeps
+// two so that two workgroups share a compute unit)
+template <int TM, int TN>
+struct TiledCfg {
+    static constexpr int NBX = 4 * TM, NBW = 4 * TN;
+    static constexpr int NWB = (TM * TN <= 16) ? 2 : ((2 * NBX + 3 * NBW <= 160) ? 3 : 2);
+    static constexpr int LDS = (2 * NBX + NWB * NBW) * 1024;
+};
+
 template <int TM, int TN, bool DEQ>
 __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
                                                     const float *__restrict__ sx, const float *__restrict__ sw,
@@ -120,8 +137,10 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
     constexpr int NBX = BM / 8, NBW = BN / 8;  // 1 KB blocks (8 rows x 128 B) per stage
-    constexpr int STAGE = (NBX + NBW) * 1024;
     constexpr int G = 2 * TN;                  // MFMA groups per stage
+    constexpr int NWB = TiledCfg<TM, TN>::NWB;
+    constexpr int XSTAGE = NBX * 1024, WSTAGE = NBW * 1024, XAREA = 2 * XSTAGE;
+    constexpr int R = (G % 3 == 0) ? 3 : ((G % 4 == 0) ? 4 : 3);  // weight fragment registers in rotation
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -142,39 +161,52 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // load side: this wave fills blocks b = wave, wave+4, ...
+    // load side: this wave fills blocks b = wave, wave+4, ... of each stage.  Addresses are a uniform
+    // 64-bit base (SGPR pair, advanced per stage) plus a 32-bit per-lane offset: the scalar-base form
+    // occupies the wave's issue slot for fewer cycles than a 64-bit VGPR address, and with one wave
+    // per SIMD every cycle a load holds the issue slot is a cycle the MFMA pipe is not fed.
     constexpr int LX = NBX / 4, LW = NBW / 4;
-    const int8_t *xsrc[LX];
-    const int8_t *wsrc[LW];
+    unsigned vx[LX], vw[LW];
     {
         const int rho = lane >> 3, c = lane & 7;
 #pragma unroll
         for (int i = 0; i < LX; ++i) {
             const int b = wave + 4 * i;
             const int sigma = (rho & 6) | ((rho ^ b) & 1);
-            int row = m0 + b * 8 + rho;
-            if (row > M - 1) row = M - 1;  // rows past the edge are computed from a valid row and never stored
-            xsrc[i] = qx + (int64_t)row * K + ((c ^ sigma) << 4);
+            int row = b * 8 + rho;
+            if (row > M - 1 - m0) row = M - 1 - m0;  // rows past the edge are computed from a valid row and never stored
+            vx[i] = (unsigned)row * (unsigned)K + (unsigned)((c ^ sigma) << 4);
         }
 #pragma unroll
         for (int i = 0; i < LW; ++i) {
             const int b = wave + 4 * i;
             const int sigma = (rho & 6) | ((rho ^ b) & 1);
-            int row = n0 + b * 8 + rho;
-            if (row > N - 1) row = N - 1;
-            wsrc[i] = qw + (int64_t)row * K + ((c ^ sigma) << 4);
+            int row = b * 8 + rho;
+            if (row > N - 1 - n0) row = N - 1 - n0;
+            vw[i] = (unsigned)row * (unsigned)K + (unsigned)((c ^ sigma) << 4);
         }
     }
-    auto issue = [&](int stage, int kt) {
-        char *sb = smem + stage * STAGE;
-        const int64_t koff = (int64_t)kt * 128;
-#pragma unroll
-        for (int i = 0; i < LX; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + koff), (lptr_t)(sb + (wave + 4 * i) * 1024), 16, 0, 0);
-#pragma unroll
-        for (int i = 0; i < LW; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + koff), (lptr_t)(sb + (NBX + wave + 4 * i) * 1024), 16, 0, 0);
+    const int8_t *const xtile = qx + (int64_t)m0 * K;
+    const int8_t *const wtile = qw + (int64_t)n0 * K;
+    const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
+    const unsigned lds_x = lds_base + wave * 1024, lds_w = lds_base + XAREA + wave * 1024;
+    // the activation loads of a stage are scheduled over SPX groups, the weight loads over SPW groups
+    constexpr int SPX = (TN - 2 < LX) ? TN - 2 : LX, SPW = LW;
+    auto issue_x = [&](auto P, unsigned buf, int kt) {
+        const int8_t *src = xtile + (int64_t)kt * 128;
+        static_for<LX>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if constexpr (decltype(P)::value < 0 || i * SPX / LX == decltype(P)::value) dma16(src, vx[i], lds_x + buf + i * 4096);
+        });
     };
+    auto issue_w = [&](auto P, unsigned buf, int kt) {
+        const int8_t *src = wtile + (int64_t)kt * 128;
+        static_for<LW>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if constexpr (decltype(P)::value < 0 || i * SPW / LW == decltype(P)::value) dma16(src, vw[i], lds_w + buf + i * 4096);
+        });
+    };
+    constexpr std::integral_constant<int, -1> ALL{};
 
     // read side
     const int r = lane & 15, g_ = lane >> 4;
@@ -186,21 +218,35 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
         roff0 = bpar * 1024 + ((8 * rho + ((0 + g_) ^ sigma)) << 4);
         roff1 = bpar * 1024 + ((8 * rho + ((4 + g_) ^ sigma)) << 4);
     }
-    const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
-    const unsigned xo = lds_base + wm * TM * 2048, wo = lds_base + NBX * 1024 + wn * TN * 2048;
+    const unsigned xo = lds_base + wm * TM * 2048, wo = lds_base + XAREA + wn * TN * 2048;
 
     v4i acc[TN][TM];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int i = 0; i < TM; ++i) acc[j][i] = (v4i){0, 0, 0, 0};
-    v4i xb0[TM], xb1[TM], wa[3];
+    v4i xb0[TM], xb1[TM], wa[R];
 
     const int nk = K >> 7;
-    issue(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // stage s lives in activation buffer s % 2 and weight buffer s % NWB; the offsets rotate with the stage
+    unsigned xcur = 0, xnxt = XSTAGE;
+    unsigned wcur = 0, wnxt = WSTAGE, wnn = (NWB == 3) ? 2 * WSTAGE : 0;
+    issue_x(ALL, 0u, 0);
+    issue_w(ALL, 0u, 0);
+    if (nk > 1) {
+        issue_w(ALL, wnxt, 1);
+        issue_x(ALL, xnxt, 1);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LX + LW) : "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __syncthreads();
-    if (nk > 1) issue(1, 1);
+    if constexpr (NWB == 3) {
+        if (nk > 2) {
+            issue_w(std::integral_constant<int, 0>{}, wnn, 2);
+            if constexpr (SPW > 1) issue_w(std::integral_constant<int, 1>{}, wnn, 2);
+        }
+    }
     {   // first fragments of stage 0
         const unsigned ax0 = xo + roff0, aw0 = wo + roff0;
         static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb0[decltype(I)::value], ax0); });
@@ -208,22 +254,37 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
         ds_read128<2048>(wa[1], aw0);
     }
     for (int kt = 0; kt < nk; ++kt) {
-        const unsigned cb = (kt & 1) * STAGE, nb = ((kt & 1) ^ 1) * STAGE;
-        const unsigned ax1 = xo + cb + roff1, aw0 = wo + cb + roff0, aw1 = wo + cb + roff1;
-        const unsigned nax0 = xo + nb + roff0, naw0 = wo + nb + roff0;
+        const unsigned ax1 = xo + xcur + roff1, aw0 = wo + wcur + roff0, aw1 = wo + wcur + roff1;
+        const unsigned nax0 = xo + xnxt + roff0, naw0 = wo + wnxt + roff0;
+        const bool more = kt + 2 < nk;
         static_for<G>([&](auto GG) {
             constexpr int g = decltype(GG)::value;
             constexpr int kk = g / TN, j = g % TN;
+            // weight loads continue from the two slots used under the previous stage's last two groups
+            if constexpr (g + 2 < SPW) {
+                if constexpr (NWB == 3) {
+                    if (more) issue_w(std::integral_constant<int, g + 2>{}, wnn, kt + 2);
+                } else {
+                    if (kt > 0 && kt + 1 < nk) issue_w(std::integral_constant<int, g + 2>{}, wnxt, kt + 1);
+                }
+            }
+            if constexpr (g > TN && g - TN < SPX && g < G - 2) {
+                if (more) issue_x(std::integral_constant<int, g - TN>{}, xcur, kt + 2);
+            }
             if constexpr (g == G - 2) {
-                // all reads of the current buffer have been issued: drain them and this wave's
-                // share of the next stage, then the one barrier of the stage
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                // all reads of the current buffers have been issued: drain them and this wave's share of
+                // the next stage (loads return in order, so the loads of later stages may stay in flight)
+                if (more) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LX + (NWB == 3 ? LW : 0)) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 __syncthreads();
-                if (kt + 2 < nk) issue(kt & 1, kt + 2);
+                if (kt + NWB < nk) issue_w(std::integral_constant<int, 0>{}, wcur, kt + NWB);
                 static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb0[decltype(I)::value], nax0); });
-                ds_read128<0>(wa[G % 3], naw0);
+                ds_read128<0>(wa[G % R], naw0);
             } else if constexpr (g == G - 1) {
-                ds_read128<2048>(wa[(G + 1) % 3], naw0);
+                if constexpr (SPW > 1) {
+                    if (kt + NWB < nk) issue_w(std::integral_constant<int, 1>{}, wcur, kt + NWB);
+                }
+                ds_read128<2048>(wa[(G + 1) % R], naw0);
             } else {
                 if constexpr (kk == 0) {
                     static_for<TM>([&](auto I) {
@@ -232,72 +293,95 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
                     });
                 }
                 constexpr int g2 = g + 2;  // <= G - 1
-                ds_read128<(g2 % TN) * 2048>(wa[g2 % 3], (g2 / TN) ? aw1 : aw0);
-                // LDS returns in order: allow the reads issued after wa[g % 3] to stay in flight
+                ds_read128<(g2 % TN) * 2048>(wa[g2 % R], (g2 / TN) ? aw1 : aw0);
+                // LDS returns in order: allow the reads issued after wa[g % R] to stay in flight
                 constexpr int c_prev = (kk == 0 && g >= 1) ? xb1_count<TM, TN>(g - 1) : 0;
                 constexpr int c_cur = (kk == 0) ? xb1_count<TM, TN>(g) : 0;
                 wait_lgkm<2 + c_prev + c_cur>();
+                if constexpr (g == TN) {
+                    // this wave now holds all its activation fragments of the stage in registers; once
+                    // every wave does, the activation buffer is free for the stage after next
+                    __builtin_amdgcn_s_barrier();
+                    if (more) issue_x(std::integral_constant<int, 0>{}, xcur, kt + 2);
+                }
             }
 #pragma unroll
-            for (int i = 0; i < TM; ++i) mfma_i8(acc[j][i], wa[g % 3], kk ? xb1[i] : xb0[i]);
+            for (int i = 0; i < TM; ++i) mfma_i8(acc[j][i], wa[g % R], kk ? xb1[i] : xb0[i]);
         });
         // the next stage numbers its groups from 0 again
-        if constexpr (G % 3 != 0) {
+        if constexpr (G % R != 0) {
             wait_lgkm<0>();
-            const v4i t0 = wa[G % 3], t1 = wa[(G + 1) % 3];
+            const v4i t0 = wa[G % R], t1 = wa[(G + 1) % R];
             wa[0] = t0;
             wa[1] = t1;
+        }
+        {
+            const unsigned t = xcur; xcur = xnxt; xnxt = t;
+            if constexpr (NWB == 3) { const unsigned u = wcur; wcur = wnxt; wnxt = wnn; wnn = u; }
+            else { const unsigned u = wcur; wcur = wnxt; wnxt = u; }
         }
     }
     // drain the trailing fragment reads; 2 x 16 wait states cover the longest MFMA-result -> VALU-read hazard
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
 
-    // epilogue: lane holds channels nb + 4*g_ .. +3 of token mrow + r for each (i, j)
+    // epilogue: lane holds channels nb + 4*g_ .. +3 of token mrow + r for each (i, j).  Every scale is
+    // fetched before the first store: the memory counter is shared by loads and stores and counts in
+    // order, so a load issued between stores would wait for all stores before it
     const bool lo = r < 8;
+    float sxA[TM], sxB[TM], sxO[TM];
+    float4 swP[(TN + 1) / 2];
+    if constexpr (DEQ) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int mrow = m0 + (wm * TM + i) * 16;
-        const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7);
-        float sxA = 0.0f, sxB = 0.0f;
-        if constexpr (DEQ) {
-            sxA = sx[mA < M ? mA : M - 1];
-            sxB = sx[mB < M ? mB : M - 1];
+        for (int i = 0; i < TM; ++i) {
+            const int mrow = m0 + (wm * TM + i) * 16;
+            const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7), mO = mrow + r;
+            sxA[i] = sx[mA < M ? mA : M - 1];
+            sxB[i] = sx[mB < M ? mB : M - 1];
+            if constexpr (TN & 1) sxO[i] = sx[mO < M ? mO : M - 1];
         }
 #pragma unroll
-        for (int j = 0; j + 1 < TN; j += 2) {
-            const int nb0 = n0 + (wn * TN + j) * 16;
-            const v4i a0 = acc[j][i], a1 = acc[j + 1][i];
-            v4i t0, t1;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                t0[e] = ror8(a0[e]);
-                t1[e] = ror8(a1[e]);
-            }
-            const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
-            const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
-            const int n = nb0 + (lo ? 0 : 16) + 4 * g_;
-            if (n < N) {
-                float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                if constexpr (DEQ) s4 = *reinterpret_cast<const float4 *>(sw + n);
-                if (mA < M) store4<DEQ>(y, acc_out, (int64_t)mA * N + n, vA, sxA, s4);
-                if (mB < M) store4<DEQ>(y, acc_out, (int64_t)mB * N + n, vB, sxB, s4);
-            }
-        }
-        if constexpr (TN & 1) {
-            constexpr int j = TN - 1;
-            const int m = mrow + r;
-            const int n = n0 + (wn * TN + j) * 16 + 4 * g_;
-            if (m < M && n < N) {
-                float sxm = 0.0f;
-                float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                if constexpr (DEQ) {
-                    sxm = sx[m];
-                    s4 = *reinterpret_cast<const float4 *>(sw + n);
-                }
-                store4<DEQ>(y, acc_out, (int64_t)m * N + n, acc[j][i], sxm, s4);
-            }
+        for (int j = 0; j < TN; j += 2) {
+            int n = n0 + (wn * TN + j) * 16 + ((!lo && j + 1 < TN) ? 16 : 0) + 4 * g_;
+            if (n > N - 4) n = N - 4;
+            swP[j / 2] = *reinterpret_cast<const float4 *>(sw + n);
         }
     }
+    // interior tiles take a branch-free path: with divergent branches between the stores the compiler
+    // can no longer count how many are in flight and falls back to waiting for each one
+    auto emit = [&](auto CHECKED) {
+        constexpr bool checked = decltype(CHECKED)::value;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mrow = m0 + (wm * TM + i) * 16;
+            const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7);
+#pragma unroll
+            for (int j = 0; j + 1 < TN; j += 2) {
+                const int nb0 = n0 + (wn * TN + j) * 16;
+                const v4i a0 = acc[j][i], a1 = acc[j + 1][i];
+                v4i t0, t1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    t0[e] = ror8(a0[e]);
+                    t1[e] = ror8(a1[e]);
+                }
+                const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
+                const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
+                const int n = nb0 + (lo ? 0 : 16) + 4 * g_;
+                if (!checked || n < N) {
+                    if (!checked || mA < M) store4<DEQ>(y, acc_out, (int64_t)mA * N + n, vA, sxA[i], swP[j / 2]);
+                    if (!checked || mB < M) store4<DEQ>(y, acc_out, (int64_t)mB * N + n, vB, sxB[i], swP[j / 2]);
+                }
+            }
+            if constexpr (TN & 1) {
+                constexpr int j = TN - 1;
+                const int m = mrow + r;
+                const int n = n0 + (wn * TN + j) * 16 + 4 * g_;
+                if (!checked || (m < M && n < N)) store4<DEQ>(y, acc_out, (int64_t)m * N + n, acc[j][i], sxO[i], swP[j / 2]);
+            }
+        }
+    };
+    if (m0 + BM <= M && n0 + BN <= N) emit(std::false_type{});
+    else emit(std::true_type{});
 }
 
 struct TileShape {
@@ -309,7 +393,7 @@ static int32_t launch_shape(const int8_t *qx, const float *sx, const int8_t *qw,
                             float *y, int M, int N, int K, hipStream_t s)
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
-    constexpr int LDS = 2 * (BM / 8 + BN / 8) * 1024;
+    constexpr int LDS = TiledCfg<TM, TN>::LDS;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_w8a8_tiled<TM, TN, DEQ>),
@@ -340,7 +424,7 @@ int32_t launch_tiled(const int8_t *qx, const float *sx, const int8_t *qw, const 
 {
     const int M = (int)M64, N = (int)N64, K = (int)K64;
     const int cus = compute_units();
-    // pick the tile whose (rounds of tiles over the CUs) x (tile area) is least
+    // pick the tile with the least (rounds of tiles over the chip) x (work a compute unit does per round)
     const TileShape shapes[] = {{8, 8}, {8, 7}, {8, 6}, {4, 8}, {4, 4}};
     int pick = 0;
     double best = 0;
@@ -348,10 +432,12 @@ int32_t launch_tiled(const int8_t *qx, const float *sx, const int8_t *qw, const 
         const int bm = 32 * shapes[i].tm, bn = 32 * shapes[i].tn;
         const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         const int per_cu = (shapes[i].tm * shapes[i].tn <= 16) ? 2 : 1;  // small tiles fit twice in LDS
-        const int64_t rounds = (tiles + (int64_t)cus * per_cu - 1) / ((int64_t)cus * per_cu);
-        // smaller tiles re-read more operand bytes per MFMA: mild penalty
-        const double eff = (shapes[i].tm * shapes[i].tn >= 48) ? 1.0 : (shapes[i].tm * shapes[i].tn >= 32 ? 1.08 : 1.3);
-        const double cost = (double)rounds * bm * bn * eff / per_cu;
+        const int64_t slots = (int64_t)cus * per_cu;
+        const int64_t rounds = (tiles + slots - 1) / slots;
+        // co-resident tiles share the compute unit's MFMA and LDS; smaller wave tiles read more LDS bytes per MFMA
+        const int area = shapes[i].tm * shapes[i].tn;
+        const double eff = area >= 48 ? 1.0 : (area >= 32 ? 1.08 : 1.5);
+        const double cost = (double)rounds * per_cu * bm * bn * eff;
         if (i == 0 || cost < best) { best = cost; pick = i; }
     }
     switch (pick) {
