@@ -127,57 +127,81 @@ __device__ __forceinline__ void fold_slots(float (&p)[64], int lane)
     }
 }
 
-constexpr int WAVE_GROUPS = 16;   // 8-token groups per wave: a workgroup covers at most 4 * 16 * 8 = 512 tokens
+constexpr int WAVE_TILES = 8;     // 16-token tiles per wave: a workgroup covers at most 4 * 8 * 16 = 512 tokens
+constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each)
 
-template <bool DUMP>
-__global__ __launch_bounds__(256) void k_gqa_split(Params p)
+// RAGGED: the span of this workgroup runs past the end of the cache or of its split; token indices are
+// clamped for the loads and masked in the scores.  Otherwise every address is base + constant.
+template <bool DUMP, bool RAGGED>
+__device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
+                                               float (&s_red)[4][4][D], float (&s_sc)[4][WAVE_TILES][16][4],
+                                               float (&s_m)[4][4], float (&s_l)[4][4], float (&s_c)[4][4])
 {
-    __shared__ __attribute__((aligned(16))) int8_t s_q[4][4][D];
-    __shared__ float s_sq[4][4];
-    __shared__ float s_red[4][4][D];
-    __shared__ float s_m[4][4], s_l[4][4], s_c[4][4];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int split = blockIdx.x, bkv = blockIdx.y;
     const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
     const int G = p.G, T = p.T;
     const int ntiles = (T + 15) >> 4;
     const int tile_lo = split * p.tiles_per_split;
     const int tile_hi = min(tile_lo + p.tiles_per_split, ntiles);
-    // lane layout of both passes: token slot = l/8 of an 8-token group, 16-byte chunk = l%8; head = l%4
-    const int hh = lane & 3, slot = lane >> 3, chunk = lane & 7;
     const int t_lo = tile_lo << 4;
-    const int ngroups = max(0, min(tile_hi << 4, T) - t_lo + 7) >> 3;   // 8-token groups of this split
-    const int8_t *kbase = p.kq + (int64_t)bkv * T * D + 16 * chunk;
-    const int8_t *vbase = p.vq + (int64_t)bkv * T * D + 16 * chunk;
-    const float *ksb = p.ks + (int64_t)bkv * T;
-    const float *vsb = p.vs + (int64_t)bkv * T;
+    const int t_end = min(tile_hi << 4, T);   // first token this workgroup does not own
+    // pass 1 lane layout (MFMA operand B): token l%16 of a 16-token tile, 16-byte chunk l/16 (+4 for the
+    // second half of the head dimension); pass 2 lane layout: token slot l/8 of an 8-token group, chunk l%8
+    const int tk16 = lane & 15, ck = lane >> 4;
+    const int hh = lane & 3, slot = lane >> 3, chunk = lane & 7;
+    const int t_wave = t_lo + wave * 16;      // first token of this wave's tile 0; tile j starts 64 tokens further
+    const int8_t *kwave = p.kq + ((int64_t)bkv * T + t_wave) * D;
+    const int8_t *vwave = p.vq + ((int64_t)bkv * T + t_wave) * D;
+    const float *kswave = p.ks + (int64_t)bkv * T + t_wave;
+    const float *vswave = p.vs + (int64_t)bkv * T + t_wave;
+    const unsigned koff = (unsigned)(tk16 * D + 16 * ck);
 
-    // ---- every K byte of this wave and the first half of its V bytes are requested before anything else:
-    // one load = 8 tokens x 128 B contiguous; wave w takes groups w, w+4, ...
-    v4i kv[WAVE_GROUPS], va[WAVE_GROUPS / 2];
-    float ksv[WAVE_GROUPS], vsa[WAVE_GROUPS / 2];
-#pragma unroll
-    for (int u = 0; u < WAVE_GROUPS; ++u) {
-        const int tk = min(t_lo + (wave + 4 * u) * 8 + slot, T - 1);
-        kv[u] = *reinterpret_cast<const v4i *>(kbase + (int64_t)tk * D);
-        ksv[u] = ksb[tk];
-    }
-#pragma unroll
-    for (int u = 0; u < WAVE_GROUPS / 2; ++u) {
-        const int tk = min(t_lo + (wave + 4 * u) * 8 + slot, T - 1);
-        va[u] = *reinterpret_cast<const v4i *>(vbase + (int64_t)tk * D);
-        vsa[u] = vsb[tk];
-    }
+    // the query row goes first: loads return in order, and the rotation of q can then run under the key loads
+    const int hr = lane >> 4, jj = lane & 15;
+    const int head = kvh * G + min(hr, G - 1);
+    const float *qr = p.q + ((int64_t)b * p.Hq + head) * D;
+    const float4 qlo = *reinterpret_cast<const float4 *>(qr + 4 * jj);
+    const float4 qhi = *reinterpret_cast<const float4 *>(qr + 64 + 4 * jj);
 
-    // ---- query heads of this group: rotate, quantize, park the codes in LDS
+    // ---- the wave streams its 8 key tiles (two 1 KB loads each) and then its 16 value groups (one 1 KB load
+    // each) through a ring of RING register slots.  A slot is refilled as soon as it has been consumed, so RING
+    // KB stay in flight per wave from the first instruction to the last and the arithmetic runs under the stream.
+    v4i ring[RING];
+    float ksr[RING / 2], vsr[RING];
+    auto load_k = [&](int j) {   // tile j -> slots (2j) % RING, (2j+1) % RING
+        if constexpr (RAGGED) {
+            const int tk = min(t_wave + j * 64 + tk16, T - 1) - t_wave;
+            ring[(2 * j) % RING] = *reinterpret_cast<const v4i *>(kwave + (int64_t)tk * D + 16 * ck);
+            ring[(2 * j + 1) % RING] = *reinterpret_cast<const v4i *>(kwave + (int64_t)tk * D + 64 + 16 * ck);
+            ksr[j % (RING / 2)] = kswave[tk];
+        } else {
+            ring[(2 * j) % RING] = *reinterpret_cast<const v4i *>(kwave + (koff + (unsigned)(j * 64 * D)));
+            ring[(2 * j + 1) % RING] = *reinterpret_cast<const v4i *>(kwave + (koff + (unsigned)(j * 64 * D + 64)));
+            ksr[j % (RING / 2)] = kswave[(unsigned)(j * 64) + (unsigned)tk16];
+        }
+    };
+    auto load_v = [&](int u) {   // group u = 2*tile + half -> slot (2*WAVE_TILES + u) % RING
+        const int j = u >> 1, g = u & 1;
+        if constexpr (RAGGED) {
+            const int tk = min(t_wave + j * 64 + g * 8 + slot, T - 1) - t_wave;
+            ring[(2 * WAVE_TILES + u) % RING] = *reinterpret_cast<const v4i *>(vwave + (int64_t)tk * D + 16 * chunk);
+            vsr[u % RING] = vswave[tk];
+        } else {
+            ring[(2 * WAVE_TILES + u) % RING] =
+                *reinterpret_cast<const v4i *>(vwave + ((unsigned)(lane * 16) + (unsigned)(j * 64 * D + g * 8 * D)));
+            vsr[u % RING] = vswave[(unsigned)(j * 64 + g * 8) + (unsigned)slot];
+        }
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < RING / 2; ++j) load_k(j);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- query heads of this group: every wave rotates and quantizes them for itself (no workgroup barrier)
     {
-        const int hr = lane >> 4, jj = lane & 15;
-        const int head = kvh * G + min(hr, G - 1);
-        const float *qr = p.q + ((int64_t)b * p.Hq + head) * D;
-        const float4 lo = *reinterpret_cast<const float4 *>(qr + 4 * jj);
-        const float4 hi = *reinterpret_cast<const float4 *>(qr + 64 + 4 * jj);
-        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        float v[8] = {qlo.x, qlo.y, qlo.z, qlo.w, qhi.x, qhi.y, qhi.z, qhi.w};
         fwht128(v, jj);
         float a = 0.0f;
 #pragma unroll
@@ -201,81 +225,96 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
             }
         }
     }
-    __syncthreads();
-    v4i qd[4];       // query codes of the 4 heads for this lane's chunk
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // MFMA operand A: row l%16 = query head (rows >= G are zero), 16-byte chunk l/16 (+4)
+    v4i qa0 = {0, 0, 0, 0}, qa1 = {0, 0, 0, 0};
+    if (tk16 < G) {
+        qa0 = *reinterpret_cast<const v4i *>(&s_q[wave][tk16][16 * ck]);
+        qa1 = *reinterpret_cast<const v4i *>(&s_q[wave][tk16][64 + 16 * ck]);
+    }
+    float cq[4];     // per-head factor of the score, log2 units
 #pragma unroll
-    for (int h = 0; h < 4; ++h)
-        qd[h] = h < G ? *reinterpret_cast<const v4i *>(&s_q[wave][h][16 * chunk]) : (v4i){0, 0, 0, 0};
-    const float cq = hh < G ? s_sq[wave][hh] * p.score_scale : 0.0f;   // per-head factor of the score, log2 units
+    for (int h = 0; h < 4; ++h) cq[h] = h < G ? s_sq[wave][h] * p.score_scale : 0.0f;
 
-    // ---- pass 1: scores.  v_dot4_i32_i8 against the 4 heads, then the 8 lanes of a token add up
-    // (xor 1, 2, 4).  The score of (token l/8, head l%4) stays in a register, in log2 units.
-    float sc[WAVE_GROUPS];
-    float mx = -INFINITY;
+    // ---- pass 1: scores.  Two v_mfma_i32_16x16x64_i8 per tile give the exact int32 dot products of the 16
+    // tokens with the G heads; lane l < 16 holds token l, register r = head r.  Scores (log2 units) go to LDS.
+    float m4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
-    for (int u = 0; u < WAVE_GROUPS; ++u) {
-        const int gi = wave + 4 * u;
-        const int tt = t_lo + gi * 8 + slot;
-        int d[4];
+    for (int j = 0; j < WAVE_TILES; ++j) {
+        v4i dots = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa0, ring[(2 * j) % RING], (v4i){0, 0, 0, 0}, 0, 0, 0);
+        dots = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa1, ring[(2 * j + 1) % RING], dots, 0, 0, 0);
+        const float kscale = ksr[j % (RING / 2)];
+        // the two slots are free: next key tile, or the first value groups once the keys are all requested
+        if (j + RING / 2 < WAVE_TILES) load_k(j + RING / 2);
+        else { load_v(2 * (j + RING / 2 - WAVE_TILES)); load_v(2 * (j + RING / 2 - WAVE_TILES) + 1); }
+        __builtin_amdgcn_sched_barrier(0);
+        const int tt = t_wave + j * 64 + tk16;
+        const bool live = !RAGGED || tt < t_end;
+        float4 sc;
+        sc.x = live ? (float)dots[0] * (kscale * cq[0]) : -INFINITY;
+        sc.y = live ? (float)dots[1] * (kscale * cq[1]) : -INFINITY;
+        sc.z = live ? (float)dots[2] * (kscale * cq[2]) : -INFINITY;
+        sc.w = live ? (float)dots[3] * (kscale * cq[3]) : -INFINITY;
+        if (lane < 16) {
+            *reinterpret_cast<float4 *>(&s_sc[wave][j][tk16][0]) = sc;
+            m4[0] = fmaxf(m4[0], sc.x); m4[1] = fmaxf(m4[1], sc.y);
+            m4[2] = fmaxf(m4[2], sc.z); m4[3] = fmaxf(m4[3], sc.w);
+            if constexpr (DUMP) {
+                if (live) {
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
-            int a = __builtin_amdgcn_sdot4(kv[u][0], qd[h][0], 0, false);
-            a = __builtin_amdgcn_sdot4(kv[u][1], qd[h][1], a, false);
-            a = __builtin_amdgcn_sdot4(kv[u][2], qd[h][2], a, false);
-            a = __builtin_amdgcn_sdot4(kv[u][3], qd[h][3], a, false);
-            a += __builtin_amdgcn_update_dpp(0, a, 0xB1, 0xf, 0xf, true);   // lane ^ 1
-            a += __builtin_amdgcn_update_dpp(0, a, 0x4E, 0xf, 0xf, true);   // lane ^ 2
-            a += __builtin_amdgcn_ds_swizzle(a, 0x101F);                    // lane ^ 4
-            d[h] = a;
+                    for (int h = 0; h < 4; ++h)
+                        if (h < G) p.dump_dots[((int64_t)b * p.Hq + kvh * G + h) * T + tt] = dots[h];
+                }
+            }
         }
-        const int mine = hh == 0 ? d[0] : hh == 1 ? d[1] : hh == 2 ? d[2] : d[3];
-        const bool live = gi < ngroups && tt < T;
-        sc[u] = live ? (float)mine * (ksv[u] * cq) : -INFINITY;
-        if constexpr (DUMP) {
-            if (live && hh < G && chunk < 4) p.dump_dots[((int64_t)b * p.Hq + kvh * G + hh) * T + tt] = mine;
-        }
-        mx = fmaxf(mx, sc[u]);
     }
-    // the key registers are free: request the second half of V
-    v4i vb[WAVE_GROUPS / 2];
-    float vsb2[WAVE_GROUPS / 2];
+    // maximum per head over the wave's tokens (lanes 0..15 hold partial maxima, the rest hold -inf); the softmax
+    // of this wave is taken against the wave's own maximum and rescaled when the waves meet
 #pragma unroll
-    for (int u = 0; u < WAVE_GROUPS / 2; ++u) {
-        const int tk = min(t_lo + (wave + 4 * (u + WAVE_GROUPS / 2)) * 8 + slot, T - 1);
-        vb[u] = *reinterpret_cast<const v4i *>(vbase + (int64_t)tk * D);
-        vsb2[u] = vsb[tk];
+    for (int h = 0; h < 4; ++h) {
+        m4[h] = fmaxf(m4[h], lane_xor<1>(m4[h]));
+        m4[h] = fmaxf(m4[h], lane_xor<2>(m4[h]));
+        m4[h] = fmaxf(m4[h], lane_xor<4>(m4[h]));
+        m4[h] = fmaxf(m4[h], lane_xor<8>(m4[h]));
     }
-    // lanes that share l%4 hold partial maxima of head l%4
-    mx = fmaxf(mx, slot_xor<8>(mx));
-    mx = fmaxf(mx, slot_xor<16>(mx));
-    mx = fmaxf(mx, slot_xor<32>(mx));
-    if (lane < 4) s_m[wave][lane] = mx;
-    __syncthreads();
+    if (lane == 0) { s_m[wave][0] = m4[0]; s_m[wave][1] = m4[1]; s_m[wave][2] = m4[2]; s_m[wave][3] = m4[3]; }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float m_h = s_m[wave][hh];
 
     // ---- pass 2: P.V on the fp32 matrix pipe
-    const float m_h = fmaxf(fmaxf(s_m[0][hh], s_m[1][hh]), fmaxf(s_m[2][hh], s_m[3][hh]));
     const bool counts = (lane & 4) == 0;  // each (token, head) is held by two lanes; one of them counts
     v4f acc[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = (v4f){0.f, 0.f, 0.f, 0.f};
     float lsum = 0.0f, csum = 0.0f;
-    auto pv = [&](const v4i &vv, float vscale, float score) {
-        const float pe = __builtin_amdgcn_exp2f(score - m_h);   // masked tokens: exp2(-inf) = 0
-        const float a = pe * vscale;
-        if (counts) { lsum += pe; csum += a; }
+#pragma unroll
+    for (int u = 0; u < 2 * WAVE_TILES; ++u) {
+        const v4i vv = ring[(2 * WAVE_TILES + u) % RING];
+        const float vscale = vsr[u % RING];
+        // int8 -> fp32 as (byte ^ 0x80) - 128: v_cvt_f32_ubyteN on the biased byte, the bias leaves at the end
+        float f[16];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const uint32_t x = (uint32_t)vv[w] ^ 0x80808080u;
-            acc[4 * w + 0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x & 0xffu), acc[4 * w + 0], 0, 0, 0);
-            acc[4 * w + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 8) & 0xffu), acc[4 * w + 1], 0, 0, 0);
-            acc[4 * w + 2] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)((x >> 16) & 0xffu), acc[4 * w + 2], 0, 0, 0);
-            acc[4 * w + 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, (float)(x >> 24), acc[4 * w + 3], 0, 0, 0);
+            f[4 * w + 0] = (float)(x & 0xffu);
+            f[4 * w + 1] = (float)((x >> 8) & 0xffu);
+            f[4 * w + 2] = (float)((x >> 16) & 0xffu);
+            f[4 * w + 3] = (float)(x >> 24);
         }
-    };
+        if (u + RING < 2 * WAVE_TILES) load_v(u + RING);
+        __builtin_amdgcn_sched_barrier(0);
+        const float score = s_sc[wave][u >> 1][8 * (u & 1) + slot][hh];
+        // a wave whose tokens are all masked has m_h = -inf: exp2(-inf - -inf) would be NaN
+        const float pe = (score == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(score - m_h);
+        const float a = pe * vscale;
+        if (counts) { lsum += pe; csum += a; }
 #pragma unroll
-    for (int u = 0; u < WAVE_GROUPS / 2; ++u) pv(va[u], vsa[u], sc[u]);
-#pragma unroll
-    for (int u = 0; u < WAVE_GROUPS / 2; ++u) pv(vb[u], vsb2[u], sc[u + WAVE_GROUPS / 2]);
+        for (int e = 0; e < 16; ++e) acc[e] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, f[e], acc[e], 0, 0, 0);
+    }
 
     // sum the 8 token slots (lanes that share l%8): transposed butterfly over lane bits 5, 4, 3, after which
     // lane l holds the 8 totals with flat index 8*(l/8) .. +7, flat = 4*e + head  (56 shuffles, not 192)
@@ -297,45 +336,96 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     if (lane < 4) { s_l[wave][lane] = lsum; s_c[wave][lane] = csum; }
     __syncthreads();
 
+    // the four waves meet: rescale each wave's sums from its own maximum to the common one
     const int64_t pbase = ((int64_t)bkv * gridDim.x + split);
     for (int o = tid; o < 4 * D; o += 256) {
         const int h = o >> 7, d = o & (D - 1);
-        const float c = s_c[0][h] + s_c[1][h] + s_c[2][h] + s_c[3][h];
-        const float sum = s_red[0][h][d] + s_red[1][h][d] + s_red[2][h][d] + s_red[3][h][d];
-        p.part_o[(pbase * 4 + h) * D + d] = sum - 128.0f * c;
+        const float m = fmaxf(fmaxf(s_m[0][h], s_m[1][h]), fmaxf(s_m[2][h], s_m[3][h]));
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float f = (s_m[w][h] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(s_m[w][h] - m);
+            sum += (s_red[w][h][d] - 128.0f * s_c[w][h]) * f;
+        }
+        p.part_o[(pbase * 4 + h) * D + d] = sum;
     }
     if (tid < 4) {
-        p.part_ml[pbase * 8 + tid] = fmaxf(fmaxf(s_m[0][tid], s_m[1][tid]), fmaxf(s_m[2][tid], s_m[3][tid]));
-        p.part_ml[pbase * 8 + 4 + tid] = s_l[0][tid] + s_l[1][tid] + s_l[2][tid] + s_l[3][tid];
+        const float m = fmaxf(fmaxf(s_m[0][tid], s_m[1][tid]), fmaxf(s_m[2][tid], s_m[3][tid]));
+        float l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) l += (s_m[w][tid] == -INFINITY) ? 0.0f : s_l[w][tid] * __builtin_amdgcn_exp2f(s_m[w][tid] - m);
+        p.part_ml[pbase * 8 + tid] = m;
+        p.part_ml[pbase * 8 + 4 + tid] = l;
     }
 }
 
-// merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row
+template <bool DUMP>
+__global__ __launch_bounds__(256) void k_gqa_split(Params p)
+{
+    __shared__ __attribute__((aligned(16))) int8_t s_q[4][4][D];
+    __shared__ float s_sq[4][4];
+    __shared__ float s_red[4][4][D];
+    __shared__ __attribute__((aligned(16))) float s_sc[4][WAVE_TILES][16][4];
+    __shared__ float s_m[4][4], s_l[4][4], s_c[4][4];
+    const int tile_lo = blockIdx.x * p.tiles_per_split;
+    const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= p.T && p.tiles_per_split >= 4 * WAVE_TILES;
+    if (full) gqa_split_body<DUMP, false>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+    else gqa_split_body<DUMP, true>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+}
+
+// merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row.  SP > 0: the split count is known at
+// compile time and every load of the row goes out before the first use (one memory round trip).
+template <int SP>
 __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ part_o,
                                                    const float *__restrict__ part_ml, float *__restrict__ o,
-                                                   int rows, int Hq, int Hkv, int G, int splits, int out_rotated)
+                                                   int rows, int Hq, int Hkv, int G, int splits_rt, int out_rotated)
 {
+    const int splits = SP > 0 ? SP : splits_rt;
     const int tid = threadIdx.x, j = tid & 15;
     const int row = blockIdx.x * 16 + (tid >> 4);
     const bool live = row < rows;
     const int rr = live ? row : rows - 1;
     const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
     const int64_t bkv = (int64_t)b * Hkv + kvh;
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, part_ml[(bkv * splits + s) * 8 + hl]);
+    const float *ml0 = part_ml + bkv * splits * 8;
+    const float *po0 = part_o + (bkv * splits * 4 + hl) * attn::D;
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float l = 0.0f;
-    for (int s = 0; s < splits; ++s) {
-        const float *ml = part_ml + (bkv * splits + s) * 8;
-        const float w = __builtin_amdgcn_exp2f(ml[hl] - mx);
-        l = __builtin_fmaf(ml[4 + hl], w, l);
-        const float *po = part_o + ((bkv * splits + s) * 4 + hl) * attn::D;
-        const float4 lo = *reinterpret_cast<const float4 *>(po + 4 * j);
-        const float4 hi = *reinterpret_cast<const float4 *>(po + 64 + 4 * j);
-        v[0] = __builtin_fmaf(lo.x, w, v[0]); v[1] = __builtin_fmaf(lo.y, w, v[1]);
-        v[2] = __builtin_fmaf(lo.z, w, v[2]); v[3] = __builtin_fmaf(lo.w, w, v[3]);
-        v[4] = __builtin_fmaf(hi.x, w, v[4]); v[5] = __builtin_fmaf(hi.y, w, v[5]);
-        v[6] = __builtin_fmaf(hi.z, w, v[6]); v[7] = __builtin_fmaf(hi.w, w, v[7]);
+    if constexpr (SP > 0) {
+        float ms[SP], ls[SP];
+        float4 lo[SP], hi[SP];
+#pragma unroll
+        for (int s = 0; s < SP; ++s) {
+            ms[s] = ml0[s * 8 + hl];
+            ls[s] = ml0[s * 8 + 4 + hl];
+            lo[s] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
+            hi[s] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
+        }
+        float mx = ms[0];
+#pragma unroll
+        for (int s = 1; s < SP; ++s) mx = fmaxf(mx, ms[s]);
+#pragma unroll
+        for (int s = 0; s < SP; ++s) {
+            const float w = __builtin_amdgcn_exp2f(ms[s] - mx);
+            l = __builtin_fmaf(ls[s], w, l);
+            v[0] = __builtin_fmaf(lo[s].x, w, v[0]); v[1] = __builtin_fmaf(lo[s].y, w, v[1]);
+            v[2] = __builtin_fmaf(lo[s].z, w, v[2]); v[3] = __builtin_fmaf(lo[s].w, w, v[3]);
+            v[4] = __builtin_fmaf(hi[s].x, w, v[4]); v[5] = __builtin_fmaf(hi[s].y, w, v[5]);
+            v[6] = __builtin_fmaf(hi[s].z, w, v[6]); v[7] = __builtin_fmaf(hi[s].w, w, v[7]);
+        }
+    } else {
+        float mx = -INFINITY;
+        for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml0[s * 8 + hl]);
+        for (int s = 0; s < splits; ++s) {
+            const float w = __builtin_amdgcn_exp2f(ml0[s * 8 + hl] - mx);
+            l = __builtin_fmaf(ml0[s * 8 + 4 + hl], w, l);
+            const float4 lo = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
+            const float4 hi = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
+            v[0] = __builtin_fmaf(lo.x, w, v[0]); v[1] = __builtin_fmaf(lo.y, w, v[1]);
+            v[2] = __builtin_fmaf(lo.z, w, v[2]); v[3] = __builtin_fmaf(lo.w, w, v[3]);
+            v[4] = __builtin_fmaf(hi.x, w, v[4]); v[5] = __builtin_fmaf(hi.y, w, v[5]);
+            v[6] = __builtin_fmaf(hi.z, w, v[6]); v[7] = __builtin_fmaf(hi.w, w, v[7]);
+        }
     }
     const float rl = 1.0f / l;
 #pragma unroll
@@ -352,7 +442,7 @@ static int pick_splits(int64_t B, int64_t Hkv, int64_t T)
 {
     const int ntiles = (int)((T + 15) / 16);
     const int cus = compute_units();
-    constexpr int MAX_TILES = 4 * WAVE_GROUPS / 2;   // 16-token tiles one workgroup can hold in registers
+    constexpr int MAX_TILES = 4 * WAVE_TILES;   // 16-token tiles one workgroup can hold in registers
     int splits = (ntiles + MAX_TILES - 1) / MAX_TILES;
     // short caches / few heads: more, shorter splits until there are about two workgroups per compute unit
     while (B * Hkv * splits < 2LL * cus && (ntiles + splits - 1) / splits > 8) splits *= 2;
@@ -412,8 +502,18 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     rc = launch_status();
     if (rc || !o) return rc;
     const int rows = (int)(B * Hq);
-    hipLaunchKernelGGL(attn::k_gqa_merge, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, p.part_o, p.part_ml, o,
-                       rows, (int)Hq, (int)Hkv, p.G, splits, out_rotated);
+    const dim3 mgrid((unsigned)((rows + 15) / 16));
+#define MI_MERGE(SP)                                                                                        \
+    hipLaunchKernelGGL(attn::k_gqa_merge<SP>, mgrid, dim3(256), 0, s, p.part_o, p.part_ml, o, rows, (int)Hq, \
+                       (int)Hkv, p.G, splits, out_rotated)
+    switch (splits) {
+    case 1: MI_MERGE(1); break;
+    case 2: MI_MERGE(2); break;
+    case 4: MI_MERGE(4); break;
+    case 8: MI_MERGE(8); break;
+    default: MI_MERGE(0); break;
+    }
+#undef MI_MERGE
     return launch_status();
 }
 

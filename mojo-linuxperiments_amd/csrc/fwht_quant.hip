@@ -98,7 +98,7 @@ __device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d, f
 // One workgroup per row; thread t owns chunks t, t + T, ... (C of them).
 // QUANT: write int8 codes + scale; otherwise write the rotated fp32 row.
 template <int BLOCK, int C, bool QUANT>
-__global__ __launch_bounds__(1024) void k_fwht_rows(const float *x, int8_t *__restrict__ q,
+__global__ __launch_bounds__(256) void k_fwht_rows(const float *x, int8_t *__restrict__ q,
                                                     float *__restrict__ scale, float *xrot, int K)
 {
     constexpr int LPB = BLOCK / 8;
