@@ -127,11 +127,14 @@ __device__ __forceinline__ void fold_slots(float (&p)[64], int lane)
     }
 }
 
-constexpr int WAVE_TILES = 8;     // 16-token tiles per wave: a workgroup covers at most 4 * 8 * 16 = 512 tokens
+#ifndef MI_ATTN_TILES
+#define MI_ATTN_TILES 11
+#endif
+constexpr int WAVE_TILES = MI_ATTN_TILES;   // 16-token tiles per wave: a workgroup covers at most 4 * WAVE_TILES * 16 tokens
 constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each)
 
-// RAGGED: the span of this workgroup runs past the end of the cache or of its split; token indices are
-// clamped for the loads and masked in the scores.  Otherwise every address is base + constant.
+// RAGGED: the span a workgroup can cover runs past the end of the cache and token indices are clamped for the
+// loads; otherwise every address is base + constant.  Tokens past the end of the split are masked in the scores.
 template <bool DUMP, bool RAGGED>
 __device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
                                                float (&s_red)[4][4][D], float (&s_sc)[4][WAVE_TILES][16][4],
@@ -251,7 +254,7 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4]
         else { load_v(2 * (j + RING / 2 - WAVE_TILES)); load_v(2 * (j + RING / 2 - WAVE_TILES) + 1); }
         __builtin_amdgcn_sched_barrier(0);
         const int tt = t_wave + j * 64 + tk16;
-        const bool live = !RAGGED || tt < t_end;
+        const bool live = tt < t_end;
         float4 sc;
         sc.x = live ? (float)dots[0] * (kscale * cq[0]) : -INFINITY;
         sc.y = live ? (float)dots[1] * (kscale * cq[1]) : -INFINITY;
@@ -368,7 +371,7 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     __shared__ __attribute__((aligned(16))) float s_sc[4][WAVE_TILES][16][4];
     __shared__ float s_m[4][4], s_l[4][4], s_c[4][4];
     const int tile_lo = blockIdx.x * p.tiles_per_split;
-    const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= p.T && p.tiles_per_split >= 4 * WAVE_TILES;
+    const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= p.T;
     if (full) gqa_split_body<DUMP, false>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
     else gqa_split_body<DUMP, true>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
 }
@@ -510,6 +513,7 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     case 1: MI_MERGE(1); break;
     case 2: MI_MERGE(2); break;
     case 4: MI_MERGE(4); break;
+    case 6: MI_MERGE(6); break;
     case 8: MI_MERGE(8); break;
     default: MI_MERGE(0); break;
     }
