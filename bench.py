@@ -161,6 +161,14 @@ def main():
         gemm_ms[name] = timer.run(one, max(10, args.steps))
     gemm_total_ms = sum(gemm_ms.values())
     gemm_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
+    # HBM-side bytes per launch of the tiled GEMM, measured with hardware counters in a separate run
+    traffic, traffic_total = None, None
+    tpath = os.path.join(os.path.dirname(os.path.abspath(mi.__file__)), "hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as fh:
+            per = json.load(fh)["tiled_gemm_bytes_per_launch"]
+        traffic = {k: v["fetch"] + v["write"] for k, v in per.items()}
+        traffic_total = sum(traffic.values())
     roofline = {
         "kernel": "k_w8a8_tiled (v_mfma_i32_16x16x64_i8), four cfg3 shapes, ops-weighted",
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
