@@ -148,8 +148,11 @@ __global__ __launch_bounds__(256) void k_moe_topk(const float *__restrict__ logi
 // One workgroup.  bm[e][t/32] bit t%32 = "token t picked expert e" (a token
 // picks an expert at most once), so the stable rank of pair (t, slot) inside
 // its expert is the number of set bits below t in row e.
+// order (optional): expert ids by descending segment size, so that the grouped GEMMs can start their longest
+// workgroups first.
 __global__ __launch_bounds__(1024) void k_moe_dispatch(const int32_t *__restrict__ idx, int32_t *__restrict__ perm,
-                                                       int32_t *__restrict__ seg_off, int T, int E, int topk)
+                                                       int32_t *__restrict__ seg_off, int32_t *__restrict__ order,
+                                                       int T, int E, int topk)
 {
     extern __shared__ uint32_t s_dyn[];
     const int W = (T + 31) >> 5;
@@ -180,6 +183,17 @@ __global__ __launch_bounds__(1024) void k_moe_dispatch(const int32_t *__restrict
     }
     __syncthreads();
     for (int e = tid; e <= E; e += nt) seg_off[e] = seg[e];
+    if (order) {
+        for (int e = tid; e < E; e += nt) {
+            const int c = seg[e + 1] - seg[e];
+            int rank = 0;
+            for (int o = 0; o < E; ++o) {
+                const int co = seg[o + 1] - seg[o];
+                rank += (co > c || (co == c && o < e)) ? 1 : 0;
+            }
+            order[rank] = e;
+        }
+    }
     for (int pr = tid; pr < P; pr += nt) {
         const int e = idx[pr], t = pr / topk;
         if (e < 0 || e >= E) continue;
@@ -371,6 +385,229 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
     }
 }
 
+// The same contraction with the activation fragments held in registers (possible when a wave's K slice is at
+// most NSMAX steps of 128 bytes): only weights travel through the ring, twice as many of them are in flight
+// for the same LDS, and a workgroup walks several row chunks against one set of activation registers.
+constexpr int RX_RING = 3;
+constexpr int RX_STAGE = 2 * NGRP * 1024;
+constexpr int RX_RING_BYTES = 4 * RX_RING * RX_STAGE;
+constexpr int RX_MT = 3;   // most 16-token fragments per pass
+constexpr int RX_LDS = RX_RING_BYTES + 4 * NGRP * RX_MT * 4 * 64 * 4 + 16 * RX_MT * 8 + 8 * 128 * 4;   // + metadata + scales of <= 8 chunks
+
+template <bool DOWN, int NSMAX, int MTT>
+__device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ act,
+                                                         const float *__restrict__ act_scale,
+                                                         const int32_t *__restrict__ perm,
+                                                         const int32_t *__restrict__ seg_off,
+                                                         const int8_t *__restrict__ w0, const float *__restrict__ sc0,
+                                                         const int8_t *__restrict__ w1, const float *__restrict__ sc1,
+                                                         float *__restrict__ out, int Kdim, int Nrows, int Hout,
+                                                         int topk, int nch, int e)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int seg0 = seg_off[e], count = seg_off[e + 1] - seg0;
+    if (count <= 0) return;
+    // gate/up: the 4 waves split K (2048 bytes = 16 steps).  down: K is short (768 bytes = 6 steps), so each
+    // wave takes its own 32 rows over the whole of K and nothing has to be added across waves
+    // A workgroup walks `nch` consecutive row chunks (16 rows for gate/up, 128 for down) as ONE stream: the
+    // loads of the next chunk are already in flight while the partial sums of this one are added and stored,
+    // and the segment / permutation lookups are paid once per workgroup.
+    constexpr int CHUNK_ROWS = DOWN ? 128 : 16;
+    const int n0 = DOWN ? blockIdx.x * nch * 128 + wave * 32 : blockIdx.x * nch * 16;
+    char *ring = smem + wave * (RX_RING * RX_STAGE);
+    int *s_part = reinterpret_cast<int *>(smem + RX_RING_BYTES);   // [4 waves][NGRP][MTT][4][64]
+    // per-pass token metadata and per-chunk weight scales sit in LDS so that the epilogue of a chunk issues no
+    // dependent global loads (each would cost a memory round trip per chunk)
+    int *s_dst = reinterpret_cast<int *>(smem + RX_RING_BYTES + 4 * NGRP * MTT * 4 * 64 * 4);   // [16*MTT] output row
+    float *s_tsc = reinterpret_cast<float *>(s_dst + 16 * MTT);                                  // [16*MTT] token scale
+    float *s_wsc = s_tsc + 16 * MTT;                                                             // [nch][SCW]
+    constexpr int SCW = DOWN ? 128 : 32;
+    for (int o = tid; o < nch * SCW; o += 256) {
+        const int ch = o / SCW, nl = o - ch * SCW;
+        float v = 0.0f;
+        if constexpr (DOWN) {
+            const int n = (blockIdx.x * nch + ch) * 128 + nl;
+            if (n < Nrows) v = sc0[(int64_t)e * Nrows + n];
+        } else {
+            const int n = (blockIdx.x * nch + ch) * 16 + (nl & 15);
+            if (n < Nrows) v = (nl < 16 ? sc0 : sc1)[(int64_t)e * Nrows + n];
+        }
+        s_wsc[o] = v;
+    }
+
+    // load side: lane l = 8*rho + c fetches chunk c ^ sigma(rho, block parity) of row rho of the block
+    const int rho = lane >> 3, c8 = lane & 7;
+    const int8_t *wsrc[2 * NGRP];
+#pragma unroll
+    for (int b = 0; b < 2 * NGRP; ++b) {
+        const int sigma = (rho & 6) | ((rho ^ b) & 1);
+        const int grp = b >> 1;
+        int rowi = n0 + (DOWN ? grp * 16 : 0) + (b & 1) * 8 + rho;
+        if (rowi > Nrows - 1) rowi = Nrows - 1;
+        const int8_t *base = (DOWN || grp == 0) ? w0 : w1;
+        wsrc[b] = base + ((int64_t)e * Nrows + rowi) * Kdim + ((c8 ^ sigma) << 4);
+    }
+    const int steps = Kdim >> 7;
+    const int s0 = DOWN ? 0 : steps * wave / 4, s1 = DOWN ? steps : steps * (wave + 1) / 4;
+
+    // read side: fragment (16-row group, K half kk): lane (r = l%16, g = l/16) reads row r, chunk 4*kk + g
+    const int r = lane & 15, g_ = lane >> 4;
+    int roff[2];
+    {
+        const int rr = r & 7, bpar = r >> 3;
+        const int sigma = (rr & 6) | ((rr ^ bpar) & 1);
+        roff[0] = bpar * 1024 + ((8 * rr + ((0 + g_) ^ sigma)) << 4);
+        roff[1] = bpar * 1024 + ((8 * rr + ((4 + g_) ^ sigma)) << 4);
+    }
+
+    for (int base = 0; base < count; base += 16 * MTT) {
+        const int nsw = s1 - s0;            // K steps of this wave per chunk (<= NSMAX)
+        const int total_f = nch * nsw;      // flattened (chunk, step) stages of this wave
+        auto issue = [&](int slot, int f) {
+            const int fc = f < total_f ? f : total_f - 1;   // past the end: re-fetch the last stage (uniform vmcnt arithmetic)
+            const int ch = fc / nsw, st = s0 + (fc - ch * nsw);
+            char *sb = ring + slot * RX_STAGE;
+            const int64_t woff = (int64_t)ch * CHUNK_ROWS * Kdim + (int64_t)st * 128;
+#pragma unroll
+            for (int b = 0; b < 2 * NGRP; ++b)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[b] + woff), (lptr_t)(sb + b * 1024), 16, 0, 0);
+        };
+        // Activation rows of this pass, as MFMA fragments held in registers for every row chunk the workgroup
+        // walks: lane (token r, 16-byte chunk g_ (+4)).  Rows past the segment repeat its last row and are never
+        // stored.
+        v4i xr[MTT][NSMAX][2];
+        __syncthreads();   // the previous pass has finished with the token metadata and every ring is idle
+        if (tid < 16 * MTT && base + tid < count) {
+            const int pos = seg0 + base + tid;
+            const int pr = perm[pos];
+            s_dst[tid] = DOWN ? pr : pos;
+            s_tsc[tid] = act_scale[DOWN ? pos : pr / topk];
+        }
+        {
+            // the weight stream starts first: its addresses do not depend on the tokens, whose lookups cost two
+            // dependent memory round trips
+            if (nsw > 0) {
+#pragma unroll
+                for (int d = 0; d < RX_RING; ++d) issue(d, d);
+            }
+#pragma unroll
+            for (int b = 0; b < MTT; ++b) {
+                const int pos = seg0 + min(base + b * 16 + r, count - 1);
+                const int8_t *xp = act + (DOWN ? (int64_t)pos : (int64_t)(perm[pos] / topk)) * Kdim + g_ * 16;
+#pragma unroll
+                for (int i = 0; i < NSMAX; ++i) {
+                    const int st = min(s0 + i, steps - 1);
+                    xr[b][i][0] = *reinterpret_cast<const v4i *>(xp + (int64_t)st * 128);
+                    xr[b][i][1] = *reinterpret_cast<const v4i *>(xp + (int64_t)st * 128 + 64);
+                }
+            }
+        }
+
+        int slot = 0, f = 0;
+        for (int ch = 0; ch < nch; ++ch) {
+        const int nc0 = n0 + ch * CHUNK_ROWS;
+        v4i acc[NGRP][MTT];
+#pragma unroll
+        for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+            for (int b = 0; b < MTT; ++b) acc[a][b] = (v4i){0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < NSMAX; ++i) {
+            if (i < nsw) {
+                wait_vm<(RX_RING - 1) * 2 * NGRP>();   // the oldest stage in flight has landed
+                const char *sb = ring + slot * RX_STAGE;
+                v4i wf[NGRP][2];
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                    for (int a = 0; a < NGRP; ++a) wf[a][kk] = *reinterpret_cast<const v4i *>(sb + a * 2048 + roff[kk]);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot may be refilled
+                issue(slot, f + RX_RING);
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                    for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+                        for (int b = 0; b < MTT; ++b)
+                            acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[a][kk], xr[b][i][kk], acc[a][b], 0, 0, 0);
+                slot = slot + 1 == RX_RING ? 0 : slot + 1;
+                ++f;
+            }
+        }
+        __syncthreads();   // the previous chunk's epilogue has finished reading s_part
+#pragma unroll
+        for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+            for (int b = 0; b < MTT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) s_part[(((wave * NGRP + a) * MTT + b) * 4 + q) * 64 + lane] = acc[a][b][q];
+        __syncthreads();
+        // accumulator layout: lane l, register q  <->  weight row 4*(l/16)+q, token l%16
+        auto total = [&](int a, int row, int nn) {
+            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
+            int sum = 0;
+#pragma unroll
+            for (int wv = 0; wv < 4; ++wv) sum += s_part[(((wv * NGRP + a) * MTT + b) * 4 + q) * 64 + src];
+            return sum;
+        };
+        auto own = [&](int wv, int a, int row, int nn) {   // down: one wave's accumulator is already the total
+            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
+            return s_part[(((wv * NGRP + a) * MTT + b) * 4 + q) * 64 + src];
+        };
+        const float *wsc = s_wsc + ch * SCW;
+        if constexpr (!DOWN) {
+            // 32 tokens x 16 channels, channel fastest; h = silu(g) * u in sorted-pair order
+#pragma unroll
+            for (int o = tid; o < 16 * MTT * 16; o += 256) {
+                const int nl = o & 15, row = o >> 4;
+                if (base + row < count && nc0 + nl < Nrows) {
+                    const float sxt = s_tsc[row];
+                    const float gv = ((float)total(0, row, nl) * sxt) * wsc[nl];
+                    const float uv = ((float)total(1, row, nl) * sxt) * wsc[16 + nl];
+                    out[(int64_t)s_dst[row] * Nrows + nc0 + nl] = (gv / (1.0f + expf(-gv))) * uv;
+                }
+            }
+        } else {
+            // 32 tokens x 128 channels (32 per wave); out[pair] in pair order, channel fastest
+            const int nbase = (blockIdx.x * nch + ch) * 128;
+#pragma unroll
+            for (int o = tid; o < 16 * MTT * 128; o += 256) {
+                const int nl = o & 127, row = o >> 7;
+                if (base + row < count && nbase + nl < Nrows) {
+                    const int sum = own(nl >> 5, (nl >> 4) & 1, row, nl & 15);
+                    out[(int64_t)s_dst[row] * Hout + nbase + nl] = ((float)sum * s_tsc[row]) * wsc[nl];
+                }
+            }
+        }
+        }   // chunks
+        wait_vm<0>();   // trailing re-fetches must not write LDS after the workgroup has gone
+    }
+}
+
+template <bool DOWN, int NSMAX>
+__global__ __launch_bounds__(256) void k_moe_expert_rx(const int8_t *__restrict__ act,
+                                                       const float *__restrict__ act_scale,
+                                                       const int32_t *__restrict__ perm,
+                                                       const int32_t *__restrict__ seg_off,
+                                                       const int8_t *__restrict__ w0, const float *__restrict__ sc0,
+                                                       const int8_t *__restrict__ w1, const float *__restrict__ sc1,
+                                                       float *__restrict__ out, int Kdim, int Nrows, int Hout,
+                                                       int topk, int nch, const int32_t *__restrict__ order)
+{
+    // workgroups are handed out in grid order: the experts with the most tokens go first
+    const int e = order[blockIdx.y];
+    // tokens per pass follow the size of the expert's segment: every extra pass streams the weights again
+    const int count = seg_off[e + 1] - seg_off[e];
+    if (count <= 16)
+        moe_expert_rx_body<DOWN, NSMAX, 1>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+    else if (count <= 32 || NSMAX > 6)
+        moe_expert_rx_body<DOWN, NSMAX, 2>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+    else
+        moe_expert_rx_body<DOWN, NSMAX, 3>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+}
+
 // y[t, n] = sum over slots in order of w[t, slot] * out[t*topk + slot, n]
 __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ out, const float *__restrict__ w,
                                                      float *__restrict__ y, int T, int H, int topk)
@@ -395,7 +632,7 @@ struct Layout {
 static Layout layout(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk)
 {
     const int64_t P = T * topk;
-    const int64_t sz[11] = {T * H, T * 4, P * 4, (E + 1) * 4, P * I * 4, P * I, P * 4, P * H * 4, P * 4, P * 4, T * E * 4};
+    const int64_t sz[11] = {T * H, T * 4, P * 4, (2 * E + 1) * 4 /* seg_off, then experts by size */, P * I * 4, P * I, P * 4, P * H * 4, P * 4, P * 4, T * E * 4};
     Layout L;
     int64_t o = 0;
     for (int i = 0; i < 11; ++i) { L.off[i] = o; o += align_up(sz[i], 256); }
@@ -443,8 +680,8 @@ extern "C" int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, f
     return launch_status();
 }
 
-extern "C" int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off, int64_t T, int64_t E,
-                                   int32_t topk, void *stream)
+static int32_t launch_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off, int32_t *order, int64_t T,
+                               int64_t E, int32_t topk, void *stream)
 {
     if (!idx || !perm || !seg_off || T < 0 || E <= 0 || topk <= 0) return MI_EINVAL;
     if (T * topk > (1LL << 24) || E > 65535) return MI_ERANGE;
@@ -457,8 +694,14 @@ extern "C" int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *s
         attr_set = true;
     }
     hipLaunchKernelGGL(moe::k_moe_dispatch, dim3(1), dim3(1024), (size_t)words * 4, as_stream(stream), idx, perm,
-                       seg_off, (int)T, (int)E, (int)topk);
+                       seg_off, order, (int)T, (int)E, (int)topk);
     return launch_status();
+}
+
+extern "C" int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off, int64_t T, int64_t E,
+                                   int32_t topk, void *stream)
+{
+    return launch_dispatch(idx, perm, seg_off, nullptr, T, E, topk, stream);
 }
 
 extern "C" int64_t mi_moe_ffn_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk)
@@ -506,7 +749,8 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     hipStream_t s = as_stream(stream);
     const int64_t P = T * topk;
 
-    rc = mi_moe_dispatch(idx, perm, seg, T, E, topk, stream);
+    int32_t *order = seg + E + 1;
+    rc = launch_dispatch(idx, perm, seg, order, T, E, topk, stream);
     if (rc) return rc;
     rc = mi_fwht_quant_f32_i8(x, qx, sx, T, H, 128, stream);
     if (rc) return rc;
@@ -518,19 +762,68 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
                                    hipFuncAttributeMaxDynamicSharedMemorySize, moe::EXPERT_LDS));
         attr_set = true;
     }
-    // Row chunks per workgroup.  Walking several chunks as one stream measured no faster than one chunk per
-    // workgroup (the activation rows are re-fetched per chunk either way), so one it is.
-    const int nch_gu = 1, nch_dn = 1;
-    hipLaunchKernelGGL(moe::k_moe_expert_gemm<false>, dim3((unsigned)(I / 16 / nch_gu), (unsigned)E), dim3(256),
-                       moe::EXPERT_LDS, s, qx, sx, perm, seg, wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk,
-                       nch_gu);
+    // Row chunks per workgroup: with the activation fragments in registers a workgroup walks several chunks
+    // against them; about four workgroups per compute unit keep the stream dense.
+    const int cus = compute_units();
+    auto pick_nch = [&](int64_t chunks) {
+        int64_t n = chunks * E / (4LL * cus);
+        return (int)(n < 1 ? 1 : (n > 8 ? 8 : n));
+    };
+    const int steps_gu = (int)(H / 128), ns_gu = (steps_gu + 3) / 4;   // K steps per wave (the four waves split K)
+    if (ns_gu <= 8) {
+        const int nch = pick_nch(I / 16);
+        const dim3 grid((unsigned)((I / 16 + nch - 1) / nch), (unsigned)E);
+#define MI_RX_GU(NS)                                                                                            \
+    do {                                                                                                        \
+        static bool set = false;                                                                                \
+        if (!set) {                                                                                             \
+            MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<false, NS>),        \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::RX_LDS));               \
+            set = true;                                                                                         \
+        }                                                                                                       \
+        hipLaunchKernelGGL((moe::k_moe_expert_rx<false, NS>), grid, dim3(256), moe::RX_LDS, s, qx, sx, perm, seg, \
+                           wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk, nch, order);                   \
+    } while (0)
+        if (ns_gu <= 2) MI_RX_GU(2);
+        else if (ns_gu <= 4) MI_RX_GU(4);
+        else MI_RX_GU(8);
+#undef MI_RX_GU
+    } else {
+        hipLaunchKernelGGL(moe::k_moe_expert_gemm<false>, dim3((unsigned)(I / 16), (unsigned)E), dim3(256),
+                           moe::EXPERT_LDS, s, qx, sx, perm, seg, wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk,
+                           1);
+    }
     rc = launch_status();
     if (rc) return rc;
     rc = mi_fwht_quant_f32_i8(h, hq, hs, P, I, 256, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_expert_gemm<true>, dim3((unsigned)((H + 128 * nch_dn - 1) / (128 * nch_dn)), (unsigned)E),
-                       dim3(256), moe::EXPERT_LDS, s, hq, hs, perm, seg, wd, sd, (const int8_t *)nullptr,
-                       (const float *)nullptr, out, (int)I, (int)H, (int)H, (int)topk, nch_dn);
+    const int steps_dn = (int)(I / 128);   // every wave walks the whole of K
+    if (steps_dn <= 8) {
+        const int64_t chunks = (H + 127) / 128;
+        const int nch = pick_nch(chunks);
+        const dim3 grid((unsigned)((chunks + nch - 1) / nch), (unsigned)E);
+#define MI_RX_DN(NS)                                                                                            \
+    do {                                                                                                        \
+        static bool set = false;                                                                                \
+        if (!set) {                                                                                             \
+            MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<true, NS>),         \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::RX_LDS));               \
+            set = true;                                                                                         \
+        }                                                                                                       \
+        hipLaunchKernelGGL((moe::k_moe_expert_rx<true, NS>), grid, dim3(256), moe::RX_LDS, s, hq, hs, perm, seg, wd, \
+                           sd, (const int8_t *)nullptr, (const float *)nullptr, out, (int)I, (int)H, (int)H,    \
+                           (int)topk, nch, order);                                                              \
+    } while (0)
+        if (steps_dn <= 2) MI_RX_DN(2);
+        else if (steps_dn <= 4) MI_RX_DN(4);
+        else if (steps_dn <= 6) MI_RX_DN(6);
+        else MI_RX_DN(8);
+#undef MI_RX_DN
+    } else {
+        hipLaunchKernelGGL(moe::k_moe_expert_gemm<true>, dim3((unsigned)((H + 127) / 128), (unsigned)E), dim3(256),
+                           moe::EXPERT_LDS, s, hq, hs, perm, seg, wd, sd, (const int8_t *)nullptr,
+                           (const float *)nullptr, out, (int)I, (int)H, (int)H, (int)topk, 1);
+    }
     rc = launch_status();
     if (rc) return rc;
     hipLaunchKernelGGL(moe::k_moe_combine, dim3((unsigned)((T * H / 4 + 255) / 256)), dim3(256), 0, s, out, w, y,
