@@ -164,6 +164,67 @@ __global__ __launch_bounds__(256) void k_fwht_rows(const float *x, int8_t *__res
     }
 }
 
+// Short rows (K <= 2048): one wave per row, four rows per workgroup; lane l owns chunks l, l + 64, ...
+// The absmax never leaves the wave, so there is no LDS and no barrier.
+template <int BLOCK, int C, bool QUANT>
+__global__ __launch_bounds__(256) void k_fwht_wave(const float *x, int8_t *__restrict__ q, float *__restrict__ scale,
+                                                   float *xrot, int K, int64_t M)
+{
+    constexpr int LPB = BLOCK / 8;
+    const int lane = threadIdx.x & 63;
+    const int j = lane % LPB;
+    const int nchunk = K / 8;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const float *xr = x + row * (int64_t)K;
+    float v[C][8];
+    int base[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int c = lane + i * 64;
+        base[i] = (c / LPB) * BLOCK + 4 * j;
+        if (c < nchunk) {
+            const float4 lo = *reinterpret_cast<const float4 *>(xr + base[i]);
+            const float4 hi = *reinterpret_cast<const float4 *>(xr + base[i] + BLOCK / 2);
+            v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+            v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        fwht_chunk<BLOCK>(v[i], j);
+        amax = fmaxf(amax, abs8(v[i]));
+    }
+    if constexpr (!QUANT) {
+        float *orow = xrot + row * (int64_t)K;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (lane + i * 64 < nchunk) {
+                *reinterpret_cast<float4 *>(orow + base[i]) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+                *reinterpret_cast<float4 *>(orow + base[i] + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        const float sc = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+        const float inv = (amax == 0.0f) ? 0.0f : 127.0f / amax;
+        if (lane == 0) scale[row] = sc;
+        int8_t *qrow = q + row * (int64_t)K;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (lane + i * 64 < nchunk) {
+                *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                *reinterpret_cast<uint32_t *>(qrow + base[i] + BLOCK / 2) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+            }
+        }
+    }
+}
+
 // K == BLOCK (a row is one Hadamard block, e.g. attention heads and KV-cache
 // rows): BLOCK/8 lanes per row, 256*8/BLOCK rows per workgroup, the absmax is
 // reduced inside the lane group only.
@@ -218,6 +279,18 @@ static int32_t launch_rows(const float *x, int8_t *q, float *scale, float *xrot,
         return launch_status();
     }
     const int nchunk = (int)(K / 8);
+    if (nchunk <= 256 && M >= 1024) {
+        // many short rows: a wave per row
+        const dim3 grid((unsigned)((M + 3) / 4));
+        const int CW = (nchunk + 63) / 64;
+#define MI_WAVE_CASE(CC)                                                                                    \
+    hipLaunchKernelGGL((k_fwht_wave<BLOCK, CC, QUANT>), grid, dim3(256), 0, s, x, q, scale, xrot, (int)K, M)
+        if (CW <= 1) MI_WAVE_CASE(1);
+        else if (CW <= 2) MI_WAVE_CASE(2);
+        else MI_WAVE_CASE(4);
+#undef MI_WAVE_CASE
+        return launch_status();
+    }
     int T = nchunk >= 256 ? 256 : ((nchunk + 63) / 64) * 64;
     const int C = (nchunk + T - 1) / T;
     const dim3 grid((unsigned)M), blk((unsigned)T);

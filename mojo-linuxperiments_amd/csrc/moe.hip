@@ -388,11 +388,12 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
 // The same contraction with the activation fragments held in registers (possible when a wave's K slice is at
 // most NSMAX steps of 128 bytes): only weights travel through the ring, twice as many of them are in flight
 // for the same LDS, and a workgroup walks several row chunks against one set of activation registers.
-constexpr int RX_RING = 3;
+constexpr int RX_RING = 4;
 constexpr int RX_STAGE = 2 * NGRP * 1024;
 constexpr int RX_RING_BYTES = 4 * RX_RING * RX_STAGE;
 constexpr int RX_MT = 3;   // most 16-token fragments per pass
-constexpr int RX_LDS = RX_RING_BYTES + 4 * NGRP * RX_MT * 4 * 64 * 4 + 16 * RX_MT * 8 + 8 * 128 * 4;   // + metadata + scales of <= 8 chunks
+constexpr int RX_RED_BYTES = NGRP * RX_MT * 4 * 64 * 4;
+constexpr int RX_LDS = RX_RING_BYTES + RX_RED_BYTES + 16 * RX_MT * 8 + 8 * 128 * 4;   // + metadata + scales of <= 8 chunks
 
 template <bool DOWN, int NSMAX, int MTT>
 __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ act,
@@ -417,10 +418,10 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     constexpr int CHUNK_ROWS = DOWN ? 128 : 16;
     const int n0 = DOWN ? blockIdx.x * nch * 128 + wave * 32 : blockIdx.x * nch * 16;
     char *ring = smem + wave * (RX_RING * RX_STAGE);
-    int *s_part = reinterpret_cast<int *>(smem + RX_RING_BYTES);   // [4 waves][NGRP][MTT][4][64]
+    int *s_red = reinterpret_cast<int *>(smem + RX_RING_BYTES);    // [NGRP][MTT][4][64] sums over the four K slices (gate/up)
     // per-pass token metadata and per-chunk weight scales sit in LDS so that the epilogue of a chunk issues no
     // dependent global loads (each would cost a memory round trip per chunk)
-    int *s_dst = reinterpret_cast<int *>(smem + RX_RING_BYTES + 4 * NGRP * MTT * 4 * 64 * 4);   // [16*MTT] output row
+    int *s_dst = reinterpret_cast<int *>(smem + RX_RING_BYTES + RX_RED_BYTES);                  // [16*MTT] output row
     float *s_tsc = reinterpret_cast<float *>(s_dst + 16 * MTT);                                  // [16*MTT] token scale
     float *s_wsc = s_tsc + 16 * MTT;                                                             // [nch][SCW]
     constexpr int SCW = DOWN ? 128 : 32;
@@ -435,6 +436,9 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
             if (n < Nrows) v = (nl < 16 ? sc0 : sc1)[(int64_t)e * Nrows + n];
         }
         s_wsc[o] = v;
+    }
+    if constexpr (!DOWN) {
+        for (int o = tid; o < NGRP * MTT * 256; o += 256) s_red[o] = 0;
     }
 
     // load side: lane l = 8*rho + c fetches chunk c ^ sigma(rho, block parity) of row rho of the block
@@ -505,6 +509,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
             }
         }
 
+        __syncthreads();   // token metadata, weight scales and the zeroed sums are visible to every wave
         int slot = 0, f = 0;
         for (int ch = 0; ch < nch; ++ch) {
         const int nc0 = n0 + ch * CHUNK_ROWS;
@@ -536,48 +541,54 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
                 ++f;
             }
         }
-        __syncthreads();   // the previous chunk's epilogue has finished reading s_part
-#pragma unroll
-        for (int a = 0; a < NGRP; ++a)
-#pragma unroll
-            for (int b = 0; b < MTT; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) s_part[(((wave * NGRP + a) * MTT + b) * 4 + q) * 64 + lane] = acc[a][b][q];
-        __syncthreads();
-        // accumulator layout: lane l, register q  <->  weight row 4*(l/16)+q, token l%16
-        auto total = [&](int a, int row, int nn) {
-            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
-            int sum = 0;
-#pragma unroll
-            for (int wv = 0; wv < 4; ++wv) sum += s_part[(((wv * NGRP + a) * MTT + b) * 4 + q) * 64 + src];
-            return sum;
-        };
-        auto own = [&](int wv, int a, int row, int nn) {   // down: one wave's accumulator is already the total
-            const int b = row >> 4, src = (nn >> 2) * 16 + (row & 15), q = nn & 3;
-            return s_part[(((wv * NGRP + a) * MTT + b) * 4 + q) * 64 + src];
-        };
         const float *wsc = s_wsc + ch * SCW;
+        // accumulator layout: lane l, register q  <->  weight row 4*(l/16)+q, token l%16
         if constexpr (!DOWN) {
-            // 32 tokens x 16 channels, channel fastest; h = silu(g) * u in sorted-pair order
+            // the four K slices meet in LDS by integer atomic adds (exact, order-free); whoever reads a sum puts
+            // the zero back for the next chunk
+#pragma unroll
+            for (int a = 0; a < NGRP; ++a)
+#pragma unroll
+                for (int b = 0; b < MTT; ++b)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) atomicAdd(&s_red[((a * MTT + b) * 4 + q) * 64 + lane], acc[a][b][q]);
+            __syncthreads();
+            // 16*MTT tokens x 16 channels, channel fastest; h = silu(g) * u in sorted-pair order
 #pragma unroll
             for (int o = tid; o < 16 * MTT * 16; o += 256) {
                 const int nl = o & 15, row = o >> 4;
+                const int bq = (((row >> 4) * 4) + (nl & 3)) * 64 + (nl >> 2) * 16 + (row & 15);
+                const int gi = s_red[bq], ui = s_red[MTT * 256 + bq];
+                s_red[bq] = 0;
+                s_red[MTT * 256 + bq] = 0;
                 if (base + row < count && nc0 + nl < Nrows) {
                     const float sxt = s_tsc[row];
-                    const float gv = ((float)total(0, row, nl) * sxt) * wsc[nl];
-                    const float uv = ((float)total(1, row, nl) * sxt) * wsc[16 + nl];
+                    const float gv = ((float)gi * sxt) * wsc[nl];
+                    const float uv = ((float)ui * sxt) * wsc[16 + nl];
                     out[(int64_t)s_dst[row] * Nrows + nc0 + nl] = (gv / (1.0f + expf(-gv))) * uv;
                 }
             }
+            __syncthreads();   // the zeroes are in place before the next chunk's sums arrive
         } else {
-            // 32 tokens x 128 channels (32 per wave); out[pair] in pair order, channel fastest
+            // every wave owns its 32 rows over the whole of K: results leave straight from the accumulators, four
+            // consecutive channels of one token per lane; out[pair] in pair order
             const int nbase = (blockIdx.x * nch + ch) * 128;
 #pragma unroll
-            for (int o = tid; o < 16 * MTT * 128; o += 256) {
-                const int nl = o & 127, row = o >> 7;
-                if (base + row < count && nbase + nl < Nrows) {
-                    const int sum = own(nl >> 5, (nl >> 4) & 1, row, nl & 15);
-                    out[(int64_t)s_dst[row] * Hout + nbase + nl] = ((float)sum * s_tsc[row]) * wsc[nl];
+            for (int a = 0; a < NGRP; ++a) {
+                const int nl = wave * 32 + a * 16 + 4 * g_;
+                const float4 ws = *reinterpret_cast<const float4 *>(wsc + nl);
+#pragma unroll
+                for (int b = 0; b < MTT; ++b) {
+                    const int row = b * 16 + r;
+                    if (base + row < count && nbase + nl < Nrows) {
+                        const float ts = s_tsc[row];
+                        float4 o;
+                        o.x = ((float)acc[a][b][0] * ts) * ws.x;
+                        o.y = ((float)acc[a][b][1] * ts) * ws.y;
+                        o.z = ((float)acc[a][b][2] * ts) * ws.z;
+                        o.w = ((float)acc[a][b][3] * ts) * ws.w;
+                        *reinterpret_cast<float4 *>(out + (int64_t)s_dst[row] * Hout + nbase + nl) = o;
+                    }
                 }
             }
         }

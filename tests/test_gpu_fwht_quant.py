@@ -25,6 +25,9 @@ def run_quant(mi, dev, x, block):
     (1, 4096, 128),
     (5, 2048, 128),       # MoE hidden
     (37, 768, 256),       # MoE inner dim, 3 blocks of 256
+    (1501, 768, 256),     # many short rows: the wave-per-row kernel (ragged last workgroup)
+    (1024, 2048, 128),    # wave-per-row, four chunks per lane
+    (1030, 256, 256),     # wave-per-row, half of the lanes idle
     (64, 128, 128),       # attention heads / KV rows: one block per row
     (1000, 128, 128),     # ragged count of small rows
     (9, 256, 256),
@@ -60,7 +63,7 @@ def test_zero_rows_ties_and_extremes(mi, dev, orc):
     assert np.array_equal(s, so) and np.array_equal(q, qo)
 
 
-@pytest.mark.parametrize("M,K,block", [(7, 4096, 128), (3, 768, 256), (33, 128, 128)])
+@pytest.mark.parametrize("M,K,block", [(7, 4096, 128), (3, 768, 256), (33, 128, 128), (1027, 512, 256)])
 def test_rotation_only_bit_exact_and_in_place(mi, dev, orc, M, K, block):
     x = workload.normal(3, (M, K))
     mark = dev.mark()
