@@ -172,7 +172,9 @@ def main():
     roofline = {
         "kernel": "k_w8a8_tiled (v_mfma_i32_16x16x64_i8), four cfg3 shapes, ops-weighted",
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-        "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": None,
+        "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_total,
+        "traffic_unit": "bytes over the four launches (fetched + written), rocprofv3 PMC, calibrated",
+        "traffic_per_shape": traffic,
         "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
         "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
                            for name, K, N in wl.PROJECTIONS},
