@@ -425,17 +425,24 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     float *s_tsc = reinterpret_cast<float *>(s_dst + 16 * MTT);                                  // [16*MTT] token scale
     float *s_wsc = s_tsc + 16 * MTT;                                                             // [nch][SCW]
     constexpr int SCW = DOWN ? 128 : 32;
-    for (int o = tid; o < nch * SCW; o += 256) {
+    // weight scales of every chunk: requested here, parked in LDS only after the weight stream and the
+    // activation loads have been issued, so that the whole set-up costs one memory round trip
+    float wsv[4];   // nch * SCW <= 8 * 128 = 4 values per thread
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int o = tid + u * 256;
         const int ch = o / SCW, nl = o - ch * SCW;
         float v = 0.0f;
-        if constexpr (DOWN) {
-            const int n = (blockIdx.x * nch + ch) * 128 + nl;
-            if (n < Nrows) v = sc0[(int64_t)e * Nrows + n];
-        } else {
-            const int n = (blockIdx.x * nch + ch) * 16 + (nl & 15);
-            if (n < Nrows) v = (nl < 16 ? sc0 : sc1)[(int64_t)e * Nrows + n];
+        if (o < nch * SCW) {
+            if constexpr (DOWN) {
+                const int n = (blockIdx.x * nch + ch) * 128 + nl;
+                if (n < Nrows) v = sc0[(int64_t)e * Nrows + n];
+            } else {
+                const int n = (blockIdx.x * nch + ch) * 16 + (nl & 15);
+                if (n < Nrows) v = (nl < 16 ? sc0 : sc1)[(int64_t)e * Nrows + n];
+            }
         }
-        s_wsc[o] = v;
+        wsv[u] = v;
     }
     if constexpr (!DOWN) {
         for (int o = tid; o < NGRP * MTT * 256; o += 256) s_red[o] = 0;
@@ -483,11 +490,11 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
         // stored.
         v4i xr[MTT][NSMAX][2];
         __syncthreads();   // the previous pass has finished with the token metadata and every ring is idle
+        int m_dst = 0, m_pr = 0;
         if (tid < 16 * MTT && base + tid < count) {
             const int pos = seg0 + base + tid;
-            const int pr = perm[pos];
-            s_dst[tid] = DOWN ? pr : pos;
-            s_tsc[tid] = act_scale[DOWN ? pos : pr / topk];
+            m_pr = perm[pos];
+            m_dst = DOWN ? m_pr : pos;
         }
         {
             // the weight stream starts first: its addresses do not depend on the tokens, whose lookups cost two
@@ -509,6 +516,15 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
             }
         }
 
+        if (tid < 16 * MTT && base + tid < count) {
+            s_dst[tid] = m_dst;
+            s_tsc[tid] = act_scale[DOWN ? seg0 + base + tid : m_pr / topk];
+        }
+        if (base == 0) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (tid + u * 256 < nch * SCW) s_wsc[tid + u * 256] = wsv[u];
+        }
         __syncthreads();   // token metadata, weight scales and the zeroed sums are visible to every wave
         int slot = 0, f = 0;
         for (int ch = 0; ch < nch; ++ch) {
