@@ -249,7 +249,7 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
         const int rho = lane >> 3, c = lane & 7;
 #pragma unroll
         for (int b = 0; b < BLK; ++b) {
-            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            const int sigma = ((b & 1) << 2) | (rho >> 1);
             const int8_t *base;
             if (b < 2 * NG) {
                 int rowi = n0 + b * 8 + rho;
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
     int roff[2];
     {
         const int rho = r & 7, bpar = r >> 3;
-        const int sigma = (rho & 6) | ((rho ^ bpar) & 1);
+        const int sigma = (bpar << 2) | (rho >> 1);
         roff[0] = bpar * 1024 + ((8 * rho + ((0 + g_) ^ sigma)) << 4);
         roff[1] = bpar * 1024 + ((8 * rho + ((4 + g_) ^ sigma)) << 4);
     }

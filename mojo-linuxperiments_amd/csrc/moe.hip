@@ -258,7 +258,7 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
     const int8_t *wsrc[2 * NGRP];
 #pragma unroll
     for (int b = 0; b < 2 * NGRP; ++b) {
-        const int sigma = (rho & 6) | ((rho ^ b) & 1);
+        const int sigma = ((b & 1) << 2) | (rho >> 1);
         const int grp = b >> 1;
         int rowi = n0 + (DOWN ? grp * 16 : 0) + (b & 1) * 8 + rho;
         if (rowi > Nrows - 1) rowi = Nrows - 1;
@@ -273,7 +273,7 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
     int roff[2];
     {
         const int rr = r & 7, bpar = r >> 3;
-        const int sigma = (rr & 6) | ((rr ^ bpar) & 1);
+        const int sigma = (bpar << 2) | (rr >> 1);
         roff[0] = bpar * 1024 + ((8 * rr + ((0 + g_) ^ sigma)) << 4);
         roff[1] = bpar * 1024 + ((8 * rr + ((4 + g_) ^ sigma)) << 4);
     }
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
         const int8_t *xsrc[2 * MT];
 #pragma unroll
         for (int b = 0; b < 2 * MT; ++b) {
-            const int sigma = (rho & 6) | ((rho ^ b) & 1);
+            const int sigma = ((b & 1) << 2) | (rho >> 1);
             const int pos = seg0 + min(base + b * 8 + rho, count - 1);
             const int64_t arow = DOWN ? (int64_t)pos : (int64_t)(perm[pos] / topk);
             xsrc[b] = act + arow * Kdim + ((c8 ^ sigma) << 4);
@@ -453,7 +453,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     const int8_t *wsrc[2 * NGRP];
 #pragma unroll
     for (int b = 0; b < 2 * NGRP; ++b) {
-        const int sigma = (rho & 6) | ((rho ^ b) & 1);
+        const int sigma = ((b & 1) << 2) | (rho >> 1);
         const int grp = b >> 1;
         int rowi = n0 + (DOWN ? grp * 16 : 0) + (b & 1) * 8 + rho;
         if (rowi > Nrows - 1) rowi = Nrows - 1;
@@ -468,7 +468,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     int roff[2];
     {
         const int rr = r & 7, bpar = r >> 3;
-        const int sigma = (rr & 6) | ((rr ^ bpar) & 1);
+        const int sigma = (bpar << 2) | (rr >> 1);
         roff[0] = bpar * 1024 + ((8 * rr + ((0 + g_) ^ sigma)) << 4);
         roff[1] = bpar * 1024 + ((8 * rr + ((4 + g_) ^ sigma)) << 4);
     }
