@@ -10,6 +10,9 @@ template <bool DEQ>
 int32_t launch_tiled(const int8_t *, const float *, const int8_t *, const float *, int32_t *, float *, int64_t,
                      int64_t, int64_t, hipStream_t);
 
+int32_t launch_linear_fused(const float *, const int8_t *, const float *, float *, int8_t *, float *, int64_t, int64_t,
+                            int64_t, hipStream_t);
+
 __global__ void k_dequant(const int32_t *__restrict__ acc, const float *__restrict__ sx,
                           const float *__restrict__ sw, float *__restrict__ y, int64_t M, int64_t N)
 {
@@ -93,6 +96,11 @@ extern "C" int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const fl
     int32_t rc = check_gemm(qx, qw, y, M, N, K);
     if (rc) return rc;
     if (!x || !sw || !aligned16(sw)) return MI_EINVAL;
+    if (M == 1 && block == 128 && aligned16(x)) {
+        // decode: one kernel that quantizes its own activations (MI_EINVAL = shape not covered)
+        rc = launch_linear_fused(x, qw, sw, y, qx, sx, M, N, K, as_stream(stream));
+        if (rc != MI_EINVAL) return rc;
+    }
     rc = mi_fwht_quant_f32_i8(x, qx, sx, M, K, block, stream);
     if (rc) return rc;
     return gemm_dispatch(qx, sx, qw, sw, nullptr, y, M, N, K, as_stream(stream));

@@ -25,6 +25,7 @@
 //  flight per wave.  Waves of a workgroup split K; their partial accumulators
 //  meet in LDS at the end.
 #include "common.h"
+#include "fwht_core.h"
 
 namespace mi {
 
@@ -144,6 +145,173 @@ __global__ __launch_bounds__(256) void k_gemv_reg(const int8_t *__restrict__ qx,
             else acc_out[(int64_t)m * N + n] = total;
         }
     }
+}
+
+// k_gemv_fused: k_gemv_reg with the rotate + quantize prologue inside.  The weight loads of every wave
+// go out first; while they are in flight the workgroup rotates and quantizes the M activation rows (the same
+// per-chunk code as the stand-alone quantizer, so the codes and scales are bit-identical), parks the codes in
+// LDS and every lane picks up its share.  One launch per linear instead of two.
+template <int MB, int CW, int CQ>
+__global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x, const int8_t *__restrict__ qw,
+                                                    const float *__restrict__ sw, float *__restrict__ y,
+                                                    int8_t *__restrict__ qx_out, float *__restrict__ sx_out, int M,
+                                                    int N, int K, int QW)
+{
+    constexpr int BLOCK = 128, LPB = BLOCK / 8;
+    constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);   // rows per wave
+    constexpr int V = pow2_ceil(R * MB);
+    extern __shared__ __attribute__((aligned(16))) char s_dyn[];
+    int8_t *s_x = reinterpret_cast<int8_t *>(s_dyn);                       // [MB][K] codes
+    float *s_scale = reinterpret_cast<float *>(s_dyn + (size_t)MB * K);    // [MB]
+    float *s_max = s_scale + MB;                                           // [4]
+    int *s_red = reinterpret_cast<int *>(s_max + 4);                       // [4][V]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = wave % QW;                  // which CW-chunk slice of the row
+    const int rows_per_wg = (4 / QW) * R;
+    const int row0 = blockIdx.x * rows_per_wg + (wave / QW) * R;
+    const int kbase = q * CW * 1024 + lane * 16;
+
+    v4i w[R][CW];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int c = 0; c < CW; ++c) {
+            const int off = kbase + c * 1024;
+            w[r][c] = (row0 + r < N && off < K) ? *reinterpret_cast<const v4i *>(qw + (int64_t)(row0 + r) * K + off)
+                                                : (v4i){0, 0, 0, 0};
+        }
+
+    // rotate + quantize, one row at a time: thread t owns chunks t, t + 256, ... of the row
+    const int j = tid % LPB;
+    const int nchunk = K / 8;
+    for (int m = 0; m < MB && m < M; ++m) {
+        const float *xr = x + (int64_t)m * K;
+        float v[CQ][8];
+        int base[CQ];
+#pragma unroll
+        for (int i = 0; i < CQ; ++i) {
+            const int c = tid + i * 256;
+            base[i] = (c / LPB) * BLOCK + 4 * j;
+            if (c < nchunk) {
+                const float4 lo = *reinterpret_cast<const float4 *>(xr + base[i]);
+                const float4 hi = *reinterpret_cast<const float4 *>(xr + base[i] + BLOCK / 2);
+                v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+                v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+            }
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < CQ; ++i) {
+            fwht_chunk<BLOCK>(v[i], j);
+            amax = fmaxf(amax, abs8(v[i]));
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        __syncthreads();   // the previous row's maxima have been read
+        if (lane == 0) s_max[wave] = amax;
+        __syncthreads();
+        const float a = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+        const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+        const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+        if (tid == 0) s_scale[m] = sc;
+        int8_t *qrow = s_x + (size_t)m * K;
+        const bool keeper = blockIdx.x == 0;   // one workgroup also leaves the codes and scales in the caller's workspace
+        if (keeper && tid == 0) sx_out[m] = sc;
+#pragma unroll
+        for (int i = 0; i < CQ; ++i) {
+            if (tid + i * 256 < nchunk) {
+                const uint32_t c0 = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                const uint32_t c1 = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+                *reinterpret_cast<uint32_t *>(qrow + base[i]) = c0;
+                *reinterpret_cast<uint32_t *>(qrow + base[i] + BLOCK / 2) = c1;
+                if (keeper) {
+                    *reinterpret_cast<uint32_t *>(qx_out + (int64_t)m * K + base[i]) = c0;
+                    *reinterpret_cast<uint32_t *>(qx_out + (int64_t)m * K + base[i] + BLOCK / 2) = c1;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    v4i xr[MB][CW];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < CW; ++c) {
+            const int off = kbase + c * 1024;
+            const int ms = m < M ? m : M - 1;
+            xr[m][c] = off < K ? *reinterpret_cast<const v4i *>(s_x + (size_t)ms * K + off) : (v4i){0, 0, 0, 0};
+        }
+    int p[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) p[i] = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            int a = 0;
+#pragma unroll
+            for (int c = 0; c < CW; ++c) {
+                a = __builtin_amdgcn_sdot4(w[r][c][0], xr[m][c][0], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][1], xr[m][c][1], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][2], xr[m][c][2], a, false);
+                a = __builtin_amdgcn_sdot4(w[r][c][3], xr[m][c][3], a, false);
+            }
+            p[r * MB + m] = a;
+        }
+    fold_sum<V, 32>(p, lane);
+    constexpr int SH = 6 - __builtin_ctz(V);
+    const int vi = lane >> SH;
+    const bool speaker = (lane & ((1 << SH) - 1)) == 0;
+    int total = p[0];
+    if (QW > 1) {
+        if (speaker) s_red[wave * V + vi] = total;
+        __syncthreads();
+        if (q == 0 && speaker) {
+            for (int o = 1; o < QW; ++o) total += s_red[(wave + o) * V + vi];
+        }
+    }
+    if (q == 0 && speaker && vi < R * MB) {
+        const int r = vi / MB, m = vi % MB, n = row0 + r;
+        if (n < N && m < M) y[(int64_t)m * N + n] = ((float)total * s_scale[m]) * sw[n];
+    }
+}
+
+template <int MB, int CW, int CQ>
+static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx, int M,
+                            int N, int K, int QW, hipStream_t s)
+{
+    constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);
+    constexpr int V = pow2_ceil(R * MB);
+    const size_t lds = (size_t)MB * K + (MB + 4) * sizeof(float) + 4 * V * sizeof(int);
+    static bool attr_set = false;  // idempotent; a race only repeats the call
+    if (!attr_set) {
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+        attr_set = true;
+    }
+    const int rows_per_wg = (4 / QW) * R;
+    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL((k_gemv_fused<MB, CW, CQ>), dim3(grid), dim3(256), lds, s, x, qw, sw, y, qx, sx, M, N, K, QW);
+    return launch_status();
+}
+
+// The fused decode linear is taken for one token and K <= 4096 only (MI_EINVAL tells the caller to take the
+// two-kernel path).  Measured: 9.3 against 10.6 us for 4096 -> 6144 at M = 1, but every workgroup repeats the
+// quantization, which at M = 4 or K = 14336 costs more than the launch it saves (15.6 against 11.7 us, 20.8
+// against 18.8 us).
+int32_t launch_linear_fused(const float *x, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx,
+                            int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
+{
+    const int M = (int)M64, N = (int)N64, K = (int)K64;
+    if (M != 1 || K % 1024) return MI_EINVAL;
+    const int nchunk = K >> 10;
+    if (nchunk == 4) return launch_fused<1, 4, 2>(x, qw, sw, y, qx, sx, M, N, K, 1, s);   // K = 4096
+    if (nchunk == 2) return launch_fused<1, 2, 1>(x, qw, sw, y, qx, sx, M, N, K, 1, s);   // K = 2048
+    return MI_EINVAL;
 }
 
 template <int MB, bool DEQ>

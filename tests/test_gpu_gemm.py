@@ -65,7 +65,9 @@ def test_dequant_kernel_matches_closed_form(mi, dev, orc):
     assert np.array_equal(y, orc.dequant(acc, sx, sw))
 
 
-@pytest.mark.parametrize("M,N,K", [(32, 4096, 4096), (1, 512, 4096), (16, 256, 14336), (130, 320, 1024)])
+@pytest.mark.parametrize("M,N,K", [(32, 4096, 4096), (1, 512, 4096), (16, 256, 14336), (130, 320, 1024),
+                                   # one token, K <= 4096: the kernel with the quantizer inside; the rest: two kernels
+                                   (1, 6144, 4096), (1, 272, 2048), (4, 6144, 4096), (2, 1024, 14336), (1, 4096, 14336)])
 def test_whole_linear(mi, dev, orc, M, N, K):
     """cfg0 is the first case: x [32,4096] with outlier channels, W [4096,4096]."""
     x = workload.activations(11, M, K)
