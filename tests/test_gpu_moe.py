@@ -135,7 +135,10 @@ def check_ffn_against_oracle(orc, x, idx, w, experts, r):
     return rel
 
 
-@pytest.mark.parametrize("T,H,I,E,topk", [(24, 256, 256, 16, 2), (70, 512, 768, 64, 8), (9, 2048, 256, 16, 1)])
+@pytest.mark.parametrize("T,H,I,E,topk", [(24, 256, 256, 16, 2), (70, 512, 768, 64, 8), (9, 2048, 256, 16, 1),
+                                          # hidden and inner sizes past what a wave keeps in registers: the kernels that stream
+                                          # the activation rows through the ring as well
+                                          (6, 4352, 1280, 16, 2)])
 def test_ffn_stagewise(mi, dev, orc, T, H, I, E, topk):
     mark = dev.mark()
     x = workload.activations(51, T, H)
