@@ -26,6 +26,7 @@ def gpu_gemm_i32(mi, dev, qx, qw):
 @pytest.mark.parametrize("M,N,K", [
     (1, 64, 128), (1, 6144, 4096), (4, 4096, 14336), (16, 256, 4096), (13, 48, 1024),
     (17, 64, 768), (32, 4096, 4096), (33, 128, 2048), (48, 160, 256), (64, 512, 1408),
+    (2, 96, 9216), (3, 80, 11264),    # K that the register-resident GEMV cannot split: the LDS-staged one
 ])
 def test_skinny_accumulators_bit_exact(mi, dev, orc, M, N, K):
     qx, qw = rand_codes(M * 7 + N, (M, K)), rand_codes(K + 1, (N, K))
@@ -35,6 +36,7 @@ def test_skinny_accumulators_bit_exact(mi, dev, orc, M, N, K):
 @pytest.mark.parametrize("M,N,K", [
     (65, 256, 128), (128, 128, 256), (256, 256, 1024), (200, 192, 512), (257, 272, 384),
     (512, 448, 768), (300, 1000 // 16 * 16, 640), (2048, 224 * 3, 512), (1024, 6144, 256),
+    (4096, 4096, 256),                # the 256 x 256 tile
 ])
 def test_tiled_accumulators_bit_exact(mi, dev, orc, M, N, K):
     qx, qw = rand_codes(M + 3 * N, (M, K)), rand_codes(K + 5, (N, K))
