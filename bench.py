@@ -220,6 +220,7 @@ def main():
         sub.update(decode_attention(mi, wl, dev, s, timer))
         sub.update(moe_layer(mi, wl, dev, s, timer))
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
+        sub.update(host_staging(mi, wl, dev, s, timer))
     out["sub_metrics"] = sub
     if not args.skip_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)
@@ -398,6 +399,26 @@ def cfg0_linear(mi, wl, dev, s, timer, shapes):
     return {"cfg0_linear_m32": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                 "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                 "TOPS": round(wl.gemm_ops(M, N, K) / (ms * 1e-3) / 1e12, 2)}}
+
+
+def host_staging(mi, wl, dev, s, timer):
+    """The host-buffer variant of the boundary for the cfg3 QKV linear: activations fp32 [2048,4096] in from a
+    pinned staging slab and the fp32 [2048,6144] result back out, over the host link.  Never part of `value`."""
+    import ctypes as C
+    lib = mi.lib
+    M, K, N = wl.PREFILL_M, 4096, 6144
+    nin, nout = 4 * M * K, 4 * M * N
+    h = C.c_void_p()
+    mi.check(lib.mi_host_arena_create(dev.ctx, nin + nout + 4096, 256, 0, C.byref(h)), "mi_host_arena_create")
+    hin, hout = lib.mi_arena_alloc(h, nin), lib.mi_arena_alloc(h, nout)
+    mark = dev.mark()
+    din, dout = dev.empty((M, K), np.float32), dev.empty((M, N), np.float32)
+    ms_in = timer.run(lambda: mi.check(lib.mi_memcpy_h2d(din.ptr, hin, nin, s)), 10)
+    ms_out = timer.run(lambda: mi.check(lib.mi_memcpy_d2h(hout, dout.ptr, nout, s)), 10)
+    dev.reset_to(mark)
+    mi.check(lib.mi_arena_destroy(h))
+    return {"host_staging_cfg3_qkv": {"h2d_us": round(ms_in * 1e3, 1), "h2d_GBps": round(nin / (ms_in * 1e-3) / 1e9, 1),
+                                      "d2h_us": round(ms_out * 1e3, 1), "d2h_GBps": round(nout / (ms_out * 1e-3) / 1e9, 1)}}
 
 
 def cpu_baseline(wl):

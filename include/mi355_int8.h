@@ -76,7 +76,12 @@ MI_API int32_t mi_arena_reset_to(mi_arena *a, int64_t mark);   /* numa_arena.moj
 MI_API int32_t mi_arena_reset(mi_arena *a);                    /* numa_arena.mojo:68-70 */
 MI_API int64_t mi_arena_remaining(const mi_arena *a);          /* numa_arena.mojo:72-74 */
 MI_API int64_t mi_arena_used(const mi_arena *a);               /* numa_arena.mojo:76-78 */
-MI_API int32_t mi_arena_verify_placement(const mi_arena *a);   /* numa_arena.mojo:80-87; 1 = slab lives on the context's device */
+MI_API int32_t mi_arena_verify_placement(const mi_arena *a);   /* numa_arena.mojo:80-87; 1 = slab lives on the context's device (host slab: pinned host memory, on its node where the kernel can tell) */
+/* Pinned host staging slab bound to one NUMA node (numa_node = -1: no binding), the host-side half of the
+ * same allocator: mmap_numa + mbind(MPOL_BIND) (numa_arena.mojo:93-107), here as a memory policy held while
+ * the runtime allocates the pinned pages.  Every mi_arena_* call above works on it; copies from it to the
+ * device run at the full rate of the link (mi_memcpy_h2d is asynchronous only from pinned memory). */
+MI_API int32_t mi_host_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t alignment, int32_t numa_node, mi_arena **out);
 
 /* ---- stream pool and gate ------------------------------------------------
  * Replaces ThreadPool (threading/linux_threading.mojo:43-158) on this path:

@@ -5,6 +5,8 @@
 // memory, hipStreams and hipEvents in place of mmap/mbind, clone3 and futexes.
 #include <sched.h>
 #include <string.h>
+#include <sys/syscall.h>
+#include <unistd.h>
 
 #include <new>
 
@@ -49,6 +51,8 @@ struct mi_arena {
     int64_t size;
     int64_t offset;
     int64_t alignment;
+    bool host;      // pinned host slab (staging) instead of device memory
+    int32_t node;   // NUMA node a host slab is bound to, or -1
 };
 
 struct mi_slot {
@@ -169,6 +173,48 @@ int32_t mi_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t alignment, mi_a
     a->size = size_bytes;
     a->offset = 0;
     a->alignment = alignment;
+    a->host = false;
+    a->node = -1;
+    *out = a;
+    return MI_OK;
+}
+
+// Pinned host slab for staging, bound to one NUMA node the way mmap_numa binds its mapping
+// (threading/numa_arena.mojo:93-107): the calling thread's memory policy is MPOL_BIND to `numa_node` while the
+// runtime allocates and the pages are touched, and is put back afterwards.  The runtime pins the pages itself
+// (pinning memory that already exists is not available on every host, allocating pinned memory is).
+int32_t mi_host_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t alignment, int32_t numa_node, mi_arena **out)
+{
+    if (!out) return MI_EINVAL;
+    *out = nullptr;
+    if (!ctx || size_bytes <= 0 || alignment <= 0 || (alignment & (alignment - 1))) return MI_EINVAL;
+    if (numa_node < -1 || numa_node >= 64) return MI_EINVAL;
+    MI_HIP(hipSetDevice(ctx->device));
+    mi_arena *a = new (std::nothrow) mi_arena;
+    if (!a) return MI_ENOMEM;
+    constexpr int MPOL_DEFAULT_ = 0, MPOL_BIND_ = 2;
+    bool bound = false;
+    if (numa_node >= 0) {
+        unsigned long mask = 1UL << numa_node;
+        if (syscall(SYS_set_mempolicy, MPOL_BIND_, &mask, 65UL) != 0) { delete a; return MI_EINVAL; }
+        bound = true;
+    }
+    void *p = nullptr;
+    hipError_t e = hipHostMalloc(&p, (size_t)size_bytes, bound ? hipHostMallocNumaUser : hipHostMallocDefault);
+    if (e == hipSuccess && p) memset(p, 0, (size_t)size_bytes);   // first touch under the policy; fresh pages read as zero
+    if (bound) (void)syscall(SYS_set_mempolicy, MPOL_DEFAULT_, nullptr, 0UL);
+    if (e != hipSuccess || !p) {
+        (void)hipGetLastError();
+        delete a;
+        return MI_ENOMEM;
+    }
+    a->ctx = ctx;
+    a->base = (uint8_t *)p;
+    a->size = size_bytes;
+    a->offset = 0;
+    a->alignment = alignment;
+    a->host = true;
+    a->node = numa_node;
     *out = a;
     return MI_OK;
 }
@@ -176,7 +222,7 @@ int32_t mi_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t alignment, mi_a
 int32_t mi_arena_destroy(mi_arena *a)
 {
     if (!a) return MI_EINVAL;
-    hipError_t e = hipFree(a->base);
+    hipError_t e = a->host ? hipHostFree(a->base) : hipFree(a->base);
     delete a;
     return e == hipSuccess ? MI_OK : hip_fail(e);
 }
@@ -214,6 +260,19 @@ int32_t mi_arena_verify_placement(const mi_arena *a)
 {
     if (!a) return MI_EINVAL;
     if (a->offset == 0) return 1;
+    if (a->host) {
+        // numa_arena.mojo:80-87: ask the kernel which node holds the first page (move_pages with no target nodes).
+        // Pinned pages are mapped by the GPU driver and the kernel's page query may not see them (status
+        // -ENOENT): then what can be verified is that the slab is pinned host memory; its node is the policy
+        // that was in force while it was allocated.
+        void *page = a->base;
+        int status = -1;
+        if (syscall(SYS_move_pages, 0, 1UL, &page, nullptr, &status, 0) == 0 && status >= 0)
+            return (a->node < 0 || status == a->node) ? 1 : 0;
+        hipPointerAttribute_t hattr;
+        MI_HIP(hipPointerGetAttributes(&hattr, a->base));
+        return hattr.type == hipMemoryTypeHost ? 1 : 0;
+    }
     hipPointerAttribute_t attr;
     MI_HIP(hipPointerGetAttributes(&attr, a->base));
     return (attr.type == hipMemoryTypeDevice && attr.device == a->ctx->device) ? 1 : 0;

@@ -62,6 +62,36 @@ private:
     int64_t size_ = 0;
 };
 
+// Pinned host staging slab on one NUMA node: NumaArena as it is (numa_arena.mojo:5-87), with pages the
+// device can copy from at link rate.
+template <int64_t Alignment = 256>
+class HostArena {
+public:
+    HostArena(const Context &ctx, int node, int64_t size) : node_(node)
+    {
+        if (!ctx || mi_host_arena_create(ctx.handle(), size, Alignment, node, &h_) != MI_OK) h_ = nullptr;
+    }
+    ~HostArena() { if (h_) mi_arena_destroy(h_); }
+    HostArena(HostArena &&o) noexcept : h_(o.h_), node_(o.node_) { o.h_ = nullptr; }
+    HostArena(const HostArena &) = delete;
+    HostArena &operator=(const HostArena &) = delete;
+    explicit operator bool() const { return h_ != nullptr; }
+
+    template <typename T>
+    T *alloc(int64_t count = 1) { return h_ ? static_cast<T *>(mi_arena_alloc(h_, count * (int64_t)sizeof(T))) : nullptr; }
+    int64_t mark() const { return h_ ? mi_arena_mark(h_) : 0; }
+    void reset_to(int64_t watermark) { if (h_) (void)mi_arena_reset_to(h_, watermark); }
+    void reset() { if (h_) (void)mi_arena_reset(h_); }
+    int64_t remaining() const { return h_ ? mi_arena_remaining(h_) : 0; }
+    int64_t used() const { return h_ ? mi_arena_used(h_) : 0; }
+    bool verify_placement() const { return !h_ || mi_arena_verify_placement(h_) == 1; }
+    int node() const { return node_; }
+
+private:
+    mi_arena *h_ = nullptr;
+    int node_ = -1;
+};
+
 // MutexGate (linux_threading.mojo:174-198): trivially copyable token over a handle.
 struct Gate {
     mi_gate *h = nullptr;

@@ -39,6 +39,7 @@ SIGNATURES = {
     "mi_ctx_memory_bytes": (i64, [vp]),
     "mi_ctx_arch_name": (i32, [vp, C.c_char_p, i64]),
     "mi_arena_create": (i32, [vp, i64, i64, C.POINTER(vp)]),
+    "mi_host_arena_create": (i32, [vp, i64, i64, i32, C.POINTER(vp)]),
     "mi_arena_destroy": (i32, [vp]),
     "mi_arena_alloc": (vp, [vp, i64]),
     "mi_arena_mark": (i64, [vp]),

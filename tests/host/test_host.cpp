@@ -77,6 +77,32 @@ static void test_arena(const Context &ctx)
     report("device_arena", ok);
 }
 
+// the pinned staging slab: same watermarks, zero-filled, and a round trip through the device
+static void test_host_arena(const Context &ctx)
+{
+    HostArena<256> stage(ctx, 0, 2 << 20);
+    bool ok = (bool)stage && stage.used() == 0 && stage.node() == 0 && stage.verify_placement();
+    uint32_t *src = stage.alloc<uint32_t>(4096);
+    uint32_t *dst = stage.alloc<uint32_t>(4096);
+    ok = ok && src && dst && src[17] == 0 && stage.verify_placement();
+    ok = ok && stage.alloc<char>(4 << 20) == nullptr;
+    DeviceArena<256> arena(ctx, 1 << 20);
+    uint32_t *d = arena.alloc<uint32_t>(4096);
+    if (ok && d) {
+        for (int i = 0; i < 4096; ++i) src[i] = 0x9e3779b9u * (uint32_t)i;
+        ok = mi_memcpy_h2d(d, src, 4096 * 4, nullptr) == MI_OK && mi_memcpy_d2h(dst, d, 4096 * 4, nullptr) == MI_OK &&
+             mi_stream_synchronize(nullptr) == MI_OK;
+        for (int i = 0; ok && i < 4096; ++i) ok = dst[i] == src[i];
+    }
+    const int64_t w = stage.mark();
+    (void)stage.alloc<double>(100);
+    stage.reset_to(w);
+    ok = ok && stage.used() == w;
+    HostArena<256> moved(std::move(stage));
+    ok = ok && (bool)moved && !(bool)stage;
+    report("host_arena", ok);
+}
+
 static int32_t fill_op(void *stream, uint32_t *dst, uint32_t value, int64_t count)
 {
     return mi_fill_u32(dst, value, count, stream);
@@ -187,6 +213,7 @@ int main()
     report("context", (bool)ctx, ctx ? "CUs " + std::to_string(ctx.compute_units()) : "no gfx950 device");
     if (!ctx) return 1;
     test_arena(ctx);
+    test_host_arena(ctx);
     test_stream_pool(ctx);
     test_quant_linear(ctx);
     test_decode_attention(ctx);

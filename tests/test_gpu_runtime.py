@@ -188,6 +188,52 @@ def test_pinned_host_staging_and_events(mi, ctx):
     mi.check(lib.mi_arena_destroy(a))
 
 
+def test_host_arena_is_the_same_allocator_on_pinned_memory(mi, ctx):
+    """The pinned staging slab answers every arena call like the device slab (numa_arena.mojo:40-87), reads as
+    zero when fresh, sits on the node it was bound to, and feeds asynchronous copies."""
+    lib = mi.lib
+    h = C.c_void_p()
+    mi.check(lib.mi_host_arena_create(ctx, 4 << 20, 256, 0, C.byref(h)))       # bound to NUMA node 0
+    assert lib.mi_arena_used(h) == 0 and lib.mi_arena_remaining(h) == 4 << 20
+    assert lib.mi_arena_verify_placement(h) == 1                               # nothing allocated: true
+    p1 = lib.mi_arena_alloc(h, 1000)
+    p2 = lib.mi_arena_alloc(h, 1 << 20)
+    assert p1 and p2 and p1 % 256 == 0 and p2 - p1 == 1024
+    assert lib.mi_arena_verify_placement(h) == 1                               # pinned, and on node 0 where the kernel can tell
+    fresh = np.frombuffer((C.c_uint8 * (1 << 20)).from_address(p2), np.uint8)
+    assert not fresh.any()
+    mark = lib.mi_arena_mark(h)
+    p3 = lib.mi_arena_alloc(h, 4096)
+    assert lib.mi_arena_reset_to(h, mark + (1 << 30)) == mi.EINVAL
+    assert lib.mi_arena_reset_to(h, mark) == mi.OK
+    assert lib.mi_arena_alloc(h, 4096) == p3
+    assert lib.mi_arena_alloc(h, 8 << 20) is None                              # exhausted: null, no error
+    # host slab -> device -> host slab, all asynchronous on one stream
+    rng = np.random.default_rng(5)
+    fresh[:] = rng.integers(0, 256, 1 << 20, dtype=np.uint8)
+    want = fresh.copy()
+    a = C.c_void_p()
+    mi.check(lib.mi_arena_create(ctx, 2 << 20, 256, C.byref(a)))
+    d = lib.mi_arena_alloc(a, 1 << 20)
+    lib.mi_arena_reset_to(h, mark)
+    back_p = lib.mi_arena_alloc(h, 1 << 20)
+    mi.check(lib.mi_memcpy_h2d(d, p2, 1 << 20, None))
+    mi.check(lib.mi_memcpy_d2h(back_p, d, 1 << 20, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    back = np.frombuffer((C.c_uint8 * (1 << 20)).from_address(back_p), np.uint8)
+    assert np.array_equal(back, want)
+    unbound = C.c_void_p()
+    mi.check(lib.mi_host_arena_create(ctx, 1 << 20, 64, -1, C.byref(unbound)))  # no binding
+    assert lib.mi_arena_alloc(unbound, 64) and lib.mi_arena_verify_placement(unbound) == 1
+    bad = C.c_void_p()
+    assert lib.mi_host_arena_create(ctx, 1 << 20, 48, 0, C.byref(bad)) == mi.EINVAL
+    assert lib.mi_host_arena_create(ctx, 1 << 20, 64, 99, C.byref(bad)) == mi.EINVAL
+    del fresh, back
+    mi.check(lib.mi_arena_destroy(unbound))
+    mi.check(lib.mi_arena_destroy(a))
+    mi.check(lib.mi_arena_destroy(h))
+
+
 def test_graph_replays_match_eager(mi, dev, orc):
     """A captured rotate+quant -> GEMM -> dequant chain replayed four times with
     new inputs between replays; every replay must equal the eager result."""
