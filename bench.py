@@ -334,10 +334,25 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
     calls = [(lambda k=k: mi.gqa_decode(dq, k[0], k[1], k[2], k[3], do, False, ws, stream=s)) for k in sets]
     ms = graph_time(mi, dev, s, timer, calls, reps) if graph else eager_time(dev, s, timer, calls)
     nbytes = wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
+    # the same step as a decode loop runs it: the new token's K and V heads are appended (rotate + quantize + write
+    # at position T-1 of every sequence), then attention reads the cache through per-sequence lengths
+    knew = dev.upload(wl.normal(88, (B, Hkv, D), 2))
+    vnew = dev.upload(wl.normal(88, (B, Hkv, D), 3))
+    dpos = dev.upload(np.full(B, T - 1, np.int32))
+    dlen = dev.upload(np.full(B, T, np.int32))
+
+    def cached(k):
+        mi.check(lib.mi_kv_append_f32_i8(knew.ptr, vnew.ptr, Hkv * D, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr,
+                                         dpos.ptr, B, Hkv, D, T, s))
+        mi.check(lib.mi_gqa_decode_attn_cache(dq.ptr, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr, do.ptr, B, Hq, Hkv, D,
+                                              T, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
+    calls2 = [(lambda k=k: cached(k)) for k in sets]
+    ms2 = graph_time(mi, dev, s, timer, calls2, reps) if graph else eager_time(dev, s, timer, calls2)
     dev.reset_to(mark)
     return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                                      "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes}}
+                                      "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes,
+                                      "with_kv_append_us": round(ms2 * 1e3, 2)}}
 
 
 def eager_time(dev, s, timer, calls):

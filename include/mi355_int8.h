@@ -191,6 +191,24 @@ MI_API int32_t mi_gqa_decode_attn(const float *q, const int8_t *kq, const float 
                                   int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T,
                                   int32_t out_rotated, void *workspace, int64_t workspace_bytes,
                                   void *stream);
+/* The same attention over a cache that is being filled: rows of kq/vq/ks/vs are T_cap tokens apart, sequence b
+ * holds seq_len[b] tokens (int32 [B] in device memory; values outside [0, T_max] are clamped, a length of 0 gives
+ * a row of zeros), T_max <= T_cap bounds every length and sizes the workspace
+ * (mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max)).  No upstream counterpart: the step that follows
+ * mi_kv_append_f32_i8 in a decode loop. */
+MI_API int32_t mi_gqa_decode_attn_cache(const float *q, const int8_t *kq, const float *ks,
+                                        const int8_t *vq, const float *vs, float *o,
+                                        int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                        const int32_t *seq_len, int64_t T_max, int32_t out_rotated,
+                                        void *workspace, int64_t workspace_bytes, void *stream);
+/* a7 as the decode loop uses it: rotate (block 128 = D) and quantize the new token's key and value heads and
+ * write codes and scale at token pos[b] of sequence b (int32 [B] in device memory; a sequence whose position is
+ * outside [0, T_cap) is skipped).  Head h of sequence b is read at k_new + b*row_stride + h*D (floats), so
+ * k_new/v_new may be slices of a fused QKV output (row_stride = its row length) or packed [B,Hkv,D]
+ * (row_stride = Hkv*D).  Same arithmetic, bit for bit, as mi_fwht_quant_f32_i8 with K = block = 128. */
+MI_API int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                   int8_t *kq, float *ks, int8_t *vq, float *vs, const int32_t *pos,
+                                   int64_t B, int64_t Hkv, int64_t D, int64_t T_cap, void *stream);
 /* Gate helper: runs the same split kernel and also writes out the int8 query
  * codes [B,Hq,D], their scales [B,Hq] and the raw int32 scores [B,Hq,T] it
  * works from (no merge, no o). */

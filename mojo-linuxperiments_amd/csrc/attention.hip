@@ -97,7 +97,9 @@ struct Params {
     int8_t *dump_qq;
     float *dump_sq;
     int32_t *dump_dots;
-    int Hq, Hkv, G, T;
+    int Hq, Hkv, G, T;    // T: tokens per sequence (the longest one when seq_len is given)
+    int Tstride;          // tokens between consecutive (batch, kv head) rows of the cache
+    const int32_t *seq_len;   // per-sequence token counts [B] (device), or null: every sequence holds T tokens
     int tiles_per_split;  // 16-token tiles
     float score_scale;    // log2(e) / sqrt(D)
 };
@@ -136,7 +138,7 @@ constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each)
 // RAGGED: the span a workgroup can cover runs past the end of the cache and token indices are clamped for the
 // loads; otherwise every address is base + constant.  Tokens past the end of the split are masked in the scores.
 template <bool DUMP, bool RAGGED>
-__device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
+__device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
                                                float (&s_red)[4][4][D], float (&s_sc)[4][WAVE_TILES][16][4],
                                                float (&s_m)[4][4], float (&s_l)[4][4], float (&s_c)[4][4])
 {
@@ -144,7 +146,7 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4]
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int split = blockIdx.x, bkv = blockIdx.y;
     const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
-    const int G = p.G, T = p.T;
+    const int G = p.G;
     const int ntiles = (T + 15) >> 4;
     const int tile_lo = split * p.tiles_per_split;
     const int tile_hi = min(tile_lo + p.tiles_per_split, ntiles);
@@ -155,10 +157,10 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, int8_t (&s_q)[4]
     const int tk16 = lane & 15, ck = lane >> 4;
     const int hh = lane & 3, slot = lane >> 3, chunk = lane & 7;
     const int t_wave = t_lo + wave * 16;      // first token of this wave's tile 0; tile j starts 64 tokens further
-    const int8_t *kwave = p.kq + ((int64_t)bkv * T + t_wave) * D;
-    const int8_t *vwave = p.vq + ((int64_t)bkv * T + t_wave) * D;
-    const float *kswave = p.ks + (int64_t)bkv * T + t_wave;
-    const float *vswave = p.vs + (int64_t)bkv * T + t_wave;
+    const int8_t *kwave = p.kq + ((int64_t)bkv * p.Tstride + t_wave) * D;
+    const int8_t *vwave = p.vq + ((int64_t)bkv * p.Tstride + t_wave) * D;
+    const float *kswave = p.ks + (int64_t)bkv * p.Tstride + t_wave;
+    const float *vswave = p.vs + (int64_t)bkv * p.Tstride + t_wave;
     const unsigned koff = (unsigned)(tk16 * D + 16 * ck);
 
     // the query row goes first: loads return in order, and the rotation of q can then run under the key loads
@@ -371,9 +373,25 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     __shared__ __attribute__((aligned(16))) float s_sc[4][WAVE_TILES][16][4];
     __shared__ float s_m[4][4], s_l[4][4], s_c[4][4];
     const int tile_lo = blockIdx.x * p.tiles_per_split;
-    const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= p.T;
-    if (full) gqa_split_body<DUMP, false>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
-    else gqa_split_body<DUMP, true>(p, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+    int T = p.T;
+    if (p.seq_len) {
+        // a cache that is filled to a different length per sequence: lengths outside [0, T] are clamped
+        const int b = blockIdx.y / p.Hkv;
+        T = min(max(__builtin_amdgcn_readfirstlane(p.seq_len[b]), 0), p.T);
+        if (tile_lo * 16 >= T) {
+            // this split lies past the end of the sequence: an empty partial (weight 0 in the merge)
+            const int64_t pbase = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x);
+            for (int o = threadIdx.x; o < 4 * D; o += 256) p.part_o[pbase * 4 * D + o] = 0.0f;
+            if (threadIdx.x < 4) {
+                p.part_ml[pbase * 8 + threadIdx.x] = -INFINITY;
+                p.part_ml[pbase * 8 + 4 + threadIdx.x] = 0.0f;
+            }
+            return;
+        }
+    }
+    const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= T;
+    if (full) gqa_split_body<DUMP, false>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+    else gqa_split_body<DUMP, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
 }
 
 // merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row.  SP > 0: the split count is known at
@@ -409,7 +427,7 @@ __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ par
         for (int s = 1; s < SP; ++s) mx = fmaxf(mx, ms[s]);
 #pragma unroll
         for (int s = 0; s < SP; ++s) {
-            const float w = __builtin_amdgcn_exp2f(ms[s] - mx);
+            const float w = (ms[s] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[s] - mx);   // empty split
             l = __builtin_fmaf(ls[s], w, l);
             v[0] = __builtin_fmaf(lo[s].x, w, v[0]); v[1] = __builtin_fmaf(lo[s].y, w, v[1]);
             v[2] = __builtin_fmaf(lo[s].z, w, v[2]); v[3] = __builtin_fmaf(lo[s].w, w, v[3]);
@@ -420,7 +438,8 @@ __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ par
         float mx = -INFINITY;
         for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml0[s * 8 + hl]);
         for (int s = 0; s < splits; ++s) {
-            const float w = __builtin_amdgcn_exp2f(ml0[s * 8 + hl] - mx);
+            const float ms = ml0[s * 8 + hl];
+            const float w = (ms == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);   // empty split
             l = __builtin_fmaf(ml0[s * 8 + 4 + hl], w, l);
             const float4 lo = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
             const float4 hi = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
@@ -430,7 +449,7 @@ __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ par
             v[6] = __builtin_fmaf(hi.z, w, v[6]); v[7] = __builtin_fmaf(hi.w, w, v[7]);
         }
     }
-    const float rl = 1.0f / l;
+    const float rl = l > 0.0f ? 1.0f / l : 0.0f;   // a sequence of length 0 gives a row of zeros
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] *= rl;
     if (!out_rotated) fwht128(v, j);  // whole workgroup takes the same branch
@@ -480,7 +499,7 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
 static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const int8_t *vq, const float *vs,
                         float *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T, int32_t out_rotated,
                         void *workspace, int64_t workspace_bytes, int8_t *dqq, float *dsq, int32_t *ddots,
-                        hipStream_t s)
+                        hipStream_t s, int64_t Tstride = 0, const int32_t *seq_len = nullptr)
 {
     int32_t rc = check_attn(B, Hq, Hkv, D, T);
     if (rc) return rc;
@@ -497,6 +516,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
                                           attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256));
     p.dump_qq = dqq; p.dump_sq = dsq; p.dump_dots = ddots;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.G = (int)(Hq / Hkv); p.T = (int)T;
+    p.Tstride = (int)(Tstride > 0 ? Tstride : T);
+    p.seq_len = seq_len;
     p.tiles_per_split = (ntiles + splits - 1) / splits;
     p.score_scale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
     const dim3 grid((unsigned)splits, (unsigned)(B * Hkv));
@@ -529,6 +550,19 @@ extern "C" int32_t mi_gqa_decode_attn(const float *q, const int8_t *kq, const fl
     if (!o || !aligned16(o)) return MI_EINVAL;
     return run_attn(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T, out_rotated, workspace, workspace_bytes, nullptr, nullptr,
                     nullptr, as_stream(stream));
+}
+
+extern "C" int32_t mi_gqa_decode_attn_cache(const float *q, const int8_t *kq, const float *ks, const int8_t *vq,
+                                            const float *vs, float *o, int64_t B, int64_t Hq, int64_t Hkv,
+                                            int64_t D, int64_t T_cap, const int32_t *seq_len, int64_t T_max,
+                                            int32_t out_rotated, void *workspace, int64_t workspace_bytes,
+                                            void *stream)
+{
+    if (!o || !aligned16(o) || !seq_len || !aligned4(seq_len)) return MI_EINVAL;
+    if (T_cap <= 0 || T_max <= 0 || T_max > T_cap) return MI_EINVAL;
+    if (T_cap > (1LL << 24)) return MI_ERANGE;
+    return run_attn(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_max, out_rotated, workspace, workspace_bytes, nullptr,
+                    nullptr, nullptr, as_stream(stream), T_cap, seq_len);
 }
 
 extern "C" int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const float *ks, const int8_t *vq,

@@ -194,6 +194,48 @@ __global__ __launch_bounds__(256) void k_fwht_small(const float *x, int8_t *__re
     }
 }
 
+// KV-cache append: the new token's key and value heads (128 floats each) are rotated and quantized exactly as
+// k_fwht_small<128> does, and the codes and the scale land at position pos[b] of sequence b in the cache
+// [B, Hkv, T_cap, 128] / [B, Hkv, T_cap].  16 lanes per head, 16 heads per workgroup; blockIdx.y = 0: keys, 1: values.
+__global__ __launch_bounds__(256) void k_kv_append(const float *__restrict__ k_new, const float *__restrict__ v_new,
+                                                   int64_t row_stride, int8_t *__restrict__ kq,
+                                                   float *__restrict__ ks, int8_t *__restrict__ vq,
+                                                   float *__restrict__ vs, const int32_t *__restrict__ pos, int B,
+                                                   int Hkv, int T_cap)
+{
+    constexpr int BLOCK = 128, LPB = 16;
+    const int t = threadIdx.x, j = t % LPB;
+    const int head = blockIdx.x * 16 + t / LPB;      // flat (b, h)
+    const bool is_v = blockIdx.y != 0;
+    const int b = min(head / Hkv, B - 1), h = head % Hkv;
+    const int tp = pos[b];
+    const bool live = head < B * Hkv && tp >= 0 && tp < T_cap;
+    const float *src = (is_v ? v_new : k_new) + (int64_t)b * row_stride + (int64_t)h * BLOCK + 4 * j;
+    float v[8];
+    if (live) {
+        const float4 lo = *reinterpret_cast<const float4 *>(src);
+        const float4 hi = *reinterpret_cast<const float4 *>(src + BLOCK / 2);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+        v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    }
+    fwht_chunk<BLOCK>(v, j);
+    float a = abs8(v);
+#pragma unroll
+    for (int m = LPB / 2; m >= 1; m >>= 1) a = fmaxf(a, __shfl_xor(a, m, 64));
+    const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+    const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+    if (live) {
+        const int64_t row = ((int64_t)b * Hkv + h) * T_cap + tp;
+        int8_t *q = (is_v ? vq : kq) + row * BLOCK + 4 * j;
+        if (j == 0) (is_v ? vs : ks)[row] = sc;
+        *reinterpret_cast<uint32_t *>(q) = quant4(v[0], v[1], v[2], v[3], inv);
+        *reinterpret_cast<uint32_t *>(q + BLOCK / 2) = quant4(v[4], v[5], v[6], v[7], inv);
+    }
+}
+
 template <int BLOCK, bool QUANT>
 static int32_t launch_rows(const float *x, int8_t *q, float *scale, float *xrot, int64_t M, int64_t K,
                            hipStream_t s)
@@ -256,6 +298,23 @@ extern "C" int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale,
     if (M == 0) return MI_OK;
     return block == 128 ? launch_rows<128, true>(x, q, scale, nullptr, M, K, as_stream(stream))
                         : launch_rows<256, true>(x, q, scale, nullptr, M, K, as_stream(stream));
+}
+
+extern "C" int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, int64_t row_stride, int8_t *kq,
+                                       float *ks, int8_t *vq, float *vs, const int32_t *pos, int64_t B,
+                                       int64_t Hkv, int64_t D, int64_t T_cap, void *stream)
+{
+    if (!k_new || !v_new || !kq || !ks || !vq || !vs || !pos) return MI_EINVAL;
+    if (B <= 0 || Hkv <= 0 || T_cap <= 0 || D != 128) return MI_EINVAL;
+    if (row_stride < Hkv * D || row_stride % 4) return MI_EINVAL;
+    if (B * Hkv > (1LL << 24) || T_cap > (1LL << 24)) return MI_ERANGE;
+    if (!aligned16(k_new) || !aligned16(v_new) || !aligned4(kq) || !aligned4(vq) || !aligned4(ks) || !aligned4(vs) ||
+        !aligned4(pos))
+        return MI_EINVAL;
+    const dim3 grid((unsigned)((B * Hkv + 15) / 16), 2);
+    hipLaunchKernelGGL(k_kv_append, grid, dim3(256), 0, as_stream(stream), k_new, v_new, row_stride, kq, ks, vq, vs,
+                       pos, (int)B, (int)Hkv, (int)T_cap);
+    return launch_status();
 }
 
 extern "C" int32_t mi_fwht_f32(const float *x, float *out, int64_t M, int64_t K, int32_t block, void *stream)

@@ -201,6 +201,43 @@ struct DecodeAttention {
     }
 };
 
+// An int8 KV cache of fixed capacity held in an arena: the decode loop appends one token per sequence at its own
+// position and attends over what each sequence holds.  Positions and lengths are int32 [B] arrays in device memory
+// (the loop that produces them runs on the device side of the stream, not on the host).
+struct KvCache {
+    int64_t B = 0, Hq = 0, Hkv = 0, D = 128, T_cap = 0;
+    int8_t *kq = nullptr, *vq = nullptr;
+    float *ks = nullptr, *vs = nullptr;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t_cap)
+    {
+        B = b; Hq = hq; Hkv = hkv; T_cap = t_cap;
+        workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap);
+        if (workspace_bytes <= 0) return false;
+        kq = arena.template alloc<int8_t>(B * Hkv * T_cap * D);
+        vq = arena.template alloc<int8_t>(B * Hkv * T_cap * D);
+        ks = arena.template alloc<float>(B * Hkv * T_cap);
+        vs = arena.template alloc<float>(B * Hkv * T_cap);
+        workspace = arena.template alloc<uint8_t>(workspace_bytes);
+        return kq && vq && ks && vs && workspace;
+    }
+    explicit operator bool() const { return workspace != nullptr; }
+    // k_new / v_new: head h of sequence b at + b*row_stride + h*128 floats (slices of a fused QKV row are fine)
+    int32_t append(const float *k_new, const float *v_new, int64_t row_stride, const int32_t *pos, void *stream) const
+    {
+        return mi_kv_append_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, pos, B, Hkv, D, T_cap, stream);
+    }
+    // t_max bounds every entry of seq_len (<= T_cap); a tighter bound launches fewer splits
+    int32_t attend(const float *q, float *o, const int32_t *seq_len, int64_t t_max, bool out_rotated, void *stream) const
+    {
+        return mi_gqa_decode_attn_cache(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_cap, seq_len, t_max,
+                                        out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+    }
+};
+
 // Router + top-k dispatch + grouped expert SwiGLU FFN.
 struct MoeFfn {
     int64_t T = 0, H = 0, I = 0, E = 0;

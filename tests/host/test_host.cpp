@@ -207,6 +207,74 @@ static void test_decode_attention(const Context &ctx)
     report("decode_attention_vs_oracle", ok && err <= 2e-3f, "max-abs " + std::to_string(err));
 }
 
+// three decode steps through KvCache: append at per-sequence positions, attend over per-sequence lengths; the
+// cache rows follow the oracle quantizer bit for bit and the output follows the oracle on each sequence's prefix
+static void test_kv_cache(const Context &ctx)
+{
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 128, T_cap = 40;
+    DeviceArena<256> arena(ctx, 64 << 20);
+    KvCache cache;
+    bool ok = cache.prepare(arena, B, Hq, Hkv, T_cap) && (bool)cache;
+    Rng rng{11};
+    std::vector<int8_t> rkq(B * Hkv * T_cap * D, 0), rvq(B * Hkv * T_cap * D, 0);
+    std::vector<float> rks(B * Hkv * T_cap, 0.0f), rvs(B * Hkv * T_cap, 0.0f);
+    const int32_t start[2] = {0, 30};
+    float err = 0;
+    int32_t *dpos = arena.alloc<int32_t>(B), *dlen = arena.alloc<int32_t>(B);
+    float *dq = arena.alloc<float>(B * Hq * D), *dk = arena.alloc<float>(B * Hkv * D), *dv = arena.alloc<float>(B * Hkv * D);
+    float *dout = arena.alloc<float>(B * Hq * D);
+    ok = ok && dpos && dlen && dq && dk && dv && dout;
+    for (int step = 0; ok && step < 3; ++step) {
+        std::vector<float> q(B * Hq * D), k(B * Hkv * D), v(B * Hkv * D);
+        for (auto &e : q) e = rng.normal();
+        for (auto &e : k) e = rng.normal();
+        for (auto &e : v) e = rng.normal();
+        // sequence 1 starts with 30 tokens the cache never received: they stay zero codes with zero scales,
+        // which the oracle sees too
+        int32_t pos[2] = {start[0] + step, start[1] + step}, len[2] = {pos[0] + 1, pos[1] + 1};
+        mi_memcpy_h2d(dpos, pos, sizeof(pos), nullptr);
+        mi_memcpy_h2d(dlen, len, sizeof(len), nullptr);
+        mi_memcpy_h2d(dq, q.data(), (int64_t)q.size() * 4, nullptr);
+        mi_memcpy_h2d(dk, k.data(), (int64_t)k.size() * 4, nullptr);
+        mi_memcpy_h2d(dv, v.data(), (int64_t)v.size() * 4, nullptr);
+        ok = ok && cache.append(dk, dv, Hkv * D, dpos, nullptr) == MI_OK;
+        ok = ok && cache.attend(dq, dout, dlen, len[1], false, nullptr) == MI_OK;
+        std::vector<float> o = download(dout, (size_t)(B * Hq * D));
+        std::vector<int8_t> cq(B * Hkv * D), cvq(B * Hkv * D);
+        std::vector<float> cs(B * Hkv), cvs(B * Hkv);
+        orc_rotate_quant_rows(k.data(), B * Hkv, D, 128, cq.data(), cs.data(), nullptr);
+        orc_rotate_quant_rows(v.data(), B * Hkv, D, 128, cvq.data(), cvs.data(), nullptr);
+        for (int64_t b = 0; b < B; ++b)
+            for (int64_t h = 0; h < Hkv; ++h) {
+                const int64_t row = (b * Hkv + h) * T_cap + pos[b];
+                std::copy(cq.begin() + (b * Hkv + h) * D, cq.begin() + (b * Hkv + h + 1) * D, rkq.begin() + row * D);
+                std::copy(cvq.begin() + (b * Hkv + h) * D, cvq.begin() + (b * Hkv + h + 1) * D, rvq.begin() + row * D);
+                rks[row] = cs[b * Hkv + h];
+                rvs[row] = cvs[b * Hkv + h];
+            }
+        for (int64_t b = 0; b < B; ++b) {
+            // the oracle takes a dense [1, Hkv, len, D] cache: gather this sequence's prefix
+            const int64_t n = len[b];
+            std::vector<int8_t> pk(Hkv * n * D), pv(Hkv * n * D);
+            std::vector<float> pks(Hkv * n), pvs(Hkv * n), o_ref(Hq * D);
+            for (int64_t h = 0; h < Hkv; ++h) {
+                const int64_t row = (b * Hkv + h) * T_cap;
+                std::copy(rkq.begin() + row * D, rkq.begin() + (row + n) * D, pk.begin() + h * n * D);
+                std::copy(rvq.begin() + row * D, rvq.begin() + (row + n) * D, pv.begin() + h * n * D);
+                std::copy(rks.begin() + row, rks.begin() + row + n, pks.begin() + h * n);
+                std::copy(rvs.begin() + row, rvs.begin() + row + n, pvs.begin() + h * n);
+            }
+            orc_gqa_decode(q.data() + b * Hq * D, pk.data(), pks.data(), pv.data(), pvs.data(), o_ref.data(), 1, Hq, Hkv,
+                           D, n, 0, nullptr, nullptr, nullptr);
+            for (int64_t i = 0; i < Hq * D; ++i) err = std::fmax(err, std::fabs(o[b * Hq * D + i] - o_ref[i]));
+        }
+    }
+    std::vector<int8_t> hkq = download(cache.kq, (size_t)(B * Hkv * T_cap * D));
+    std::vector<float> hvs = download(cache.vs, (size_t)(B * Hkv * T_cap));
+    ok = ok && hkq == rkq && hvs == rvs;
+    report("kv_cache_append_attend_vs_oracle", ok && err <= 2e-3f, "max-abs " + std::to_string(err));
+}
+
 int main()
 {
     Context ctx(0);
@@ -217,6 +285,7 @@ int main()
     test_stream_pool(ctx);
     test_quant_linear(ctx);
     test_decode_attention(ctx);
+    test_kv_cache(ctx);
     std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;
 }
