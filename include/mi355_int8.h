@@ -256,6 +256,30 @@ MI_API int32_t mi_moe_layer(const float *x, const float *wr,
                             void *workspace, int64_t workspace_bytes, void *stream);
 MI_API int64_t mi_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk);
 
+/* ---- the fp32 operators between the int8 kernels of one decoder layer (decode step).  No upstream
+ * counterpart (upstream holds no model code); they chain the entry points above into
+ * RMSNorm -> QKV -> rotary + cache append -> attention -> O -> RMSNorm -> gate|up -> SwiGLU -> down.
+ * RMSNorm: h = x (+ residual, then also written to h_out); y = (h * r) * g, r = 1/sqrt(mean(h^2) + eps).
+ * x, residual, h_out, y fp32 [M,H]; g fp32 [H]; H % 4 == 0, H <= 16384. */
+MI_API int32_t mi_rmsnorm_f32(const float *x, const float *residual, const float *g, float eps,
+                              float *h_out, float *y, int64_t M, int64_t H, void *stream);
+/* One decode token per sequence.  qkv fp32: row b = [Hq query heads | Hkv key heads | Hkv value heads] x D, rows
+ * row_stride floats apart (the output of a fused QKV projection).  Query and key heads get the rotary embedding
+ * of position pos[b]: pairs (i, i + D/2), x'[i] = x[i]*cos - x[i+D/2]*sin, x'[i+D/2] = x[i+D/2]*cos + x[i]*sin
+ * with cos/sin = rope_cos/rope_sin[pos[b]][i] (fp32 [T_cap, D/2] tables of the caller).  Queries leave packed
+ * in q_out fp32 [B,Hq,D] (what the attention entry points take); keys (after the embedding) and values are
+ * rotated (block D) and quantized exactly as mi_kv_append_f32_i8 does and stored at token pos[b] of the cache.
+ * A sequence whose position is outside [0, T_cap) writes nothing (its q_out rows keep what they held).  D == 128. */
+MI_API int32_t mi_rope_kv_append_f32_i8(const float *qkv, int64_t row_stride, const float *rope_cos,
+                                        const float *rope_sin, float *q_out, int8_t *kq, float *ks, int8_t *vq,
+                                        float *vs,
+                                        const int32_t *pos, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                        int64_t T_cap, void *stream);
+/* h[m,n] = silu(gate_up[m,n]) * gate_up[m,I+n]; gate_up fp32 [M,2I] (one projection of N = 2I), h fp32 [M,I]. */
+MI_API int32_t mi_swiglu_f32(const float *gate_up, float *h, int64_t M, int64_t I, void *stream);
+/* out = a + b over n floats (n % 4 == 0): the residual add that closes the layer. */
+MI_API int32_t mi_add_f32(const float *a, const float *b, float *out, int64_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

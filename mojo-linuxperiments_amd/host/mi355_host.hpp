@@ -6,7 +6,7 @@
 // :70-80, :103-121).  No Mojo toolchain exists where this is built, so the same
 // surface is written in C++: DeviceArena mirrors NumaArena, StreamPool mirrors
 // ThreadPool, Gate mirrors MutexGate, and QuantLinear / DecodeAttention /
-// MoeFfn are the quantize / linear / attention / MoE call surface that a Mojo
+// KvCache / DecoderLayer / MoeFfn are the quantize / linear / attention / MoE call surface that a Mojo
 // host would hold as structs over the same handles.  Nothing here throws.
 #pragma once
 #include <cstdint>
@@ -235,6 +235,63 @@ struct KvCache {
     {
         return mi_gqa_decode_attn_cache(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_cap, seq_len, t_max,
                                         out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+    }
+};
+
+// One decoder layer of a decode step (one new token per sequence), chained on one stream:
+// RMSNorm -> QKV -> rotary + cache append -> attention over the cache -> O -> residual + RMSNorm -> gate|up ->
+// SwiGLU -> down -> residual.  Holds its prepared weights, its KV cache and its scratch rows in the arena.
+struct DecoderLayer {
+    int64_t B = 0, H = 0, Hq = 0, Hkv = 0, I = 0, T_cap = 0;
+    float eps = 1e-5f;
+    QuantLinear<128> qkv, o, gate_up, down;
+    KvCache cache;
+    const float *g1 = nullptr, *g2 = nullptr, *rope_cos = nullptr, *rope_sin = nullptr;
+    float *xn = nullptr, *qkv_out = nullptr, *q = nullptr, *att = nullptr, *ao = nullptr, *h1 = nullptr, *hn = nullptr,
+          *gu = nullptr, *act = nullptr, *dn = nullptr;
+
+    // fp32 weights in device memory: wqkv [(Hq+2Hkv)*128, H], wo [H, Hq*128], wgu [2I, H] (gate rows, then up
+    // rows), wd [H, I]; norm weights g1, g2 [H]; rotary tables [T_cap, 64].  false if the arena is exhausted.
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t b, int64_t h, int64_t hq, int64_t hkv, int64_t i, int64_t t_cap,
+                 const float *wqkv, const float *wo, const float *wgu, const float *wd, const float *norm1,
+                 const float *norm2, const float *cos_table, const float *sin_table, float epsilon, void *stream)
+    {
+        B = b; H = h; Hq = hq; Hkv = hkv; I = i; T_cap = t_cap; eps = epsilon;
+        g1 = norm1; g2 = norm2; rope_cos = cos_table; rope_sin = sin_table;
+        const int64_t nqkv = (Hq + 2 * Hkv) * 128;
+        bool ok = qkv.prepare(arena, wqkv, nqkv, H, B, stream) && o.prepare(arena, wo, H, Hq * 128, B, stream) &&
+                  gate_up.prepare(arena, wgu, 2 * I, H, B, stream) && down.prepare(arena, wd, H, I, B, stream) &&
+                  cache.prepare(arena, B, Hq, Hkv, T_cap);
+        xn = arena.template alloc<float>(B * H);
+        qkv_out = arena.template alloc<float>(B * nqkv);
+        q = arena.template alloc<float>(B * Hq * 128);
+        att = arena.template alloc<float>(B * Hq * 128);
+        ao = arena.template alloc<float>(B * H);
+        h1 = arena.template alloc<float>(B * H);
+        hn = arena.template alloc<float>(B * H);
+        gu = arena.template alloc<float>(B * 2 * I);
+        act = arena.template alloc<float>(B * I);
+        dn = arena.template alloc<float>(B * H);
+        return ok && xn && qkv_out && q && att && ao && h1 && hn && gu && act && dn;
+    }
+    // x, out fp32 [B,H]; pos, seq_len int32 [B] in device memory (seq_len = pos + 1 in a plain decode step);
+    // t_max bounds seq_len.  The first failing call's status is returned.
+    int32_t step(const float *x, const int32_t *pos, const int32_t *seq_len, int64_t t_max, float *out, void *stream) const
+    {
+        int32_t rc = mi_rmsnorm_f32(x, nullptr, g1, eps, nullptr, xn, B, H, stream);
+        if (rc == MI_OK) rc = qkv.forward(xn, qkv_out, B, stream);
+        if (rc == MI_OK)
+            rc = mi_rope_kv_append_f32_i8(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, cache.kq, cache.ks,
+                                          cache.vq, cache.vs, pos, B, Hq, Hkv, 128, T_cap, stream);
+        if (rc == MI_OK) rc = cache.attend(q, att, seq_len, t_max, false, stream);
+        if (rc == MI_OK) rc = o.forward(att, ao, B, stream);
+        if (rc == MI_OK) rc = mi_rmsnorm_f32(ao, x, g2, eps, h1, hn, B, H, stream);
+        if (rc == MI_OK) rc = gate_up.forward(hn, gu, B, stream);
+        if (rc == MI_OK) rc = mi_swiglu_f32(gu, act, B, I, stream);
+        if (rc == MI_OK) rc = down.forward(act, dn, B, stream);
+        if (rc == MI_OK) rc = mi_add_f32(h1, dn, out, B * H, stream);
+        return rc;
     }
 };
 

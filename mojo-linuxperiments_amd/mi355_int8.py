@@ -89,6 +89,10 @@ SIGNATURES = {
     "mi_gqa_decode_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
     "mi_gqa_decode_attn": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp]),
     "mi_gqa_decode_attn_cache": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64, vp]),
+    "mi_rmsnorm_f32": (i32, [vp, vp, vp, C.c_float, vp, vp, i64, i64, vp]),
+    "mi_rope_kv_append_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
+    "mi_swiglu_f32": (i32, [vp, vp, i64, i64, vp]),
+    "mi_add_f32": (i32, [vp, vp, vp, i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_moe_route_workspace_bytes": (i64, [i64, i64]),
@@ -364,3 +368,62 @@ def moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=None):
     E, I, _ = wg.shape
     check(lib.mi_moe_layer(x.ptr, wr.ptr, wg.ptr, sg.ptr, wu.ptr, su.ptr, wd.ptr, sd.ptr, y.ptr,
                            T, H, I, E, topk, ws.ptr, ws.nbytes, stream), "mi_moe_layer")
+
+
+class DecoderLayer:
+    """One decoder layer of a decode step, chained from the C-ABI entry points on one stream:
+    RMSNorm -> QKV linear -> rotary + KV-cache append -> attention over the cache -> O linear -> residual +
+    RMSNorm -> gate|up linear -> SwiGLU -> down linear -> residual.  Test and bench plumbing over the same calls
+    the C++ host struct of the same name makes (host/mi355_host.hpp)."""
+
+    def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
+                 block=128):
+        D = 128
+        self.dev, self.B, self.H, self.Hq, self.Hkv, self.I, self.T_cap, self.eps, self.block = \
+            dev, B, H, Hq, Hkv, I, T_cap, eps, block
+        self.NQKV = (Hq + 2 * Hkv) * D
+
+        def prep(w):
+            mark = dev.mark()
+            N, K = w.shape
+            q, s = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+            keep = dev.mark()
+            dw = dev.upload(w)
+            fwht_quant(dw, q, s, block)
+            dev.sync()
+            dev.reset_to(keep)
+            del mark
+            return q, s
+        self.wqkv, self.wo, self.wgu, self.wd = prep(wqkv), prep(wo), prep(wgu), prep(wd)
+        self.g1, self.g2 = dev.upload(g1), dev.upload(g2)
+        self.cos, self.sin = dev.upload(rope_cos), dev.upload(rope_sin)
+        self.kq, self.ks = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
+        self.vq, self.vs = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
+        f = np.float32
+        self.xn, self.qkv = dev.empty((B, H), f), dev.empty((B, self.NQKV), f)
+        self.q, self.att = dev.empty((B, Hq, D), f), dev.empty((B, Hq * D), f)
+        self.ao, self.h1, self.hn = dev.empty((B, H), f), dev.empty((B, H), f), dev.empty((B, H), f)
+        self.gu, self.act, self.dn = dev.empty((B, 2 * I), f), dev.empty((B, I), f), dev.empty((B, H), f)
+        nws = max(lib.mi_w8a8_linear_workspace_bytes(B, n, k) for n, k in
+                  ((self.NQKV, H), (H, Hq * D), (2 * I, H), (H, I)))
+        self.lin_ws = dev.empty(nws, np.uint8)
+        self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
+
+    def step(self, x, pos, seq_len, t_max, out, stream=None):
+        """x, out fp32 [B,H]; pos, seq_len int32 [B] on the device (seq_len = pos + 1 for a plain decode step)."""
+        B, H, Hq, Hkv, I, D, s = self.B, self.H, self.Hq, self.Hkv, self.I, 128, stream
+        check(lib.mi_rmsnorm_f32(x.ptr, None, self.g1.ptr, self.eps, None, self.xn.ptr, B, H, s), "mi_rmsnorm_f32")
+        linear(self.xn, self.wqkv[0], self.wqkv[1], self.qkv, self.block, self.lin_ws, s)
+        check(lib.mi_rope_kv_append_f32_i8(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr,
+                                           self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv,
+                                           D, self.T_cap, s), "mi_rope_kv_append_f32_i8")
+        check(lib.mi_gqa_decode_attn_cache(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
+                                           self.att.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, 0,
+                                           self.att_ws.ptr, self.att_ws.nbytes, s), "mi_gqa_decode_attn_cache")
+        linear(self.att, self.wo[0], self.wo[1], self.ao, self.block, self.lin_ws, s)
+        check(lib.mi_rmsnorm_f32(self.ao.ptr, x.ptr, self.g2.ptr, self.eps, self.h1.ptr, self.hn.ptr, B, H, s),
+              "mi_rmsnorm_f32")
+        linear(self.hn, self.wgu[0], self.wgu[1], self.gu, self.block, self.lin_ws, s)
+        check(lib.mi_swiglu_f32(self.gu.ptr, self.act.ptr, B, I, s), "mi_swiglu_f32")
+        linear(self.act, self.wd[0], self.wd[1], self.dn, self.block, self.lin_ws, s)
+        check(lib.mi_add_f32(self.h1.ptr, self.dn.ptr, out.ptr, B * H, s), "mi_add_f32")

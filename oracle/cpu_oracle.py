@@ -200,5 +200,41 @@ def moe_ffn(x, idx, w, wg, sg, wu, su, wd, sd, b_in, b_mid, h_in=None, want_debu
     return (y, h, hq, hs, accd) if want_debug else y
 
 
+def rmsnorm(x, g, eps, residual=None):
+    """D10.  Returns y, or (h, y) when a residual is added first."""
+    x = _c(x, np.float32)
+    M, H = x.shape
+    g = _c(g, np.float32)
+    y = np.empty((M, H), np.float32)
+    res = _c(residual, np.float32) if residual is not None else None
+    h = np.empty((M, H), np.float32) if residual is not None else None
+    rc = lib().orc_rmsnorm(_p(x), _p(res), _p(g), C.c_float(eps), _p(h), _p(y), i64(M), i64(H))
+    if rc:
+        raise ValueError("orc_rmsnorm rc=%d" % rc)
+    return (h, y) if residual is not None else y
+
+
+def rope_rows(rows, pos, cos, sin):
+    """D11 on fp32 [R, D] rows (a copy is returned); row r takes table row pos[r]."""
+    rows = np.array(rows, np.float32, order="C", copy=True)
+    R, D = rows.shape
+    pos = _c(pos, np.int32)
+    rc = lib().orc_rope_rows(_p(rows), _p(pos), _p(_c(cos, np.float32)), _p(_c(sin, np.float32)), i64(R), i64(D))
+    if rc:
+        raise ValueError("orc_rope_rows rc=%d" % rc)
+    return rows
+
+
+def swiglu(gate_up):
+    """D12: fp32 [M, 2I] -> [M, I]."""
+    gu = _c(gate_up, np.float32)
+    M, I2 = gu.shape
+    h = np.empty((M, I2 // 2), np.float32)
+    rc = lib().orc_swiglu(_p(gu), _p(h), i64(M), i64(I2 // 2))
+    if rc:
+        raise ValueError("orc_swiglu rc=%d" % rc)
+    return h
+
+
 def num_threads():
     return int(lib().orc_num_threads())

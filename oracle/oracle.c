@@ -57,6 +57,15 @@
  *  D9  Combine: y[token] = sum over slots 0..topk-1 in that order of
  *      w[token][slot] * out[pair], starting from 0.0f, one multiply and one
  *      add per term.
+ *  D10 RMSNorm: h = x + residual (one fp32 add; h = x without a residual);
+ *      the mean of squares is accumulated in float64 in index order (the GPU
+ *      sums in fp32 and is gated by tolerance); r = (float)(1 / sqrt(ss / H +
+ *      eps)); y = (h * r) * g, two fp32 multiplies in that order.
+ *  D11 Rotary embedding over a head of D values: pairs (i, i + D/2), angles
+ *      from caller tables cos/sin[pos][i]: x'[i] = x[i]*c - x[i+D/2]*s,
+ *      x'[i+D/2] = x[i+D/2]*c + x[i]*s; every product is rounded to fp32
+ *      before the add or subtract (no FMA), so the result is fixed by IEEE-754.
+ *  D12 SwiGLU over a fused row [gate(I) | up(I)]: D8 on (g[n], u[n]).
  */
 #include <math.h>
 #include <stdint.h>
@@ -400,6 +409,56 @@ ORC_API int orc_moe_ffn(const float *x, const int32_t *idx, const float *w,
     }
     free(qx); free(sx); free(perm); free(seg); free(outp);
     return rc;
+}
+
+/* ---- decoder-layer glue (D10-D12) --------------------------------------- */
+
+ORC_API int orc_rmsnorm(const float *x, const float *residual, const float *g, float eps, float *h_out, float *y,
+                        int64_t M, int64_t H)
+{
+    if (!x || !g || !y || M < 0 || H <= 0 || (residual && !h_out)) return -1;
+    for (int64_t m = 0; m < M; ++m) {
+        double ss = 0.0;
+        for (int64_t i = 0; i < H; ++i) {
+            float h = x[m * H + i];
+            if (residual) { h = h + residual[m * H + i]; h_out[m * H + i] = h; }
+            ss += (double)h * (double)h;
+        }
+        const float r = (float)(1.0 / sqrt(ss / (double)H + (double)eps));
+        for (int64_t i = 0; i < H; ++i) {
+            const float h = residual ? h_out[m * H + i] : x[m * H + i];
+            const float t = h * r;
+            y[m * H + i] = t * g[i];
+        }
+    }
+    return 0;
+}
+
+/* rows fp32 [R, D] rotated in place; row r uses table row pos[r] */
+ORC_API int orc_rope_rows(float *rows, const int32_t *pos, const float *cs, const float *sn, int64_t R, int64_t D)
+{
+    if (!rows || !pos || !cs || !sn || R < 0 || D <= 0 || D % 2) return -1;
+    const int64_t half = D / 2;
+    for (int64_t r = 0; r < R; ++r)
+        for (int64_t i = 0; i < half; ++i) {
+            const float a = rows[r * D + i], b = rows[r * D + half + i];
+            const float c = cs[(int64_t)pos[r] * half + i], s = sn[(int64_t)pos[r] * half + i];
+            const float ac = a * c, bs = b * s, bc = b * c, as = a * s;
+            rows[r * D + i] = ac - bs;
+            rows[r * D + half + i] = bc + as;
+        }
+    return 0;
+}
+
+ORC_API int orc_swiglu(const float *gate_up, float *h, int64_t M, int64_t I)
+{
+    if (!gate_up || !h || M < 0 || I <= 0) return -1;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < I; ++n) {
+            const float g = gate_up[m * 2 * I + n], u = gate_up[m * 2 * I + I + n];
+            h[m * I + n] = (g / (1.0f + expf(-g))) * u;
+        }
+    return 0;
 }
 
 ORC_API int orc_num_threads(void)

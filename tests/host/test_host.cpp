@@ -2,6 +2,7 @@
 // upstream test program (test_linux_threading.mojo:11-16, :555-570): each test
 // prints [PASS]/[FAIL]; unlike upstream, a failure also sets the exit status.
 // The CPU oracle (oracle/oracle.c) is linked here as the checker only.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -17,6 +18,9 @@ int orc_w8a8_linear(const float *, const int8_t *, const float *, float *, int64
                     float *, int32_t *);
 int orc_gqa_decode(const float *, const int8_t *, const float *, const int8_t *, const float *, float *, int64_t,
                    int64_t, int64_t, int64_t, int64_t, int, int8_t *, float *, int32_t *);
+int orc_rmsnorm(const float *, const float *, const float *, float, float *, float *, int64_t, int64_t);
+int orc_rope_rows(float *, const int32_t *, const float *, const float *, int64_t, int64_t);
+int orc_swiglu(const float *, float *, int64_t, int64_t);
 }
 
 using namespace mi355;
@@ -275,6 +279,107 @@ static void test_kv_cache(const Context &ctx)
     report("kv_cache_append_attend_vs_oracle", ok && err <= 2e-3f, "max-abs " + std::to_string(err));
 }
 
+// DecoderLayer::step against the oracle's operators chained in the same order, every stage fed what the device
+// fed its next kernel (integer stages equal, fp32 stages to 2e-6 relative; attention to 2e-5 absolute)
+static void test_decoder_layer(const Context &ctx)
+{
+    const int64_t B = 2, H = 512, Hq = 4, Hkv = 2, I = 1024, T_cap = 24, D = 128, NQ = (Hq + 2 * Hkv) * D;
+    DeviceArena<256> arena(ctx, 256 << 20);
+    Rng rng{3};
+    auto gauss = [&](int64_t n, float s) { std::vector<float> v((size_t)n); for (auto &e : v) e = s * rng.normal(); return v; };
+    std::vector<float> wqkv = gauss(NQ * H, 0.02f), wo = gauss(H * Hq * D, 0.02f), wgu = gauss(2 * I * H, 0.02f),
+                       wd = gauss(H * I, 0.02f), g1 = gauss(H, 0.1f), g2 = gauss(H, 0.1f), x = gauss(B * H, 1.0f);
+    for (auto &e : g1) e += 1.0f;
+    for (auto &e : g2) e += 1.0f;
+    std::vector<float> cs((size_t)(T_cap * 64)), sn((size_t)(T_cap * 64));
+    for (int64_t t = 0; t < T_cap; ++t)
+        for (int64_t i = 0; i < 64; ++i) {
+            const double a = (double)t * std::pow(10000.0, -2.0 * (double)i / 128.0);
+            cs[t * 64 + i] = (float)std::cos(a);
+            sn[t * 64 + i] = (float)std::sin(a);
+        }
+    DecoderLayer layer;
+    bool ok = layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, upload(arena, wqkv), upload(arena, wo), upload(arena, wgu),
+                            upload(arena, wd), upload(arena, g1), upload(arena, g2), upload(arena, cs), upload(arena, sn),
+                            1e-5f, nullptr);
+    const std::vector<int32_t> pos = {0, 9}, len = {1, 10};
+    int32_t *dpos = upload(arena, pos), *dlen = upload(arena, len);
+    float *dx = upload(arena, x), *dout = arena.alloc<float>(B * H);
+    ok = ok && dpos && dlen && dx && dout && layer.step(dx, dpos, dlen, 10, dout, nullptr) == MI_OK;
+    if (!ok) { report("decoder_layer_vs_oracle", false, "set-up or launch failed"); return; }
+    auto close = [](const std::vector<float> &a, const std::vector<float> &b, float tol) {
+        float m = 0, d = 0;
+        for (size_t i = 0; i < a.size(); ++i) { m = std::fmax(m, std::fabs(b[i])); d = std::fmax(d, std::fabs(a[i] - b[i])); }
+        return d <= tol * std::fmax(m, 1.0f);
+    };
+    std::vector<int8_t> qw((size_t)(NQ * H)), ow((size_t)(H * Hq * D)), guw((size_t)(2 * I * H)), dw((size_t)(H * I));
+    std::vector<float> qs((size_t)NQ), os((size_t)H), gus((size_t)(2 * I)), ds((size_t)H);
+    orc_rotate_quant_rows(wqkv.data(), NQ, H, 128, qw.data(), qs.data(), nullptr);
+    orc_rotate_quant_rows(wo.data(), H, Hq * D, 128, ow.data(), os.data(), nullptr);
+    orc_rotate_quant_rows(wgu.data(), 2 * I, H, 128, guw.data(), gus.data(), nullptr);
+    orc_rotate_quant_rows(wd.data(), H, I, 128, dw.data(), ds.data(), nullptr);
+    std::vector<float> xn = download(layer.xn, (size_t)(B * H)), r((size_t)(B * H));
+    orc_rmsnorm(x.data(), nullptr, g1.data(), 1e-5f, nullptr, r.data(), B, H);
+    bool good = close(xn, r, 2e-6f);
+    std::vector<float> qkv = download(layer.qkv_out, (size_t)(B * NQ)), y((size_t)(B * NQ));
+    orc_w8a8_linear(xn.data(), qw.data(), qs.data(), y.data(), B, NQ, H, 128, nullptr, nullptr, nullptr);
+    good = good && qkv == y;
+    // rotary embedding of the query and key heads, then the cache rows of this step
+    std::vector<float> q = download(layer.q, (size_t)(B * Hq * D));
+    std::vector<int8_t> kq = download(layer.cache.kq, (size_t)(B * Hkv * T_cap * D)), vq = download(layer.cache.vq, (size_t)(B * Hkv * T_cap * D));
+    std::vector<float> ks = download(layer.cache.ks, (size_t)(B * Hkv * T_cap)), vs = download(layer.cache.vs, (size_t)(B * Hkv * T_cap));
+    for (int64_t b = 0; b < B && good; ++b) {
+        std::vector<float> rows(qkv.begin() + b * NQ, qkv.begin() + b * NQ + (Hq + Hkv) * D);
+        std::vector<int32_t> pp((size_t)(Hq + Hkv), pos[b]);
+        orc_rope_rows(rows.data(), pp.data(), cs.data(), sn.data(), Hq + Hkv, D);
+        good = good && std::equal(rows.begin(), rows.begin() + Hq * D, q.begin() + b * Hq * D);
+        std::vector<int8_t> c((size_t)(Hkv * D));
+        std::vector<float> sc((size_t)Hkv);
+        orc_rotate_quant_rows(rows.data() + Hq * D, Hkv, D, 128, c.data(), sc.data(), nullptr);
+        for (int64_t h = 0; h < Hkv; ++h) {
+            const int64_t row = (b * Hkv + h) * T_cap + pos[b];
+            good = good && std::equal(c.begin() + h * D, c.begin() + (h + 1) * D, kq.begin() + row * D) && ks[row] == sc[h];
+        }
+    }
+    std::vector<float> att = download(layer.att, (size_t)(B * Hq * D));
+    for (int64_t b = 0; b < B && good; ++b) {
+        const int64_t n = len[b];
+        std::vector<int8_t> pk((size_t)(Hkv * n * D)), pv((size_t)(Hkv * n * D));
+        std::vector<float> pks((size_t)(Hkv * n)), pvs((size_t)(Hkv * n)), o_ref((size_t)(Hq * D));
+        for (int64_t h = 0; h < Hkv; ++h) {
+            const int64_t row = (b * Hkv + h) * T_cap;
+            std::copy(kq.begin() + row * D, kq.begin() + (row + n) * D, pk.begin() + h * n * D);
+            std::copy(vq.begin() + row * D, vq.begin() + (row + n) * D, pv.begin() + h * n * D);
+            std::copy(ks.begin() + row, ks.begin() + row + n, pks.begin() + h * n);
+            std::copy(vs.begin() + row, vs.begin() + row + n, pvs.begin() + h * n);
+        }
+        orc_gqa_decode(q.data() + b * Hq * D, pk.data(), pks.data(), pv.data(), pvs.data(), o_ref.data(), 1, Hq, Hkv, D, n,
+                       0, nullptr, nullptr, nullptr);
+        for (int64_t i = 0; i < Hq * D; ++i) good = good && std::fabs(att[b * Hq * D + i] - o_ref[i]) <= 2e-5f;
+    }
+    std::vector<float> ao = download(layer.ao, (size_t)(B * H)), h1 = download(layer.h1, (size_t)(B * H)),
+                       hn = download(layer.hn, (size_t)(B * H)), gu = download(layer.gu, (size_t)(B * 2 * I)),
+                       act = download(layer.act, (size_t)(B * I)), dn = download(layer.dn, (size_t)(B * H)),
+                       out = download(dout, (size_t)(B * H));
+    y.assign((size_t)(B * H), 0.0f);
+    orc_w8a8_linear(att.data(), ow.data(), os.data(), y.data(), B, H, Hq * D, 128, nullptr, nullptr, nullptr);
+    good = good && ao == y;
+    std::vector<float> hh((size_t)(B * H));
+    orc_rmsnorm(ao.data(), x.data(), g2.data(), 1e-5f, hh.data(), r.data(), B, H);
+    good = good && h1 == hh && close(hn, r, 2e-6f);
+    y.assign((size_t)(B * 2 * I), 0.0f);
+    orc_w8a8_linear(hn.data(), guw.data(), gus.data(), y.data(), B, 2 * I, H, 128, nullptr, nullptr, nullptr);
+    good = good && gu == y;
+    std::vector<float> a((size_t)(B * I));
+    orc_swiglu(gu.data(), a.data(), B, I);
+    good = good && close(act, a, 2e-6f);
+    y.assign((size_t)(B * H), 0.0f);
+    orc_w8a8_linear(act.data(), dw.data(), ds.data(), y.data(), B, H, I, 128, nullptr, nullptr, nullptr);
+    good = good && dn == y;
+    for (int64_t i = 0; i < B * H; ++i) good = good && out[i] == h1[i] + dn[i];
+    report("decoder_layer_vs_oracle", good);
+}
+
 int main()
 {
     Context ctx(0);
@@ -286,6 +391,7 @@ int main()
     test_quant_linear(ctx);
     test_decode_attention(ctx);
     test_kv_cache(ctx);
+    test_decoder_layer(ctx);
     std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;
 }
