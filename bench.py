@@ -220,6 +220,7 @@ def main():
         sub.update(decode_attention(mi, wl, dev, s, timer))
         sub.update(moe_layer(mi, wl, dev, s, timer))
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
+        sub.update(decode_layer_chain(mi, wl, dev, s, timer))
         sub.update(host_staging(mi, wl, dev, s, timer))
     out["sub_metrics"] = sub
     if not args.skip_cpu:
@@ -414,6 +415,54 @@ def cfg0_linear(mi, wl, dev, s, timer, shapes):
     return {"cfg0_linear_m32": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                 "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                 "TOPS": round(wl.gemm_ops(M, N, K) / (ms * 1e-3) / 1e12, 2)}}
+
+
+def decode_layer_chain(mi, wl, dev, s, timer, reps=10):
+    """A decode step through decoder layers of the cfg1 / cfg2 shapes (hidden 4096, 32/8 heads of 128, FFN 14336,
+    16 sequences with 4095 cached tokens each): three layers with their own weights (654 MB) and KV caches
+    (417 MB) run one after the other, so that nothing a layer reads is left in the memory-side cache from its
+    last turn; the three-layer step is recorded into a graph and replayed."""
+    c = wl.ATTN
+    B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
+    H, I = 4096, 14336
+    mark = dev.mark()
+    inv = 10000.0 ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
+    ang = np.arange(T, dtype=np.float64)[:, None] * inv[None, :]
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    g1 = np.ones(H, np.float32)
+    layers = []
+    for li in range(3):
+        w = [wl.weights(500 + li, n, k, i) for i, (n, k) in
+             enumerate((((Hq + 2 * Hkv) * D, H), (H, Hq * D), (2 * I, H), (H, I)))]
+        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, w[0], w[1], w[2], w[3], g1, g1, cos, sin)
+        del w
+        # a cache of real rows: rotate + quantize N(0,1) keys and values
+        m2 = dev.mark()
+        src = dev.upload(wl.normal(600 + li, (B * Hkv * T, D), 0))
+        mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.kq.ptr, L.ks.ptr, B * Hkv * T, D, D, s))
+        mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.vq.ptr, L.vs.ptr, B * Hkv * T, D, D, s))
+        dev.sync(s)
+        dev.reset_to(m2)
+        layers.append(L)
+    x = dev.upload(wl.activations(700, B, H))
+    out = dev.empty((B, H), np.float32)
+    dpos, dlen = dev.upload(np.full(B, T - 1, np.int32)), dev.upload(np.full(B, T, np.int32))
+
+    def step():
+        # inside the stack a layer's closing residual add is done by the next layer's first kernel
+        layers[0].step(x, dpos, dlen, T, None, s)
+        layers[1].step(layers[0].dn, dpos, dlen, T, None, s, residual=layers[0].h1)
+        layers[2].step(layers[1].dn, dpos, dlen, T, out, s, residual=layers[1].h1)
+    ms = graph_time(mi, dev, s, timer, [step], reps) / len(layers)
+    wbytes = ((Hq + 2 * Hkv) * D * H + H * Hq * D + 2 * I * H + H * I)
+    nbytes = wbytes + wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
+    dev.reset_to(mark)
+    return {"decode_layer_b16_t4096": {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 11,
+                                       "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                       "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1),
+                                       "tokens_per_s_32_layers": round(B / (32 * ms * 1e-3), 1),
+                                       "algorithmic_bytes": nbytes}}
 
 
 def host_staging(mi, wl, dev, s, timer):

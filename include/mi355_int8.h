@@ -277,6 +277,16 @@ MI_API int32_t mi_rope_kv_append_f32_i8(const float *qkv, int64_t row_stride, co
                                         int64_t T_cap, void *stream);
 /* h[m,n] = silu(gate_up[m,n]) * gate_up[m,I+n]; gate_up fp32 [M,2I] (one projection of N = 2I), h fp32 [M,I]. */
 MI_API int32_t mi_swiglu_f32(const float *gate_up, float *h, int64_t M, int64_t I, void *stream);
+/* The two row operators above fused with the rotate + quantize prologue (mi_fwht_quant_f32_i8) of the linear that
+ * consumes them: codes int8 [M,H] (resp. [M,I]) and scales fp32 [M] go straight to mi_w8a8_gemm_dequant_f32.
+ * The arithmetic per element is that of the separate calls in the same order (codes are bit-identical to
+ * quantizing the fp32 row the separate call writes).  y_out / h_out of the activated row are optional (NULL: the
+ * fp32 row is never written); with a residual, h_out (the sum) is required as above.  H, I % block == 0. */
+MI_API int32_t mi_rmsnorm_quant_f32_i8(const float *x, const float *residual, const float *g, float eps,
+                                       float *h_out, float *y_out, int8_t *q, float *scale,
+                                       int64_t M, int64_t H, int32_t block, void *stream);
+MI_API int32_t mi_swiglu_quant_f32_i8(const float *gate_up, float *h_out, int8_t *q, float *scale,
+                                      int64_t M, int64_t I, int32_t block, void *stream);
 /* out = a + b over n floats (n % 4 == 0): the residual add that closes the layer. */
 MI_API int32_t mi_add_f32(const float *a, const float *b, float *out, int64_t n, void *stream);
 

@@ -135,6 +135,133 @@ __global__ __launch_bounds__(256) void k_swiglu(const float *__restrict__ gu, fl
     *reinterpret_cast<float4 *>(h + i) = o;
 }
 
+// The row operators fused with the rotate + quantize prologue of the linear that follows them, so that a decode
+// step launches one kernel where it launched two and the normalized / activated row never travels as fp32 unless
+// the caller asks for it.  One workgroup per row, thread t owns chunks t, t + 256, ... (C of them) in the layout
+// of fwht_core.h; the arithmetic per element is that of the separate kernels in the same order.
+// MODE 0: v = ((x (+ res)) * r) * g (RMSNorm);  MODE 1: v = silu(gate) * up from a fused [gate | up] row.
+template <int BLOCK, int C, int MODE>
+__global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ x, const float *__restrict__ res,
+                                                      const float *__restrict__ g, float eps,
+                                                      float *__restrict__ h_out, float *__restrict__ y_out,
+                                                      int8_t *__restrict__ q, float *__restrict__ scale, int K)
+{
+    constexpr int LPB = BLOCK / 8;
+    __shared__ float s_part[4], s_max[4];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int j = t % LPB;
+    const int nchunk = K / 8;
+    const int64_t row = blockIdx.x;
+    float v[C][8];
+    int base[C];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int c = t + i * 256;
+        base[i] = (c / LPB) * BLOCK + 4 * j;
+        if (c < nchunk) {
+            if constexpr (MODE == 0) {
+                const float *xr = x + row * (int64_t)K + base[i];
+                float4 lo = *reinterpret_cast<const float4 *>(xr), hi = *reinterpret_cast<const float4 *>(xr + BLOCK / 2);
+                if (res) {
+                    const float *rr = res + row * (int64_t)K + base[i];
+                    const float4 rl = *reinterpret_cast<const float4 *>(rr), rh = *reinterpret_cast<const float4 *>(rr + BLOCK / 2);
+                    lo.x = lo.x + rl.x; lo.y = lo.y + rl.y; lo.z = lo.z + rl.z; lo.w = lo.w + rl.w;
+                    hi.x = hi.x + rh.x; hi.y = hi.y + rh.y; hi.z = hi.z + rh.z; hi.w = hi.w + rh.w;
+                    float *ho = h_out + row * (int64_t)K + base[i];
+                    *reinterpret_cast<float4 *>(ho) = lo;
+                    *reinterpret_cast<float4 *>(ho + BLOCK / 2) = hi;
+                }
+                v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+                v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+            } else {
+                const float *gr = x + row * 2 * (int64_t)K + base[i];
+                const float4 gl = *reinterpret_cast<const float4 *>(gr), gh = *reinterpret_cast<const float4 *>(gr + BLOCK / 2);
+                const float4 ul = *reinterpret_cast<const float4 *>(gr + K), uh = *reinterpret_cast<const float4 *>(gr + K + BLOCK / 2);
+                const float gg[8] = {gl.x, gl.y, gl.z, gl.w, gh.x, gh.y, gh.z, gh.w};
+                const float uu[8] = {ul.x, ul.y, ul.z, ul.w, uh.x, uh.y, uh.z, uh.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[i][e] = (gg[e] / (1.0f + expf(-gg[e]))) * uu[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+        }
+    }
+    if constexpr (MODE == 0) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (lane == 0) s_part[wave] = ss;
+        __syncthreads();
+        const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+        const float r = 1.0f / sqrtf(total / (float)K + eps);
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (t + i * 256 < nchunk) {
+                const float4 gl = *reinterpret_cast<const float4 *>(g + base[i]);
+                const float4 gh = *reinterpret_cast<const float4 *>(g + base[i] + BLOCK / 2);
+                v[i][0] = (v[i][0] * r) * gl.x; v[i][1] = (v[i][1] * r) * gl.y;
+                v[i][2] = (v[i][2] * r) * gl.z; v[i][3] = (v[i][3] * r) * gl.w;
+                v[i][4] = (v[i][4] * r) * gh.x; v[i][5] = (v[i][5] * r) * gh.y;
+                v[i][6] = (v[i][6] * r) * gh.z; v[i][7] = (v[i][7] * r) * gh.w;
+            }
+        }
+    }
+    if (y_out) {
+        float *yo = y_out + row * (int64_t)K;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (t + i * 256 < nchunk) {
+                *reinterpret_cast<float4 *>(yo + base[i]) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+                *reinterpret_cast<float4 *>(yo + base[i] + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        fwht_chunk<BLOCK>(v[i], j);
+        amax = fmaxf(amax, abs8(v[i]));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if (lane == 0) s_max[wave] = amax;
+    __syncthreads();
+    const float a = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+    const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+    if (t == 0) scale[row] = sc;
+    int8_t *qrow = q + row * (int64_t)K;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        if (t + i * 256 < nchunk) {
+            *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+            *reinterpret_cast<uint32_t *>(qrow + base[i] + BLOCK / 2) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+        }
+    }
+}
+
+template <int BLOCK, int MODE>
+static int32_t launch_row_op_quant(const float *x, const float *res, const float *g, float eps, float *h_out,
+                                   float *y_out, int8_t *q, float *scale, int64_t M, int64_t K, hipStream_t s)
+{
+    const int C = (int)((K / 8 + 255) / 256);
+    const dim3 grid((unsigned)M);
+#define MI_ROWQ(CC)                                                                                              \
+    hipLaunchKernelGGL((k_row_op_quant<BLOCK, CC, MODE>), grid, dim3(256), 0, s, x, res, g, eps, h_out, y_out, q, \
+                       scale, (int)K)
+    if (C <= 1) MI_ROWQ(1);
+    else if (C <= 2) MI_ROWQ(2);
+    else if (C <= 4) MI_ROWQ(4);
+    else if (C <= 7) MI_ROWQ(7);
+    else if (C <= 8) MI_ROWQ(8);
+    else return MI_ERANGE;
+#undef MI_ROWQ
+    return launch_status();
+}
+
 __global__ __launch_bounds__(256) void k_add(const float *__restrict__ a, const float *__restrict__ b,
                                              float *__restrict__ out, int64_t n)
 {
@@ -203,6 +330,34 @@ extern "C" int32_t mi_swiglu_f32(const float *gate_up, float *h, int64_t M, int6
     hipLaunchKernelGGL(layer::k_swiglu, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, as_stream(stream),
                        gate_up, h, M, (int)I);
     return launch_status();
+}
+
+extern "C" int32_t mi_rmsnorm_quant_f32_i8(const float *x, const float *residual, const float *g, float eps,
+                                           float *h_out, float *y_out, int8_t *q, float *scale, int64_t M,
+                                           int64_t H, int32_t block, void *stream)
+{
+    if (!x || !g || !q || !scale || M < 0 || H <= 0 || !(eps >= 0.0f)) return MI_EINVAL;
+    if (residual && !h_out) return MI_EINVAL;
+    if ((block != 128 && block != 256) || H % block) return MI_EINVAL;
+    if (H > 16384 || M > 0x7fffffffLL) return MI_ERANGE;
+    if (!aligned16(x) || !aligned16(g) || !aligned4(q) || !aligned4(scale) || (y_out && !aligned16(y_out)) ||
+        (residual && (!aligned16(residual) || !aligned16(h_out))))
+        return MI_EINVAL;
+    if (M == 0) return MI_OK;
+    return block == 128 ? layer::launch_row_op_quant<128, 0>(x, residual, g, eps, h_out, y_out, q, scale, M, H, as_stream(stream))
+                        : layer::launch_row_op_quant<256, 0>(x, residual, g, eps, h_out, y_out, q, scale, M, H, as_stream(stream));
+}
+
+extern "C" int32_t mi_swiglu_quant_f32_i8(const float *gate_up, float *h_out, int8_t *q, float *scale, int64_t M,
+                                          int64_t I, int32_t block, void *stream)
+{
+    if (!gate_up || !q || !scale || M < 0 || I <= 0) return MI_EINVAL;
+    if ((block != 128 && block != 256) || I % block) return MI_EINVAL;
+    if (I > 16384 || M > 0x7fffffffLL) return MI_ERANGE;
+    if (!aligned16(gate_up) || !aligned4(q) || !aligned4(scale) || (h_out && !aligned16(h_out))) return MI_EINVAL;
+    if (M == 0) return MI_OK;
+    return block == 128 ? layer::launch_row_op_quant<128, 1>(gate_up, nullptr, nullptr, 0.0f, nullptr, h_out, q, scale, M, I, as_stream(stream))
+                        : layer::launch_row_op_quant<256, 1>(gate_up, nullptr, nullptr, 0.0f, nullptr, h_out, q, scale, M, I, as_stream(stream));
 }
 
 extern "C" int32_t mi_add_f32(const float *a, const float *b, float *out, int64_t n, void *stream)

@@ -238,24 +238,30 @@ struct KvCache {
     }
 };
 
-// One decoder layer of a decode step (one new token per sequence), chained on one stream:
-// RMSNorm -> QKV -> rotary + cache append -> attention over the cache -> O -> residual + RMSNorm -> gate|up ->
-// SwiGLU -> down -> residual.  Holds its prepared weights, its KV cache and its scratch rows in the arena.
+// One decoder layer of a decode step (one new token per sequence), chained on one stream, eleven launches:
+// (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache -> O linear ->
+// residual + RMSNorm + quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
+// Holds its prepared weights, its KV cache and its scratch rows in the arena.
 struct DecoderLayer {
     int64_t B = 0, H = 0, Hq = 0, Hkv = 0, I = 0, T_cap = 0;
     float eps = 1e-5f;
     QuantLinear<128> qkv, o, gate_up, down;
     KvCache cache;
     const float *g1 = nullptr, *g2 = nullptr, *rope_cos = nullptr, *rope_sin = nullptr;
-    float *xn = nullptr, *qkv_out = nullptr, *q = nullptr, *att = nullptr, *ao = nullptr, *h1 = nullptr, *hn = nullptr,
-          *gu = nullptr, *act = nullptr, *dn = nullptr;
+    // fp32 rows: layer input when it is a sum (h0), projections, attention output, residual stream after
+    // attention (h1), down output (dn); xn / hn / act only when prepare() was asked to trace
+    float *h0 = nullptr, *qkv_out = nullptr, *q = nullptr, *att = nullptr, *ao = nullptr, *h1 = nullptr, *gu = nullptr,
+          *dn = nullptr, *xn = nullptr, *hn = nullptr, *act = nullptr;
+    int8_t *cx = nullptr, *ci = nullptr;   // codes of the normalized rows [B,H] and of the activated rows [B,I]
+    float *sx = nullptr, *si = nullptr;
 
     // fp32 weights in device memory: wqkv [(Hq+2Hkv)*128, H], wo [H, Hq*128], wgu [2I, H] (gate rows, then up
     // rows), wd [H, I]; norm weights g1, g2 [H]; rotary tables [T_cap, 64].  false if the arena is exhausted.
     template <typename Arena>
     bool prepare(Arena &arena, int64_t b, int64_t h, int64_t hq, int64_t hkv, int64_t i, int64_t t_cap,
                  const float *wqkv, const float *wo, const float *wgu, const float *wd, const float *norm1,
-                 const float *norm2, const float *cos_table, const float *sin_table, float epsilon, void *stream)
+                 const float *norm2, const float *cos_table, const float *sin_table, float epsilon, void *stream,
+                 bool trace = false)
     {
         B = b; H = h; Hq = hq; Hkv = hkv; I = i; T_cap = t_cap; eps = epsilon;
         g1 = norm1; g2 = norm2; rope_cos = cos_table; rope_sin = sin_table;
@@ -263,34 +269,46 @@ struct DecoderLayer {
         bool ok = qkv.prepare(arena, wqkv, nqkv, H, B, stream) && o.prepare(arena, wo, H, Hq * 128, B, stream) &&
                   gate_up.prepare(arena, wgu, 2 * I, H, B, stream) && down.prepare(arena, wd, H, I, B, stream) &&
                   cache.prepare(arena, B, Hq, Hkv, T_cap);
-        xn = arena.template alloc<float>(B * H);
+        h0 = arena.template alloc<float>(B * H);
         qkv_out = arena.template alloc<float>(B * nqkv);
         q = arena.template alloc<float>(B * Hq * 128);
         att = arena.template alloc<float>(B * Hq * 128);
         ao = arena.template alloc<float>(B * H);
         h1 = arena.template alloc<float>(B * H);
-        hn = arena.template alloc<float>(B * H);
         gu = arena.template alloc<float>(B * 2 * I);
-        act = arena.template alloc<float>(B * I);
         dn = arena.template alloc<float>(B * H);
-        return ok && xn && qkv_out && q && att && ao && h1 && hn && gu && act && dn;
+        cx = arena.template alloc<int8_t>(B * H);
+        ci = arena.template alloc<int8_t>(B * I);
+        sx = arena.template alloc<float>(B);
+        si = arena.template alloc<float>(B);
+        if (trace) {
+            xn = arena.template alloc<float>(B * H);
+            hn = arena.template alloc<float>(B * H);
+            act = arena.template alloc<float>(B * I);
+            ok = ok && xn && hn && act;
+        }
+        return ok && h0 && qkv_out && q && att && ao && h1 && gu && dn && cx && ci && sx && si;
     }
-    // x, out fp32 [B,H]; pos, seq_len int32 [B] in device memory (seq_len = pos + 1 in a plain decode step);
-    // t_max bounds seq_len.  The first failing call's status is returned.
-    int32_t step(const float *x, const int32_t *pos, const int32_t *seq_len, int64_t t_max, float *out, void *stream) const
+    // x fp32 [B,H], plus residual fp32 [B,H] or nullptr: the layer input is their sum (left in h0).  pos, seq_len
+    // int32 [B] in device memory (seq_len = pos + 1 in a plain decode step); t_max bounds seq_len.  out fp32 [B,H],
+    // or nullptr: the closing residual add is left to the next layer (give it x = dn, residual = h1).
+    // The first failing call's status is returned.
+    int32_t step(const float *x, const float *residual, const int32_t *pos, const int32_t *seq_len, int64_t t_max,
+                 float *out, void *stream) const
     {
-        int32_t rc = mi_rmsnorm_f32(x, nullptr, g1, eps, nullptr, xn, B, H, stream);
-        if (rc == MI_OK) rc = qkv.forward(xn, qkv_out, B, stream);
+        int32_t rc = mi_rmsnorm_quant_f32_i8(x, residual, g1, eps, residual ? h0 : nullptr, xn, cx, sx, B, H, 128, stream);
+        const float *xin = residual ? h0 : x;
+        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(cx, sx, qkv.qw, qkv.sw, qkv_out, B, qkv.N, H, stream);
         if (rc == MI_OK)
             rc = mi_rope_kv_append_f32_i8(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, cache.kq, cache.ks,
                                           cache.vq, cache.vs, pos, B, Hq, Hkv, 128, T_cap, stream);
         if (rc == MI_OK) rc = cache.attend(q, att, seq_len, t_max, false, stream);
         if (rc == MI_OK) rc = o.forward(att, ao, B, stream);
-        if (rc == MI_OK) rc = mi_rmsnorm_f32(ao, x, g2, eps, h1, hn, B, H, stream);
-        if (rc == MI_OK) rc = gate_up.forward(hn, gu, B, stream);
-        if (rc == MI_OK) rc = mi_swiglu_f32(gu, act, B, I, stream);
-        if (rc == MI_OK) rc = down.forward(act, dn, B, stream);
-        if (rc == MI_OK) rc = mi_add_f32(h1, dn, out, B * H, stream);
+        if (rc == MI_OK) rc = mi_rmsnorm_quant_f32_i8(ao, xin, g2, eps, h1, hn, cx, sx, B, H, 128, stream);
+        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(cx, sx, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, stream);
+        if (rc == MI_OK) rc = mi_swiglu_quant_f32_i8(gu, act, ci, si, B, I, 128, stream);
+        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ci, si, down.qw, down.sw, dn, B, H, I, stream);
+        if (rc == MI_OK && out) rc = mi_add_f32(h1, dn, out, B * H, stream);
         return rc;
     }
 };

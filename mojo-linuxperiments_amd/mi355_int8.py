@@ -92,6 +92,8 @@ SIGNATURES = {
     "mi_rmsnorm_f32": (i32, [vp, vp, vp, C.c_float, vp, vp, i64, i64, vp]),
     "mi_rope_kv_append_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
     "mi_swiglu_f32": (i32, [vp, vp, i64, i64, vp]),
+    "mi_rmsnorm_quant_f32_i8": (i32, [vp, vp, vp, C.c_float, vp, vp, vp, vp, i64, i64, i32, vp]),
+    "mi_swiglu_quant_f32_i8": (i32, [vp, vp, vp, vp, i64, i64, i32, vp]),
     "mi_add_f32": (i32, [vp, vp, vp, i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
@@ -372,19 +374,20 @@ def moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=None):
 
 class DecoderLayer:
     """One decoder layer of a decode step, chained from the C-ABI entry points on one stream:
-    RMSNorm -> QKV linear -> rotary + KV-cache append -> attention over the cache -> O linear -> residual +
-    RMSNorm -> gate|up linear -> SwiGLU -> down linear -> residual.  Test and bench plumbing over the same calls
-    the C++ host struct of the same name makes (host/mi355_host.hpp)."""
+    (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + KV-cache append -> attention over the cache ->
+    O linear -> residual + RMSNorm + quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
+    Eleven launches.  Test and bench plumbing over the same calls the C++ host struct of the same name makes
+    (host/mi355_host.hpp).  trace=True also writes the fp32 rows the fused kernels normally keep in registers
+    (xn, hn, act) so that a test can gate every stage."""
 
     def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
-                 block=128):
+                 block=128, trace=False):
         D = 128
         self.dev, self.B, self.H, self.Hq, self.Hkv, self.I, self.T_cap, self.eps, self.block = \
             dev, B, H, Hq, Hkv, I, T_cap, eps, block
         self.NQKV = (Hq + 2 * Hkv) * D
 
         def prep(w):
-            mark = dev.mark()
             N, K = w.shape
             q, s = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
             keep = dev.mark()
@@ -392,7 +395,6 @@ class DecoderLayer:
             fwht_quant(dw, q, s, block)
             dev.sync()
             dev.reset_to(keep)
-            del mark
             return q, s
         self.wqkv, self.wo, self.wgu, self.wd = prep(wqkv), prep(wo), prep(wgu), prep(wd)
         self.g1, self.g2 = dev.upload(g1), dev.upload(g2)
@@ -400,20 +402,29 @@ class DecoderLayer:
         self.kq, self.ks = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
         self.vq, self.vs = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
         f = np.float32
-        self.xn, self.qkv = dev.empty((B, H), f), dev.empty((B, self.NQKV), f)
+        self.h0, self.qkv = dev.empty((B, H), f), dev.empty((B, self.NQKV), f)
         self.q, self.att = dev.empty((B, Hq, D), f), dev.empty((B, Hq * D), f)
-        self.ao, self.h1, self.hn = dev.empty((B, H), f), dev.empty((B, H), f), dev.empty((B, H), f)
-        self.gu, self.act, self.dn = dev.empty((B, 2 * I), f), dev.empty((B, I), f), dev.empty((B, H), f)
-        nws = max(lib.mi_w8a8_linear_workspace_bytes(B, n, k) for n, k in
-                  ((self.NQKV, H), (H, Hq * D), (2 * I, H), (H, I)))
-        self.lin_ws = dev.empty(nws, np.uint8)
+        self.ao, self.h1 = dev.empty((B, H), f), dev.empty((B, H), f)
+        self.gu, self.dn = dev.empty((B, 2 * I), f), dev.empty((B, H), f)
+        self.xn = dev.empty((B, H), f) if trace else None
+        self.hn = dev.empty((B, H), f) if trace else None
+        self.act = dev.empty((B, I), f) if trace else None
+        self.cx, self.sx = dev.empty((B, H), np.int8), dev.empty(B, f)        # codes of the normalized rows
+        self.ci, self.si = dev.empty((B, I), np.int8), dev.empty(B, f)        # codes of the activated rows
+        self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, H, Hq * D), np.uint8)
         self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
 
-    def step(self, x, pos, seq_len, t_max, out, stream=None):
-        """x, out fp32 [B,H]; pos, seq_len int32 [B] on the device (seq_len = pos + 1 for a plain decode step)."""
+    def step(self, x, pos, seq_len, t_max, out, stream=None, residual=None):
+        """x fp32 [B,H] (+ residual fp32 [B,H]: the layer input is their sum, left in self.h0); pos, seq_len int32
+        [B] on the device (seq_len = pos + 1 for a plain decode step).  out fp32 [B,H], or None: the closing
+        residual add is left to the next layer (pass x=self.dn, residual=self.h1 to its step)."""
         B, H, Hq, Hkv, I, D, s = self.B, self.H, self.Hq, self.Hkv, self.I, 128, stream
-        check(lib.mi_rmsnorm_f32(x.ptr, None, self.g1.ptr, self.eps, None, self.xn.ptr, B, H, s), "mi_rmsnorm_f32")
-        linear(self.xn, self.wqkv[0], self.wqkv[1], self.qkv, self.block, self.lin_ws, s)
+        p = lambda b: b.ptr if b is not None else None
+        check(lib.mi_rmsnorm_quant_f32_i8(x.ptr, p(residual), self.g1.ptr, self.eps,
+                                          self.h0.ptr if residual is not None else None, p(self.xn), self.cx.ptr,
+                                          self.sx.ptr, B, H, self.block, s), "mi_rmsnorm_quant_f32_i8")
+        xin = self.h0 if residual is not None else x
+        gemm_dequant(self.cx, self.sx, self.wqkv[0], self.wqkv[1], self.qkv, s)
         check(lib.mi_rope_kv_append_f32_i8(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr,
                                            self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv,
                                            D, self.T_cap, s), "mi_rope_kv_append_f32_i8")
@@ -421,9 +432,11 @@ class DecoderLayer:
                                            self.att.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, 0,
                                            self.att_ws.ptr, self.att_ws.nbytes, s), "mi_gqa_decode_attn_cache")
         linear(self.att, self.wo[0], self.wo[1], self.ao, self.block, self.lin_ws, s)
-        check(lib.mi_rmsnorm_f32(self.ao.ptr, x.ptr, self.g2.ptr, self.eps, self.h1.ptr, self.hn.ptr, B, H, s),
-              "mi_rmsnorm_f32")
-        linear(self.hn, self.wgu[0], self.wgu[1], self.gu, self.block, self.lin_ws, s)
-        check(lib.mi_swiglu_f32(self.gu.ptr, self.act.ptr, B, I, s), "mi_swiglu_f32")
-        linear(self.act, self.wd[0], self.wd[1], self.dn, self.block, self.lin_ws, s)
-        check(lib.mi_add_f32(self.h1.ptr, self.dn.ptr, out.ptr, B * H, s), "mi_add_f32")
+        check(lib.mi_rmsnorm_quant_f32_i8(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
+                                          self.cx.ptr, self.sx.ptr, B, H, self.block, s), "mi_rmsnorm_quant_f32_i8")
+        gemm_dequant(self.cx, self.sx, self.wgu[0], self.wgu[1], self.gu, s)
+        check(lib.mi_swiglu_quant_f32_i8(self.gu.ptr, p(self.act), self.ci.ptr, self.si.ptr, B, I, self.block, s),
+              "mi_swiglu_quant_f32_i8")
+        gemm_dequant(self.ci, self.si, self.wd[0], self.wd[1], self.dn, s)
+        if out is not None:
+            check(lib.mi_add_f32(self.h1.ptr, self.dn.ptr, out.ptr, B * H, s), "mi_add_f32")

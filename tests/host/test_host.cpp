@@ -301,11 +301,11 @@ static void test_decoder_layer(const Context &ctx)
     DecoderLayer layer;
     bool ok = layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, upload(arena, wqkv), upload(arena, wo), upload(arena, wgu),
                             upload(arena, wd), upload(arena, g1), upload(arena, g2), upload(arena, cs), upload(arena, sn),
-                            1e-5f, nullptr);
+                            1e-5f, nullptr, true);
     const std::vector<int32_t> pos = {0, 9}, len = {1, 10};
     int32_t *dpos = upload(arena, pos), *dlen = upload(arena, len);
     float *dx = upload(arena, x), *dout = arena.alloc<float>(B * H);
-    ok = ok && dpos && dlen && dx && dout && layer.step(dx, dpos, dlen, 10, dout, nullptr) == MI_OK;
+    ok = ok && dpos && dlen && dx && dout && layer.step(dx, nullptr, dpos, dlen, 10, dout, nullptr) == MI_OK;
     if (!ok) { report("decoder_layer_vs_oracle", false, "set-up or launch failed"); return; }
     auto close = [](const std::vector<float> &a, const std::vector<float> &b, float tol) {
         float m = 0, d = 0;

@@ -175,7 +175,8 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
     g = np.random.default_rng(41)
     g1 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
     g2 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
-    layer = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T_cap, fw["qkv"], fw["o"], fw["gu"], fw["d"], g1, g2, cos, sin, eps)
+    layer = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T_cap, fw["qkv"], fw["o"], fw["gu"], fw["d"], g1, g2, cos, sin, eps,
+                            trace=True)
     W = {k: orc.rotate_quant_rows(v, 128) for k, v in fw.items()}
     for k, dv in (("qkv", layer.wqkv), ("o", layer.wo), ("gu", layer.wgu), ("d", layer.wd)):
         assert np.array_equal(dev.download(dv[0]), W[k][0]) and np.array_equal(dev.download(dv[1]), W[k][1])
@@ -209,4 +210,67 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
         # five quantizers in a row (measured 2e-4 .. 6e-3)
         want = oracle_layer(orc, x, W, free, pos, lens, cos, sin, eps, Hq, Hkv)
         assert rel(out, want) <= 3e-2, "step %d rel-L2 %.3e" % (step, rel(out, want))
+    # the layer fed as the next layer of a stack is fed: input = down output + residual of the layer before, the
+    # closing add left to the layer after (out=None); positions that do not collide with the steps above
+    prev_dn, prev_h1 = dev.download(layer.dn), dev.download(layer.h1)
+    d_dn, d_h1 = dev.upload(prev_dn), dev.upload(prev_h1)
+    pos = np.minimum(start + 3, T_cap - 1).astype(np.int32)
+    lens = (pos + 1).astype(np.int32)
+    for d, a in ((dpos, pos), (dlen, lens)):
+        mi.check(mi.lib.mi_memcpy_h2d(d.ptr, a.ctypes.data, a.nbytes, None))
+    layer.step(d_dn, dpos, dlen, int(lens.max()), None, residual=d_h1)
+    gpu = {n: dev.download(getattr(layer, n)) for n in names}
+    gpu["q"] = gpu["q"].reshape(B, Hq, D)
+    x_in = prev_dn + prev_h1
+    assert np.array_equal(dev.download(layer.h0), x_in)
+    staged = oracle_layer(orc, x_in, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=gpu)
+    assert np.array_equal(gpu["h1"] + gpu["dn"], staged)
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("M,H,block", [(16, 4096, 128), (3, 14336, 128), (2, 768, 256), (1, 128, 128), (5, 16384, 256)])
+def test_fused_rmsnorm_quant_equals_the_two_calls(mi, dev, orc, M, H, block):
+    """Codes and scales of the fused kernel = the stand-alone quantizer applied to the fp32 row the fused kernel
+    reports, and that row follows the RMSNorm oracle; the residual sum is one fp32 add."""
+    mark = dev.mark()
+    g = np.random.default_rng(M + H)
+    x = workload.activations(61, M, H)
+    r = g.standard_normal((M, H)).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
+    dx, dr, dw = dev.upload(x), dev.upload(r), dev.upload(w)
+    dh, dy = dev.empty((M, H), np.float32), dev.empty((M, H), np.float32)
+    dq, ds = dev.empty((M, H), np.int8), dev.empty(M, np.float32)
+    for res in (None, dr):
+        mi.check(mi.lib.mi_rmsnorm_quant_f32_i8(dx.ptr, res.ptr if res else None, dw.ptr, 1e-5,
+                                                dh.ptr if res else None, dy.ptr, dq.ptr, ds.ptr, M, H, block, None))
+        y, q, sc = dev.download(dy), dev.download(dq), dev.download(ds)
+        xin = x + r if res else x
+        if res:
+            assert np.array_equal(dev.download(dh), xin)
+        want = orc.rmsnorm(xin, w, 1e-5)
+        assert np.max(np.abs(y - want)) <= 2e-6 * np.max(np.abs(want))
+        qo, so = orc.rotate_quant_rows(y, block)
+        assert np.array_equal(q, qo) and np.array_equal(sc, so)
+        # without the fp32 row: same codes
+        mi.check(mi.lib.mi_rmsnorm_quant_f32_i8(dx.ptr, res.ptr if res else None, dw.ptr, 1e-5,
+                                                dh.ptr if res else None, None, dq.ptr, ds.ptr, M, H, block, None))
+        assert np.array_equal(dev.download(dq), qo) and np.array_equal(dev.download(ds), so)
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("M,I,block", [(16, 14336, 128), (4, 768, 256), (1, 256, 128)])
+def test_fused_swiglu_quant_equals_the_two_calls(mi, dev, orc, M, I, block):
+    mark = dev.mark()
+    gu = (workload.normal(29, (M, 2 * I), 0) * 2).astype(np.float32)
+    dgu, dh = dev.upload(gu), dev.empty((M, I), np.float32)
+    dq, ds = dev.empty((M, I), np.int8), dev.empty(M, np.float32)
+    mi.check(mi.lib.mi_swiglu_quant_f32_i8(dgu.ptr, dh.ptr, dq.ptr, ds.ptr, M, I, block, None))
+    h, q, sc = dev.download(dh), dev.download(dq), dev.download(ds)
+    want = orc.swiglu(gu)
+    assert np.max(np.abs(h - want)) <= 2e-6 * max(1.0, float(np.max(np.abs(want))))
+    qo, so = orc.rotate_quant_rows(h, block)
+    assert np.array_equal(q, qo) and np.array_equal(sc, so)
+    mi.check(mi.lib.mi_swiglu_quant_f32_i8(dgu.ptr, None, dq.ptr, ds.ptr, M, I, block, None))
+    assert np.array_equal(dev.download(dq), qo) and np.array_equal(dev.download(ds), so)
+    assert mi.lib.mi_swiglu_quant_f32_i8(dgu.ptr, None, dq.ptr, ds.ptr, M, I + 4, block, None) == mi.EINVAL
     dev.reset_to(mark)
