@@ -201,6 +201,17 @@ MI_API int32_t mi_gqa_decode_attn_cache(const float *q, const int8_t *kq, const 
                                         int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                                         const int32_t *seq_len, int64_t T_max, int32_t out_rotated,
                                         void *workspace, int64_t workspace_bytes, void *stream);
+/* The same, with the merge of the splits fused with the int8 row quantizer of the output projection: per token the
+ * Hq*D attention outputs are left in the rotated basis of V (block D) and quantized as one row, oq int8 [B,Hq*D] and
+ * oscale fp32 [B], ready for mi_w8a8_gemm_dequant_f32 against output-projection weights that were prepared with
+ * block D along K (x.H . (W.H)^T = x . W^T): neither the inverse rotation nor the projection's own rotation is
+ * spent.  o_rot (optional, fp32 [B,Hq,D]) receives the row that was quantized.  Hq <= 64. */
+MI_API int32_t mi_gqa_decode_attn_cache_quant_i8(const float *q, const int8_t *kq, const float *ks,
+                                                 const int8_t *vq, const float *vs, float *o_rot,
+                                                 int8_t *oq, float *oscale,
+                                                 int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                                 const int32_t *seq_len, int64_t T_max,
+                                                 void *workspace, int64_t workspace_bytes, void *stream);
 /* a7 as the decode loop uses it: rotate (block 128 = D) and quantize the new token's key and value heads and
  * write codes and scale at token pos[b] of sequence b (int32 [B] in device memory; a sequence whose position is
  * outside [0, T_cap) is skipped).  Head h of sequence b is read at k_new + b*row_stride + h*D (floats), so

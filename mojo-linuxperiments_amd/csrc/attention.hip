@@ -394,23 +394,18 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     else gqa_split_body<DUMP, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
 }
 
-// merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row.  SP > 0: the split count is known at
-// compile time and every load of the row goes out before the first use (one memory round trip).
+// Merge of the splits of one (b, h) row by the 16 lanes that own it (lane j: elements 4j..4j+3 and 64+4j..).
+// SP > 0: the split count is known at compile time and every load of the row goes out before the first use (one
+// memory round trip).  Returns the normalized row in the rotated basis of V.
 template <int SP>
-__global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ part_o,
-                                                   const float *__restrict__ part_ml, float *__restrict__ o,
-                                                   int rows, int Hq, int Hkv, int G, int splits_rt, int out_rotated)
+__device__ __forceinline__ void merge_row(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                          int splits_rt, int64_t bkv, int hl, int j, float (&v)[8])
 {
     const int splits = SP > 0 ? SP : splits_rt;
-    const int tid = threadIdx.x, j = tid & 15;
-    const int row = blockIdx.x * 16 + (tid >> 4);
-    const bool live = row < rows;
-    const int rr = live ? row : rows - 1;
-    const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
-    const int64_t bkv = (int64_t)b * Hkv + kvh;
     const float *ml0 = part_ml + bkv * splits * 8;
     const float *po0 = part_o + (bkv * splits * 4 + hl) * attn::D;
-    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
     float l = 0.0f;
     if constexpr (SP > 0) {
         float ms[SP], ls[SP];
@@ -452,11 +447,66 @@ __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ par
     const float rl = l > 0.0f ? 1.0f / l : 0.0f;   // a sequence of length 0 gives a row of zeros
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] *= rl;
+}
+
+// merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row
+template <int SP>
+__global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ part_o,
+                                                   const float *__restrict__ part_ml, float *__restrict__ o,
+                                                   int rows, int Hq, int Hkv, int G, int splits_rt, int out_rotated)
+{
+    const int tid = threadIdx.x, j = tid & 15;
+    const int row = blockIdx.x * 16 + (tid >> 4);
+    const bool live = row < rows;
+    const int rr = live ? row : rows - 1;
+    const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
+    const int64_t bkv = (int64_t)b * Hkv + kvh;
+    float v[8];
+    merge_row<SP>(part_o, part_ml, splits_rt, bkv, hl, j, v);
     if (!out_rotated) fwht128(v, j);  // whole workgroup takes the same branch
     if (live) {
         float *orow = o + (int64_t)row * attn::D;
         *reinterpret_cast<float4 *>(orow + 4 * j) = make_float4(v[0], v[1], v[2], v[3]);
         *reinterpret_cast<float4 *>(orow + 64 + 4 * j) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
+// The merge of one token's Hq rows by one workgroup (16 lanes per head), followed by the int8 row quantizer over the
+// token's Hq*128 values as they stand in the rotated basis of V: the codes and the scale are what the output
+// projection's GEMV consumes when its weights were rotated along K with block 128 (x.H . (W.H)^T = x . W^T), so no
+// inverse rotation and no second rotation are spent.  o_rot (optional) receives the fp32 row.
+template <int SP>
+__global__ __launch_bounds__(1024) void k_gqa_merge_quant(const float *__restrict__ part_o,
+                                                          const float *__restrict__ part_ml,
+                                                          float *__restrict__ o_rot, int8_t *__restrict__ oq,
+                                                          float *__restrict__ oscale, int Hq, int Hkv, int G,
+                                                          int splits_rt)
+{
+    __shared__ float s_max[16];
+    const int tid = threadIdx.x, j = tid & 15, lane = tid & 63, wave = tid >> 6;
+    const int b = blockIdx.x, h = tid >> 4;
+    const int kvh = h / G, hl = h % G;
+    float v[8];
+    merge_row<SP>(part_o, part_ml, splits_rt, (int64_t)b * Hkv + kvh, hl, j, v);
+    float a = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a = fmaxf(a, fabsf(v[e]));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
+    if (lane == 0) s_max[wave] = a;
+    __syncthreads();
+    const int nwave = (int)(blockDim.x >> 6);
+    a = s_max[0];
+    for (int w = 1; w < nwave; ++w) a = fmaxf(a, s_max[w]);
+    const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
+    const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
+    const int64_t off = ((int64_t)b * Hq + h) * attn::D;
+    if (tid == 0) oscale[b] = sc;
+    *reinterpret_cast<uint32_t *>(oq + off + 4 * j) = quant4(v[0], v[1], v[2], v[3], inv);
+    *reinterpret_cast<uint32_t *>(oq + off + 64 + 4 * j) = quant4(v[4], v[5], v[6], v[7], inv);
+    if (o_rot) {
+        *reinterpret_cast<float4 *>(o_rot + off + 4 * j) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(o_rot + off + 64 + 4 * j) = make_float4(v[4], v[5], v[6], v[7]);
     }
 }
 
@@ -499,7 +549,8 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
 static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const int8_t *vq, const float *vs,
                         float *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T, int32_t out_rotated,
                         void *workspace, int64_t workspace_bytes, int8_t *dqq, float *dsq, int32_t *ddots,
-                        hipStream_t s, int64_t Tstride = 0, const int32_t *seq_len = nullptr)
+                        hipStream_t s, int64_t Tstride = 0, const int32_t *seq_len = nullptr, int8_t *oq = nullptr,
+                        float *oscale = nullptr)
 {
     int32_t rc = check_attn(B, Hq, Hkv, D, T);
     if (rc) return rc;
@@ -524,7 +575,24 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     if (ddots) hipLaunchKernelGGL(attn::k_gqa_split<true>, grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL(attn::k_gqa_split<false>, grid, dim3(256), 0, s, p);
     rc = launch_status();
-    if (rc || !o) return rc;
+    if (rc) return rc;
+    if (oq) {
+        // one workgroup per token merges its Hq rows and quantizes them for the output projection
+#define MI_MERGEQ(SP)                                                                                              \
+    hipLaunchKernelGGL(attn::k_gqa_merge_quant<SP>, dim3((unsigned)B), dim3((unsigned)(Hq * 16)), 0, s, p.part_o, \
+                       p.part_ml, o, oq, oscale, (int)Hq, (int)Hkv, p.G, splits)
+        switch (splits) {
+        case 1: MI_MERGEQ(1); break;
+        case 2: MI_MERGEQ(2); break;
+        case 4: MI_MERGEQ(4); break;
+        case 6: MI_MERGEQ(6); break;
+        case 8: MI_MERGEQ(8); break;
+        default: MI_MERGEQ(0); break;
+        }
+#undef MI_MERGEQ
+        return launch_status();
+    }
+    if (!o) return rc;
     const int rows = (int)(B * Hq);
     const dim3 mgrid((unsigned)((rows + 15) / 16));
 #define MI_MERGE(SP)                                                                                        \
@@ -563,6 +631,20 @@ extern "C" int32_t mi_gqa_decode_attn_cache(const float *q, const int8_t *kq, co
     if (T_cap > (1LL << 24)) return MI_ERANGE;
     return run_attn(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_max, out_rotated, workspace, workspace_bytes, nullptr,
                     nullptr, nullptr, as_stream(stream), T_cap, seq_len);
+}
+
+extern "C" int32_t mi_gqa_decode_attn_cache_quant_i8(const float *q, const int8_t *kq, const float *ks,
+                                                     const int8_t *vq, const float *vs, float *o_rot, int8_t *oq,
+                                                     float *oscale, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                                     int64_t T_cap, const int32_t *seq_len, int64_t T_max,
+                                                     void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!oq || !oscale || !aligned4(oq) || !aligned4(oscale) || (o_rot && !aligned16(o_rot))) return MI_EINVAL;
+    if (!seq_len || !aligned4(seq_len)) return MI_EINVAL;
+    if (T_cap <= 0 || T_max <= 0 || T_max > T_cap) return MI_EINVAL;
+    if (T_cap > (1LL << 24) || Hq > 64) return MI_ERANGE;
+    return run_attn(q, kq, ks, vq, vs, o_rot, B, Hq, Hkv, D, T_max, 1, workspace, workspace_bytes, nullptr, nullptr,
+                    nullptr, as_stream(stream), T_cap, seq_len, oq, oscale);
 }
 
 extern "C" int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const float *ks, const int8_t *vq,

@@ -137,17 +137,18 @@ __global__ __launch_bounds__(256) void k_swiglu(const float *__restrict__ gu, fl
 
 // The row operators fused with the rotate + quantize prologue of the linear that follows them, so that a decode
 // step launches one kernel where it launched two and the normalized / activated row never travels as fp32 unless
-// the caller asks for it.  One workgroup per row, thread t owns chunks t, t + 256, ... (C of them) in the layout
+// the caller asks for it.  One workgroup per row, thread t owns chunks t, t + TPB, ... (C of them) in the layout
 // of fwht_core.h; the arithmetic per element is that of the separate kernels in the same order.
 // MODE 0: v = ((x (+ res)) * r) * g (RMSNorm);  MODE 1: v = silu(gate) * up from a fused [gate | up] row.
-template <int BLOCK, int C, int MODE>
-__global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ x, const float *__restrict__ res,
+template <int BLOCK, int C, int MODE, int TPB>
+__global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ x, const float *__restrict__ res,
                                                       const float *__restrict__ g, float eps,
                                                       float *__restrict__ h_out, float *__restrict__ y_out,
                                                       int8_t *__restrict__ q, float *__restrict__ scale, int K)
 {
     constexpr int LPB = BLOCK / 8;
-    __shared__ float s_part[4], s_max[4];
+    constexpr int NW = TPB / 64;
+    __shared__ float s_part[NW], s_max[NW];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int j = t % LPB;
     const int nchunk = K / 8;
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ 
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < C; ++i) {
-        const int c = t + i * 256;
+        const int c = t + i * TPB;
         base[i] = (c / LPB) * BLOCK + 4 * j;
         if (c < nchunk) {
             if constexpr (MODE == 0) {
@@ -195,11 +196,19 @@ __global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ 
         for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
         if (lane == 0) s_part[wave] = ss;
         __syncthreads();
-        const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+        // pairwise over the waves' partial sums (a fixed order)
+        float part[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) part[w] = s_part[w];
+#pragma unroll
+        for (int n = NW; n > 1; n >>= 1)
+#pragma unroll
+            for (int w = 0; w < n / 2; ++w) part[w] = part[2 * w] + part[2 * w + 1];
+        const float total = part[0];
         const float r = 1.0f / sqrtf(total / (float)K + eps);
 #pragma unroll
         for (int i = 0; i < C; ++i) {
-            if (t + i * 256 < nchunk) {
+            if (t + i * TPB < nchunk) {
                 const float4 gl = *reinterpret_cast<const float4 *>(g + base[i]);
                 const float4 gh = *reinterpret_cast<const float4 *>(g + base[i] + BLOCK / 2);
                 v[i][0] = (v[i][0] * r) * gl.x; v[i][1] = (v[i][1] * r) * gl.y;
@@ -213,7 +222,7 @@ __global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ 
         float *yo = y_out + row * (int64_t)K;
 #pragma unroll
         for (int i = 0; i < C; ++i) {
-            if (t + i * 256 < nchunk) {
+            if (t + i * TPB < nchunk) {
                 *reinterpret_cast<float4 *>(yo + base[i]) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
                 *reinterpret_cast<float4 *>(yo + base[i] + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
             }
@@ -229,14 +238,16 @@ __global__ __launch_bounds__(256) void k_row_op_quant(const float *__restrict__ 
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) s_max[wave] = amax;
     __syncthreads();
-    const float a = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    float a = s_max[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) a = fmaxf(a, s_max[w]);
     const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
     const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
     if (t == 0) scale[row] = sc;
     int8_t *qrow = q + row * (int64_t)K;
 #pragma unroll
     for (int i = 0; i < C; ++i) {
-        if (t + i * 256 < nchunk) {
+        if (t + i * TPB < nchunk) {
             *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
             *reinterpret_cast<uint32_t *>(qrow + base[i] + BLOCK / 2) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
         }
@@ -247,16 +258,16 @@ template <int BLOCK, int MODE>
 static int32_t launch_row_op_quant(const float *x, const float *res, const float *g, float eps, float *h_out,
                                    float *y_out, int8_t *q, float *scale, int64_t M, int64_t K, hipStream_t s)
 {
-    const int C = (int)((K / 8 + 255) / 256);
+    // few rows (a decode step): a row is worth a whole compute unit, 1024 threads hold at most two chunks each
+    const int64_t nchunk = K / 8;
     const dim3 grid((unsigned)M);
-#define MI_ROWQ(CC)                                                                                              \
-    hipLaunchKernelGGL((k_row_op_quant<BLOCK, CC, MODE>), grid, dim3(256), 0, s, x, res, g, eps, h_out, y_out, q, \
+#define MI_ROWQ(CC, TT)                                                                                           \
+    hipLaunchKernelGGL((k_row_op_quant<BLOCK, CC, MODE, TT>), grid, dim3(TT), 0, s, x, res, g, eps, h_out, y_out, q, \
                        scale, (int)K)
-    if (C <= 1) MI_ROWQ(1);
-    else if (C <= 2) MI_ROWQ(2);
-    else if (C <= 4) MI_ROWQ(4);
-    else if (C <= 7) MI_ROWQ(7);
-    else if (C <= 8) MI_ROWQ(8);
+    if (nchunk <= 256) MI_ROWQ(1, 256);
+    else if (nchunk <= 512) MI_ROWQ(1, 512);
+    else if (nchunk <= 1024) MI_ROWQ(1, 1024);
+    else if (nchunk <= 2048) MI_ROWQ(2, 1024);
     else return MI_ERANGE;
 #undef MI_ROWQ
     return launch_status();

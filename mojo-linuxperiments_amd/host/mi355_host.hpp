@@ -238,9 +238,10 @@ struct KvCache {
     }
 };
 
-// One decoder layer of a decode step (one new token per sequence), chained on one stream, eleven launches:
-// (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache -> O linear ->
-// residual + RMSNorm + quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
+// One decoder layer of a decode step (one new token per sequence), chained on one stream, ten launches:
+// (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache (split, merge +
+// quantize: the output projection takes the rows in the rotated basis of V) -> O GEMV -> residual + RMSNorm +
+// quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
 // Holds its prepared weights, its KV cache and its scratch rows in the arena.
 struct DecoderLayer {
     int64_t B = 0, H = 0, Hq = 0, Hkv = 0, I = 0, T_cap = 0;
@@ -249,11 +250,12 @@ struct DecoderLayer {
     KvCache cache;
     const float *g1 = nullptr, *g2 = nullptr, *rope_cos = nullptr, *rope_sin = nullptr;
     // fp32 rows: layer input when it is a sum (h0), projections, attention output, residual stream after
-    // attention (h1), down output (dn); xn / hn / act only when prepare() was asked to trace
-    float *h0 = nullptr, *qkv_out = nullptr, *q = nullptr, *att = nullptr, *ao = nullptr, *h1 = nullptr, *gu = nullptr,
-          *dn = nullptr, *xn = nullptr, *hn = nullptr, *act = nullptr;
-    int8_t *cx = nullptr, *ci = nullptr;   // codes of the normalized rows [B,H] and of the activated rows [B,I]
-    float *sx = nullptr, *si = nullptr;
+    // attention (h1), down output (dn); xn / att (rotated basis) / hn / act only when prepare() was asked to trace
+    float *h0 = nullptr, *qkv_out = nullptr, *q = nullptr, *ao = nullptr, *h1 = nullptr, *gu = nullptr, *dn = nullptr,
+          *xn = nullptr, *att = nullptr, *hn = nullptr, *act = nullptr;
+    // codes of the normalized rows [B,H], of the attention rows [B,Hq*128] and of the activated rows [B,I]
+    int8_t *cx = nullptr, *ca = nullptr, *ci = nullptr;
+    float *sx = nullptr, *sa = nullptr, *si = nullptr;
 
     // fp32 weights in device memory: wqkv [(Hq+2Hkv)*128, H], wo [H, Hq*128], wgu [2I, H] (gate rows, then up
     // rows), wd [H, I]; norm weights g1, g2 [H]; rotary tables [T_cap, 64].  false if the arena is exhausted.
@@ -272,22 +274,24 @@ struct DecoderLayer {
         h0 = arena.template alloc<float>(B * H);
         qkv_out = arena.template alloc<float>(B * nqkv);
         q = arena.template alloc<float>(B * Hq * 128);
-        att = arena.template alloc<float>(B * Hq * 128);
         ao = arena.template alloc<float>(B * H);
         h1 = arena.template alloc<float>(B * H);
         gu = arena.template alloc<float>(B * 2 * I);
         dn = arena.template alloc<float>(B * H);
         cx = arena.template alloc<int8_t>(B * H);
+        ca = arena.template alloc<int8_t>(B * Hq * 128);
         ci = arena.template alloc<int8_t>(B * I);
         sx = arena.template alloc<float>(B);
+        sa = arena.template alloc<float>(B);
         si = arena.template alloc<float>(B);
         if (trace) {
             xn = arena.template alloc<float>(B * H);
+            att = arena.template alloc<float>(B * Hq * 128);
             hn = arena.template alloc<float>(B * H);
             act = arena.template alloc<float>(B * I);
-            ok = ok && xn && hn && act;
+            ok = ok && xn && att && hn && act;
         }
-        return ok && h0 && qkv_out && q && att && ao && h1 && gu && dn && cx && ci && sx && si;
+        return ok && h0 && qkv_out && q && ao && h1 && gu && dn && cx && ca && ci && sx && sa && si;
     }
     // x fp32 [B,H], plus residual fp32 [B,H] or nullptr: the layer input is their sum (left in h0).  pos, seq_len
     // int32 [B] in device memory (seq_len = pos + 1 in a plain decode step); t_max bounds seq_len.  out fp32 [B,H],
@@ -302,8 +306,10 @@ struct DecoderLayer {
         if (rc == MI_OK)
             rc = mi_rope_kv_append_f32_i8(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, cache.kq, cache.ks,
                                           cache.vq, cache.vs, pos, B, Hq, Hkv, 128, T_cap, stream);
-        if (rc == MI_OK) rc = cache.attend(q, att, seq_len, t_max, false, stream);
-        if (rc == MI_OK) rc = o.forward(att, ao, B, stream);
+        if (rc == MI_OK)
+            rc = mi_gqa_decode_attn_cache_quant_i8(q, cache.kq, cache.ks, cache.vq, cache.vs, att, ca, sa, B, Hq, Hkv, 128,
+                                                   T_cap, seq_len, t_max, cache.workspace, cache.workspace_bytes, stream);
+        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
         if (rc == MI_OK) rc = mi_rmsnorm_quant_f32_i8(ao, xin, g2, eps, h1, hn, cx, sx, B, H, 128, stream);
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(cx, sx, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, stream);
         if (rc == MI_OK) rc = mi_swiglu_quant_f32_i8(gu, act, ci, si, B, I, 128, stream);

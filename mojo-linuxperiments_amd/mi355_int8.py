@@ -95,6 +95,8 @@ SIGNATURES = {
     "mi_rmsnorm_quant_f32_i8": (i32, [vp, vp, vp, C.c_float, vp, vp, vp, vp, i64, i64, i32, vp]),
     "mi_swiglu_quant_f32_i8": (i32, [vp, vp, vp, vp, i64, i64, i32, vp]),
     "mi_add_f32": (i32, [vp, vp, vp, i64, vp]),
+    "mi_gqa_decode_attn_cache_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, vp,
+                                                i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_moe_route_workspace_bytes": (i64, [i64, i64]),
@@ -374,11 +376,11 @@ def moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=None):
 
 class DecoderLayer:
     """One decoder layer of a decode step, chained from the C-ABI entry points on one stream:
-    (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + KV-cache append -> attention over the cache ->
-    O linear -> residual + RMSNorm + quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
-    Eleven launches.  Test and bench plumbing over the same calls the C++ host struct of the same name makes
+    (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + KV-cache append -> attention over the cache (split,
+    merge + quantize) -> O GEMV -> residual + RMSNorm + quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV
+    (-> residual).  Ten launches.  Test and bench plumbing over the same calls the C++ host struct of the same name makes
     (host/mi355_host.hpp).  trace=True also writes the fp32 rows the fused kernels normally keep in registers
-    (xn, hn, act) so that a test can gate every stage."""
+    (xn, att, hn, act) so that a test can gate every stage."""
 
     def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
                  block=128, trace=False):
@@ -403,7 +405,9 @@ class DecoderLayer:
         self.vq, self.vs = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
         f = np.float32
         self.h0, self.qkv = dev.empty((B, H), f), dev.empty((B, self.NQKV), f)
-        self.q, self.att = dev.empty((B, Hq, D), f), dev.empty((B, Hq * D), f)
+        self.q = dev.empty((B, Hq, D), f)
+        self.att = dev.empty((B, Hq * D), f) if trace else None
+        self.ca, self.sa = dev.empty((B, Hq * D), np.int8), dev.empty(B, f)   # codes of the attention rows
         self.ao, self.h1 = dev.empty((B, H), f), dev.empty((B, H), f)
         self.gu, self.dn = dev.empty((B, 2 * I), f), dev.empty((B, H), f)
         self.xn = dev.empty((B, H), f) if trace else None
@@ -411,7 +415,6 @@ class DecoderLayer:
         self.act = dev.empty((B, I), f) if trace else None
         self.cx, self.sx = dev.empty((B, H), np.int8), dev.empty(B, f)        # codes of the normalized rows
         self.ci, self.si = dev.empty((B, I), np.int8), dev.empty(B, f)        # codes of the activated rows
-        self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, H, Hq * D), np.uint8)
         self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
 
     def step(self, x, pos, seq_len, t_max, out, stream=None, residual=None):
@@ -428,10 +431,13 @@ class DecoderLayer:
         check(lib.mi_rope_kv_append_f32_i8(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr,
                                            self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv,
                                            D, self.T_cap, s), "mi_rope_kv_append_f32_i8")
-        check(lib.mi_gqa_decode_attn_cache(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
-                                           self.att.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, 0,
-                                           self.att_ws.ptr, self.att_ws.nbytes, s), "mi_gqa_decode_attn_cache")
-        linear(self.att, self.wo[0], self.wo[1], self.ao, self.block, self.lin_ws, s)
+        # attention output stays in the rotated basis of V and is quantized by the merge itself: the O weights were
+        # rotated with block 128 = head_dim along K, so their GEMV takes these codes as they are
+        check(lib.mi_gqa_decode_attn_cache_quant_i8(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
+                                                    p(self.att), self.ca.ptr, self.sa.ptr, B, Hq, Hkv, D, self.T_cap,
+                                                    seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
+              "mi_gqa_decode_attn_cache_quant_i8")
+        gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
         check(lib.mi_rmsnorm_quant_f32_i8(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
                                           self.cx.ptr, self.sx.ptr, B, H, self.block, s), "mi_rmsnorm_quant_f32_i8")
         gemm_dequant(self.cx, self.sx, self.wgu[0], self.wgu[1], self.gu, s)

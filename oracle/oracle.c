@@ -66,6 +66,11 @@
  *      x'[i+D/2] = x[i+D/2]*c + x[i]*s; every product is rounded to fp32
  *      before the add or subtract (no FMA), so the result is fixed by IEEE-754.
  *  D12 SwiGLU over a fused row [gate(I) | up(I)]: D8 on (g[n], u[n]).
+ *  D13 In a decoder layer the output projection consumes the attention row in
+ *      the rotated basis of V (D4 with out_rotated != 0): the Hq*D values of a
+ *      token are quantized as one row by D2 with no further rotation, and the
+ *      projection weights are rotated along K with block D as for any linear
+ *      ((x.H) . (W.H)^T = x . W^T for the orthonormal H).
  */
 #include <math.h>
 #include <stdint.h>

@@ -21,6 +21,9 @@ int orc_gqa_decode(const float *, const int8_t *, const float *, const int8_t *,
 int orc_rmsnorm(const float *, const float *, const float *, float, float *, float *, int64_t, int64_t);
 int orc_rope_rows(float *, const int32_t *, const float *, const float *, int64_t, int64_t);
 int orc_swiglu(const float *, float *, int64_t, int64_t);
+void orc_quant_row(const float *, int64_t, int8_t *, float *);
+void orc_gemm_i8_i32(const int8_t *, const int8_t *, int32_t *, int64_t, int64_t, int64_t);
+void orc_dequant(const int32_t *, const float *, const float *, float *, int64_t, int64_t);
 }
 
 using namespace mi355;
@@ -354,15 +357,24 @@ static void test_decoder_layer(const Context &ctx)
             std::copy(vs.begin() + row, vs.begin() + row + n, pvs.begin() + h * n);
         }
         orc_gqa_decode(q.data() + b * Hq * D, pk.data(), pks.data(), pv.data(), pvs.data(), o_ref.data(), 1, Hq, Hkv, D, n,
-                       0, nullptr, nullptr, nullptr);
+                       1 /* rotated basis */, nullptr, nullptr, nullptr);
         for (int64_t i = 0; i < Hq * D; ++i) good = good && std::fabs(att[b * Hq * D + i] - o_ref[i]) <= 2e-5f;
     }
+    // the output projection takes each token's attention row as it stands: one quantizer row, no rotation
+    std::vector<int8_t> ca = download(layer.ca, (size_t)(B * Hq * D)), ca_ref((size_t)(B * Hq * D));
+    std::vector<float> sa = download(layer.sa, (size_t)B), sa_ref((size_t)B);
+    for (int64_t b = 0; b < B; ++b) orc_quant_row(att.data() + b * Hq * D, Hq * D, ca_ref.data() + b * Hq * D, &sa_ref[b]);
+    good = good && ca == ca_ref && sa == sa_ref;
     std::vector<float> ao = download(layer.ao, (size_t)(B * H)), h1 = download(layer.h1, (size_t)(B * H)),
                        hn = download(layer.hn, (size_t)(B * H)), gu = download(layer.gu, (size_t)(B * 2 * I)),
                        act = download(layer.act, (size_t)(B * I)), dn = download(layer.dn, (size_t)(B * H)),
                        out = download(dout, (size_t)(B * H));
     y.assign((size_t)(B * H), 0.0f);
-    orc_w8a8_linear(att.data(), ow.data(), os.data(), y.data(), B, H, Hq * D, 128, nullptr, nullptr, nullptr);
+    {
+        std::vector<int32_t> acc((size_t)(B * H));
+        orc_gemm_i8_i32(ca.data(), ow.data(), acc.data(), B, H, Hq * D);
+        orc_dequant(acc.data(), sa.data(), os.data(), y.data(), B, H);
+    }
     good = good && ao == y;
     std::vector<float> hh((size_t)(B * H));
     orc_rmsnorm(ao.data(), x.data(), g2.data(), 1e-5f, hh.data(), r.data(), B, H);

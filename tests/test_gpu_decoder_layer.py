@@ -138,11 +138,20 @@ def oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=None):
     att = np.empty((B, Hq, D), np.float32)
     for b in range(B):
         n = int(lens[b])
-        att[b] = orc.gqa_decode(q[b:b + 1], *(np.ascontiguousarray(c[b:b + 1, :, :n]) for c in cache))[0]
+        att[b] = orc.gqa_decode(q[b:b + 1], *(np.ascontiguousarray(c[b:b + 1, :, :n]) for c in cache),
+                                out_rotated=True)[0]
     att = att.reshape(B, Hq * D)
     if gpu is not None:
         assert np.max(np.abs(gpu["att"] - att)) <= 2e-5          # gate 2e-3
-    ao = orc.w8a8_linear(take("att", att), W["o"][0], W["o"][1], 128)[0]
+    # the O projection takes the attention row as it stands in the rotated basis: quantized per token, no rotation
+    a = take("att", att)
+    qa = np.empty((B, Hq * D), np.int8)
+    sa = np.empty(B, np.float32)
+    for b in range(B):
+        qa[b], sa[b] = orc.quant_row(a[b])
+    if gpu is not None:
+        assert np.array_equal(gpu["ca"], qa) and np.array_equal(gpu["sa"], sa)
+    ao = orc.dequant(orc.gemm_i8_i32(qa, W["o"][0]), sa, W["o"][1])
     if gpu is not None:
         assert np.array_equal(gpu["ao"], ao)
     h1, hn = orc.rmsnorm(take("ao", ao), W["g2"], eps, residual=x)
@@ -192,7 +201,7 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
         mi.check(mi.lib.mi_memcpy_h2d(buf.ptr, ref.ctypes.data, ref.nbytes, None))
     dpos, dlen = dev.empty(B, np.int32), dev.empty(B, np.int32)
     dx, dout = dev.empty((B, H), np.float32), dev.empty((B, H), np.float32)
-    names = ("xn", "qkv", "q", "att", "ao", "h1", "hn", "gu", "act", "dn", "kq", "ks", "vq", "vs")
+    names = ("xn", "qkv", "q", "att", "ca", "sa", "ao", "h1", "hn", "gu", "act", "dn", "kq", "ks", "vq", "vs")
     for step in range(3):
         pos = (start + step).astype(np.int32)
         lens = (pos + 1).astype(np.int32)

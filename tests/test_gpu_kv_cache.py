@@ -133,6 +133,41 @@ def test_attention_over_partly_filled_cache(mi, dev, orc, B, Hq, Hkv, T_cap, len
     assert np.max(np.abs(o - want)) <= TOL
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,T_cap,lens", [(4, 32, 8, 1024, [1, 700, 1024, 333]), (2, 8, 8, 64, [64, 0]),
+                                                  (3, 64, 16, 40, [40, 7, 22])])
+def test_attention_merge_fused_with_the_output_quantizer(mi, dev, orc, B, Hq, Hkv, T_cap, lens):
+    """The fused entry leaves the same rotated-basis rows as the plain one (same merge arithmetic) and their codes
+    and scale are the oracle's row quantizer applied to each token's Hq*128 values."""
+    mark = dev.mark()
+    g = np.random.default_rng(T_cap)
+    q = workload.normal(T_cap + 1, (B, Hq, D), 0)
+    kq = g.integers(-127, 128, (B, Hkv, T_cap, D)).astype(np.int8)
+    vq = g.integers(-127, 128, (B, Hkv, T_cap, D)).astype(np.int8)
+    ks = ((g.random((B, Hkv, T_cap)) + 0.5) * 0.02).astype(np.float32)
+    vs = ((g.random((B, Hkv, T_cap)) + 0.5) * 0.02).astype(np.float32)
+    lens = np.array(lens, np.int32)
+    cache = tuple(dev.upload(a) for a in (kq, ks, vq, vs))
+    dq, dlen = dev.upload(q), dev.upload(lens)
+    T_max = int(max(lens.max(), 1))
+    plain = cache_attention(mi, dev, dq, cache, dlen, B, Hq, Hkv, T_cap, T_max, True)
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max), np.uint8)
+    do, doq, dos = dev.empty((B, Hq, D), np.float32), dev.empty((B, Hq * D), np.int8), dev.empty(B, np.float32)
+    args = (dq.ptr, cache[0].ptr, cache[1].ptr, cache[2].ptr, cache[3].ptr)
+    tail = (B, Hq, Hkv, D, T_cap, dlen.ptr, T_max, ws.ptr, ws.nbytes, None)
+    mi.check(mi.lib.mi_gqa_decode_attn_cache_quant_i8(*args, do.ptr, doq.ptr, dos.ptr, *tail))
+    o, oq, osc = dev.download(do), dev.download(doq), dev.download(dos)
+    mi.check(mi.lib.mi_gqa_decode_attn_cache_quant_i8(*args, None, doq.ptr, dos.ptr, *tail))     # without the fp32 row
+    oq2, osc2 = dev.download(doq), dev.download(dos)
+    assert mi.lib.mi_gqa_decode_attn_cache_quant_i8(*args, None, None, dos.ptr, *tail) == mi.EINVAL
+    dev.reset_to(mark)
+    assert np.array_equal(o, plain)
+    for b in range(B):
+        qo, so = orc.quant_row(o[b].reshape(-1))
+        assert np.array_equal(oq[b], qo) and osc[b] == so
+    assert np.array_equal(oq, oq2) and np.array_equal(osc, osc2)
+    assert not o[lens == 0].any() and np.all(osc[lens == 0] == 1.0)
+
+
 def test_decode_loop_append_then_attend(mi, dev, orc):
     """Six decode steps on sequences of different lengths: each step appends one token per sequence at its own
     position and attends over what the sequence holds so far; the cache and every output follow the oracle."""
