@@ -580,7 +580,11 @@ int32_t launch_skinny(const int8_t *qx, const float *sx, const int8_t *qw, const
                       float *y, int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
 {
     const int M = (int)M64, N = (int)N64, K = (int)K64;
-    if (M <= 4) {
+    // M = 2..4 on a long K: the register kernel reads M activation rows per weight row pair and its activation
+    // traffic passes the weight traffic; the ring kernel reads them once per 16 weight rows (measured 13.4 against
+    // 16.6 us for 14336 -> 4096 at M = 4, a tie or worse on K = 4096)
+    const bool reg_path = M == 1 || (M <= 4 && K < 8192);
+    if (reg_path) {
         // K = 1024 * CW * QW (last chunk may be ragged) with CW <= 7 chunks per wave and QW in {1, 2, 4} waves per row
         const int nchunk = (K + 1023) >> 10;
         for (int QW = 1; QW <= 4; QW <<= 1) {
@@ -591,7 +595,7 @@ int32_t launch_skinny(const int8_t *qx, const float *sx, const int8_t *qw, const
             return launch_reg_cw<4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, CW, QW, s);
         }
     }
-    if (M <= 4 && (int64_t)4 * K <= 152 * 1024) {
+    if (reg_path && (int64_t)4 * K <= 152 * 1024) {
         if (M == 1) return launch_dot4<1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
         if (M == 2) return launch_dot4<2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
         return launch_dot4<4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
