@@ -349,11 +349,24 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
                                               T, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
     calls2 = [(lambda k=k: cached(k)) for k in sets]
     ms2 = graph_time(mi, dev, s, timer, calls2, reps) if graph else eager_time(dev, s, timer, calls2)
+    # the same caches read as pools of 16-token pages under a shuffled block table (the rows a pool holds are the
+    # same bytes; which token sits where does not change the time)
+    P = 16
+    max_pages = T // P
+    table = np.random.default_rng(3).permutation(B * max_pages).astype(np.int32).reshape(B, max_pages)
+    dtab = dev.upload(table)
+
+    def paged(k):
+        mi.check(lib.mi_gqa_decode_attn_paged(dq.ptr, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr, do.ptr, dtab.ptr,
+                                              max_pages, P, B, Hq, Hkv, D, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
+    calls3 = [(lambda k=k: paged(k)) for k in sets]
+    ms3 = graph_time(mi, dev, s, timer, calls3, reps) if graph else eager_time(dev, s, timer, calls3)
     dev.reset_to(mark)
     return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                       "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes,
-                                      "with_kv_append_us": round(ms2 * 1e3, 2)}}
+                                      "with_kv_append_us": round(ms2 * 1e3, 2),
+                                      "paged_16_token_pages_us": round(ms3 * 1e3, 2)}}
 
 
 def eager_time(dev, s, timer, calls):

@@ -212,6 +212,21 @@ MI_API int32_t mi_gqa_decode_attn_cache_quant_i8(const float *q, const int8_t *k
                                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                                                  const int32_t *seq_len, int64_t T_max,
                                                  void *workspace, int64_t workspace_bytes, void *stream);
+/* Paged layout of the same cache: the pools kq/vq int8 [pages, Hkv, P, D] and ks/vs fp32 [pages, Hkv, P] hold
+ * pages of P = page_size tokens (a power of two, >= 16); tokens [i*P, (i+1)*P) of sequence b live in page
+ * block_table[b*max_pages + i] (int32 in device memory; every entry that covers a token below seq_len[b], resp.
+ * the position being appended, must be a valid page of the pool: the kernels cannot check it).  Same arithmetic
+ * and same results as the dense layout.  No upstream counterpart. */
+MI_API int32_t mi_gqa_decode_attn_paged(const float *q, const int8_t *kq_pool, const float *ks_pool,
+                                        const int8_t *vq_pool, const float *vs_pool, float *o,
+                                        const int32_t *block_table, int64_t max_pages, int64_t page_size,
+                                        int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                        const int32_t *seq_len, int64_t T_max, int32_t out_rotated,
+                                        void *workspace, int64_t workspace_bytes, void *stream);
+MI_API int32_t mi_kv_append_paged_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                         int8_t *kq_pool, float *ks_pool, int8_t *vq_pool, float *vs_pool,
+                                         const int32_t *block_table, int64_t max_pages, int64_t page_size,
+                                         const int32_t *pos, int64_t B, int64_t Hkv, int64_t D, void *stream);
 /* a7 as the decode loop uses it: rotate (block 128 = D) and quantize the new token's key and value heads and
  * write codes and scale at token pos[b] of sequence b (int32 [B] in device memory; a sequence whose position is
  * outside [0, T_cap) is skipped).  Head h of sequence b is read at k_new + b*row_stride + h*D (floats), so

@@ -100,6 +100,8 @@ struct Params {
     int Hq, Hkv, G, T;    // T: tokens per sequence (the longest one when seq_len is given)
     int Tstride;          // tokens between consecutive (batch, kv head) rows of the cache
     const int32_t *seq_len;   // per-sequence token counts [B] (device), or null: every sequence holds T tokens
+    const int32_t *block_table;   // paged cache: page of tokens [i*P, (i+1)*P) of sequence b at [b*max_pages + i], or null
+    int max_pages, page_shift;    // P = 1 << page_shift tokens per page, P >= 16
     int tiles_per_split;  // 16-token tiles
     float score_scale;    // log2(e) / sqrt(D)
 };
@@ -137,7 +139,9 @@ constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each)
 
 // RAGGED: the span a workgroup can cover runs past the end of the cache and token indices are clamped for the
 // loads; otherwise every address is base + constant.  Tokens past the end of the split are masked in the scores.
-template <bool DUMP, bool RAGGED>
+// PAGED: the cache is a pool of pages [page][kv head][P tokens][128]; a 16-token tile lies in one page, so a wave
+// looks up one page per tile (uniform over the wave) and lanes are clamped inside their tile.
+template <bool DUMP, bool RAGGED, bool PAGED = false>
 __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
                                                float (&s_red)[4][4][D], float (&s_sc)[4][WAVE_TILES][16][4],
                                                float (&s_m)[4][4], float (&s_l)[4][4], float (&s_c)[4][4])
@@ -162,6 +166,21 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int
     const float *kswave = p.ks + (int64_t)bkv * p.Tstride + t_wave;
     const float *vswave = p.vs + (int64_t)bkv * p.Tstride + t_wave;
     const unsigned koff = (unsigned)(tk16 * D + 16 * ck);
+    // paged: row index (in tokens) of the first token of each of the wave's tiles inside the pool, and the last
+    // valid token offset inside that tile (tiles past the end of the sequence fall back on its last tile and are
+    // masked in the scores like any token past the end)
+    int64_t trow[PAGED ? WAVE_TILES : 1];
+    int tlast[PAGED ? WAVE_TILES : 1];
+    if constexpr (PAGED) {
+        const int last_tile = (T - 1) & ~15;
+#pragma unroll
+        for (int j = 0; j < WAVE_TILES; ++j) {
+            const int tt = min(t_wave + j * 64, last_tile);
+            const int page = __builtin_amdgcn_readfirstlane(p.block_table[(int64_t)b * p.max_pages + (tt >> p.page_shift)]);
+            trow[j] = (((int64_t)page * p.Hkv + kvh) << p.page_shift) + (tt & ((1 << p.page_shift) - 1));
+            tlast[j] = min(T - 1 - tt, 15);
+        }
+    }
 
     // the query row goes first: loads return in order, and the rotation of q can then run under the key loads
     const int hr = lane >> 4, jj = lane & 15;
@@ -176,7 +195,12 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int
     v4i ring[RING];
     float ksr[RING / 2], vsr[RING];
     auto load_k = [&](int j) {   // tile j -> slots (2j) % RING, (2j+1) % RING
-        if constexpr (RAGGED) {
+        if constexpr (PAGED) {
+            const int64_t row = trow[j] + min(tk16, tlast[j]);
+            ring[(2 * j) % RING] = *reinterpret_cast<const v4i *>(p.kq + row * D + 16 * ck);
+            ring[(2 * j + 1) % RING] = *reinterpret_cast<const v4i *>(p.kq + row * D + 64 + 16 * ck);
+            ksr[j % (RING / 2)] = p.ks[row];
+        } else if constexpr (RAGGED) {
             const int tk = min(t_wave + j * 64 + tk16, T - 1) - t_wave;
             ring[(2 * j) % RING] = *reinterpret_cast<const v4i *>(kwave + (int64_t)tk * D + 16 * ck);
             ring[(2 * j + 1) % RING] = *reinterpret_cast<const v4i *>(kwave + (int64_t)tk * D + 64 + 16 * ck);
@@ -189,7 +213,11 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int
     };
     auto load_v = [&](int u) {   // group u = 2*tile + half -> slot (2*WAVE_TILES + u) % RING
         const int j = u >> 1, g = u & 1;
-        if constexpr (RAGGED) {
+        if constexpr (PAGED) {
+            const int64_t row = trow[j] + min(g * 8 + slot, tlast[j]);
+            ring[(2 * WAVE_TILES + u) % RING] = *reinterpret_cast<const v4i *>(p.vq + row * D + 16 * chunk);
+            vsr[u % RING] = p.vs[row];
+        } else if constexpr (RAGGED) {
             const int tk = min(t_wave + j * 64 + g * 8 + slot, T - 1) - t_wave;
             ring[(2 * WAVE_TILES + u) % RING] = *reinterpret_cast<const v4i *>(vwave + (int64_t)tk * D + 16 * chunk);
             vsr[u % RING] = vswave[tk];
@@ -389,6 +417,10 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
             return;
         }
     }
+    if (p.block_table) {
+        gqa_split_body<false, true, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+        return;
+    }
     const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= T;
     if (full) gqa_split_body<DUMP, false>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
     else gqa_split_body<DUMP, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
@@ -550,7 +582,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
                         float *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T, int32_t out_rotated,
                         void *workspace, int64_t workspace_bytes, int8_t *dqq, float *dsq, int32_t *ddots,
                         hipStream_t s, int64_t Tstride = 0, const int32_t *seq_len = nullptr, int8_t *oq = nullptr,
-                        float *oscale = nullptr)
+                        float *oscale = nullptr, const int32_t *block_table = nullptr, int64_t max_pages = 0,
+                        int page_shift = 0)
 {
     int32_t rc = check_attn(B, Hq, Hkv, D, T);
     if (rc) return rc;
@@ -569,6 +602,7 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.G = (int)(Hq / Hkv); p.T = (int)T;
     p.Tstride = (int)(Tstride > 0 ? Tstride : T);
     p.seq_len = seq_len;
+    p.block_table = block_table; p.max_pages = (int)max_pages; p.page_shift = page_shift;
     p.tiles_per_split = (ntiles + splits - 1) / splits;
     p.score_scale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
     const dim3 grid((unsigned)splits, (unsigned)(B * Hkv));
@@ -645,6 +679,25 @@ extern "C" int32_t mi_gqa_decode_attn_cache_quant_i8(const float *q, const int8_
     if (T_cap > (1LL << 24) || Hq > 64) return MI_ERANGE;
     return run_attn(q, kq, ks, vq, vs, o_rot, B, Hq, Hkv, D, T_max, 1, workspace, workspace_bytes, nullptr, nullptr,
                     nullptr, as_stream(stream), T_cap, seq_len, oq, oscale);
+}
+
+extern "C" int32_t mi_gqa_decode_attn_paged(const float *q, const int8_t *kq_pool, const float *ks_pool,
+                                            const int8_t *vq_pool, const float *vs_pool, float *o,
+                                            const int32_t *block_table, int64_t max_pages, int64_t page_size,
+                                            int64_t B, int64_t Hq, int64_t Hkv, int64_t D, const int32_t *seq_len,
+                                            int64_t T_max, int32_t out_rotated, void *workspace,
+                                            int64_t workspace_bytes, void *stream)
+{
+    if (!o || !aligned16(o) || !seq_len || !aligned4(seq_len) || !block_table || !aligned4(block_table))
+        return MI_EINVAL;
+    if (page_size < 16 || (page_size & (page_size - 1)) || page_size > (1 << 20)) return MI_EINVAL;
+    if (T_max <= 0 || max_pages <= 0 || T_max > max_pages * page_size) return MI_EINVAL;
+    if (max_pages > (1LL << 24)) return MI_ERANGE;
+    int shift = 0;
+    while ((1LL << shift) < page_size) ++shift;
+    return run_attn(q, kq_pool, ks_pool, vq_pool, vs_pool, o, B, Hq, Hkv, D, T_max, out_rotated, workspace,
+                    workspace_bytes, nullptr, nullptr, nullptr, as_stream(stream), 0, seq_len, nullptr, nullptr,
+                    block_table, max_pages, shift);
 }
 
 extern "C" int32_t mi_gqa_decode_scores_i32(const float *q, const int8_t *kq, const float *ks, const int8_t *vq,

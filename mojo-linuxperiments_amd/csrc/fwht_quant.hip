@@ -201,7 +201,8 @@ __global__ __launch_bounds__(256) void k_kv_append(const float *__restrict__ k_n
                                                    int64_t row_stride, int8_t *__restrict__ kq,
                                                    float *__restrict__ ks, int8_t *__restrict__ vq,
                                                    float *__restrict__ vs, const int32_t *__restrict__ pos, int B,
-                                                   int Hkv, int T_cap)
+                                                   int Hkv, int T_cap, const int32_t *__restrict__ block_table,
+                                                   int max_pages, int page_shift)
 {
     constexpr int BLOCK = 128, LPB = 16;
     const int t = threadIdx.x, j = t % LPB;
@@ -228,7 +229,12 @@ __global__ __launch_bounds__(256) void k_kv_append(const float *__restrict__ k_n
     const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
     const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
     if (live) {
-        const int64_t row = ((int64_t)b * Hkv + h) * T_cap + tp;
+        int64_t row = ((int64_t)b * Hkv + h) * T_cap + tp;
+        if (block_table) {
+            // paged pool [page][kv head][P tokens]: the page that holds token tp of sequence b
+            const int page = block_table[(int64_t)b * max_pages + (tp >> page_shift)];
+            row = (((int64_t)page * Hkv + h) << page_shift) + (tp & ((1 << page_shift) - 1));
+        }
         int8_t *q = (is_v ? vq : kq) + row * BLOCK + 4 * j;
         if (j == 0) (is_v ? vs : ks)[row] = sc;
         *reinterpret_cast<uint32_t *>(q) = quant4(v[0], v[1], v[2], v[3], inv);
@@ -313,7 +319,30 @@ extern "C" int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, i
         return MI_EINVAL;
     const dim3 grid((unsigned)((B * Hkv + 15) / 16), 2);
     hipLaunchKernelGGL(k_kv_append, grid, dim3(256), 0, as_stream(stream), k_new, v_new, row_stride, kq, ks, vq, vs,
-                       pos, (int)B, (int)Hkv, (int)T_cap);
+                       pos, (int)B, (int)Hkv, (int)T_cap, (const int32_t *)nullptr, 0, 0);
+    return launch_status();
+}
+
+extern "C" int32_t mi_kv_append_paged_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                             int8_t *kq_pool, float *ks_pool, int8_t *vq_pool, float *vs_pool,
+                                             const int32_t *block_table, int64_t max_pages, int64_t page_size,
+                                             const int32_t *pos, int64_t B, int64_t Hkv, int64_t D, void *stream)
+{
+    if (!k_new || !v_new || !kq_pool || !ks_pool || !vq_pool || !vs_pool || !pos || !block_table) return MI_EINVAL;
+    if (B <= 0 || Hkv <= 0 || D != 128 || max_pages <= 0) return MI_EINVAL;
+    if (page_size < 16 || (page_size & (page_size - 1)) || page_size > (1 << 20)) return MI_EINVAL;
+    if (row_stride < Hkv * D || row_stride % 4) return MI_EINVAL;
+    if (B * Hkv > (1LL << 24) || max_pages * page_size > (1LL << 24)) return MI_ERANGE;
+    if (!aligned16(k_new) || !aligned16(v_new) || !aligned4(kq_pool) || !aligned4(vq_pool) || !aligned4(ks_pool) ||
+        !aligned4(vs_pool) || !aligned4(pos) || !aligned4(block_table))
+        return MI_EINVAL;
+    int shift = 0;
+    while ((1LL << shift) < page_size) ++shift;
+    const dim3 grid((unsigned)((B * Hkv + 15) / 16), 2);
+    // positions are valid inside the sequence's table: [0, max_pages * page_size)
+    hipLaunchKernelGGL(k_kv_append, grid, dim3(256), 0, as_stream(stream), k_new, v_new, row_stride, kq_pool, ks_pool,
+                       vq_pool, vs_pool, pos, (int)B, (int)Hkv, (int)(max_pages * page_size), block_table,
+                       (int)max_pages, shift);
     return launch_status();
 }
 

@@ -238,6 +238,43 @@ struct KvCache {
     }
 };
 
+// The same cache as pools of pages shared by all sequences: tokens [i*P, (i+1)*P) of sequence b live in page
+// table[b*max_pages + i].  The table is the caller's (int32 in device memory): a scheduler hands pages out.
+struct PagedKvCache {
+    int64_t B = 0, Hq = 0, Hkv = 0, D = 128, pages = 0, page_size = 0, max_pages = 0;
+    int8_t *kq = nullptr, *vq = nullptr;
+    float *ks = nullptr, *vs = nullptr;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t n_pages, int64_t p_size, int64_t max_pages_per_seq)
+    {
+        B = b; Hq = hq; Hkv = hkv; pages = n_pages; page_size = p_size; max_pages = max_pages_per_seq;
+        workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, max_pages * page_size);
+        if (workspace_bytes <= 0) return false;
+        kq = arena.template alloc<int8_t>(pages * Hkv * page_size * D);
+        vq = arena.template alloc<int8_t>(pages * Hkv * page_size * D);
+        ks = arena.template alloc<float>(pages * Hkv * page_size);
+        vs = arena.template alloc<float>(pages * Hkv * page_size);
+        workspace = arena.template alloc<uint8_t>(workspace_bytes);
+        return kq && vq && ks && vs && workspace;
+    }
+    explicit operator bool() const { return workspace != nullptr; }
+    int32_t append(const float *k_new, const float *v_new, int64_t row_stride, const int32_t *table, const int32_t *pos,
+                   void *stream) const
+    {
+        return mi_kv_append_paged_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, table, max_pages, page_size, pos, B, Hkv,
+                                         D, stream);
+    }
+    int32_t attend(const float *q, float *o, const int32_t *table, const int32_t *seq_len, int64_t t_max, bool out_rotated,
+                   void *stream) const
+    {
+        return mi_gqa_decode_attn_paged(q, kq, ks, vq, vs, o, table, max_pages, page_size, B, Hq, Hkv, D, seq_len, t_max,
+                                        out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+    }
+};
+
 // One decoder layer of a decode step (one new token per sequence), chained on one stream, ten launches:
 // (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache (split, merge +
 // quantize: the output projection takes the rows in the rotated basis of V) -> O GEMV -> residual + RMSNorm +

@@ -97,6 +97,9 @@ SIGNATURES = {
     "mi_add_f32": (i32, [vp, vp, vp, i64, vp]),
     "mi_gqa_decode_attn_cache_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, vp,
                                                 i64, vp]),
+    "mi_gqa_decode_attn_paged": (i32, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64,
+                                       vp]),
+    "mi_kv_append_paged_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_moe_route_workspace_bytes": (i64, [i64, i64]),

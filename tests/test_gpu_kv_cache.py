@@ -235,3 +235,91 @@ def test_bad_arguments_are_refused(mi, dev):
     assert lib.mi_gqa_decode_attn_cache(*args, T_cap, None, T_cap, 0, ws.ptr, ws.nbytes, None) == mi.EINVAL
     assert lib.mi_gqa_decode_attn_cache(*args, T_cap, pos.ptr, T_cap, 0, ws.ptr, 16, None) == mi.ENOSPC
     dev.reset_to(mark)
+
+
+def to_pages(g, dense, P, max_pages, spare=3):
+    """Scatter dense cache arrays [B,Hkv,T,...] into pools [pages,Hkv,P,...] under a random block table."""
+    B, Hkv, T = dense[0].shape[:3]
+    npages = B * max_pages + spare
+    table = g.permutation(npages)[:B * max_pages].astype(np.int32).reshape(B, max_pages)
+    pools = []
+    for a in dense:
+        pool = np.zeros((npages, Hkv, P) + a.shape[3:], a.dtype)
+        if a.dtype == np.float32:
+            pool[...] = np.float32(np.nan)            # a page that is not in the table must never be read
+        for b in range(B):
+            for i in range(max_pages):
+                lo, hi = i * P, min((i + 1) * P, T)
+                if lo < T:
+                    pool[table[b, i], :, :hi - lo] = a[b, :, lo:hi]
+        pools.append(pool)
+    return pools, table
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,P,lens", [
+    (4, 8, 2, 1024, 16, [1, 700, 1024, 333]),
+    (2, 32, 8, 4096, 256, [4096, 2500]),
+    (3, 4, 1, 200, 64, [200, 17, 64]),
+    (2, 8, 4, 96, 32, [0, 96]),
+])
+@pytest.mark.parametrize("out_rotated", [False, True])
+def test_paged_attention_equals_dense(mi, dev, orc, B, Hq, Hkv, T, P, lens, out_rotated):
+    mark = dev.mark()
+    g = np.random.default_rng(T + P)
+    q = workload.normal(T + P, (B, Hq, D), 0)
+    dense = [g.integers(-127, 128, (B, Hkv, T, D)).astype(np.int8), ((g.random((B, Hkv, T)) + 0.5) * 0.02).astype(np.float32),
+             g.integers(-127, 128, (B, Hkv, T, D)).astype(np.int8), ((g.random((B, Hkv, T)) + 0.5) * 0.02).astype(np.float32)]
+    lens = np.array(lens, np.int32)
+    max_pages = (T + P - 1) // P
+    pools, table = to_pages(g, dense, P, max_pages)
+    # tokens past a sequence's length: poison in the pools as well (same page, later offset)
+    cache = tuple(dev.upload(a) for a in dense)
+    dpools = tuple(dev.upload(a) for a in pools)
+    dq, dlen, dtab = dev.upload(q), dev.upload(lens), dev.upload(table)
+    T_max = int(max(lens.max(), 1))
+    want_gpu = cache_attention(mi, dev, dq, cache, dlen, B, Hq, Hkv, T, T_max, out_rotated)
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max), np.uint8)
+    do = dev.empty((B, Hq, D), np.float32)
+    mi.check(mi.lib.mi_gqa_decode_attn_paged(dq.ptr, dpools[0].ptr, dpools[1].ptr, dpools[2].ptr, dpools[3].ptr, do.ptr,
+                                             dtab.ptr, max_pages, P, B, Hq, Hkv, D, dlen.ptr, T_max,
+                                             1 if out_rotated else 0, ws.ptr, ws.nbytes, None),
+             "mi_gqa_decode_attn_paged")
+    o = dev.download(do)
+    dev.reset_to(mark)
+    assert np.isfinite(o).all()
+    assert np.array_equal(o, want_gpu)                          # same arithmetic in the same order
+    want = oracle_per_sequence(orc, q, *dense, lens, out_rotated)
+    assert np.max(np.abs(o - want)) <= 2e-5                     # gate: TOL
+
+
+def test_paged_append_lands_in_the_right_page(mi, dev, orc):
+    mark = dev.mark()
+    B, Hkv, P, max_pages = 5, 2, 16, 4
+    g = np.random.default_rng(77)
+    npages = B * max_pages + 2
+    table = g.permutation(npages)[:B * max_pages].astype(np.int32).reshape(B, max_pages)
+    bgq = g.integers(-127, 128, (npages, Hkv, P, D)).astype(np.int8)
+    bgs = g.random((npages, Hkv, P), dtype=np.float32)
+    pools = [dev.upload(bgq), dev.upload(bgs), dev.upload(bgq), dev.upload(bgs)]
+    k = workload.normal(5, (B, Hkv, D), 1)
+    v = workload.normal(5, (B, Hkv, D), 2)
+    pos = np.array([0, 15, 16, 63, 64], np.int32)              # the last one is past the table: skipped
+    dk, dv, dpos, dtab = dev.upload(k), dev.upload(v), dev.upload(pos), dev.upload(table)
+    mi.check(mi.lib.mi_kv_append_paged_f32_i8(dk.ptr, dv.ptr, Hkv * D, pools[0].ptr, pools[1].ptr, pools[2].ptr,
+                                              pools[3].ptr, dtab.ptr, max_pages, P, dpos.ptr, B, Hkv, D, None),
+             "mi_kv_append_paged_f32_i8")
+    kq, ks, vq, vs = (dev.download(b) for b in pools)
+    assert mi.lib.mi_kv_append_paged_f32_i8(dk.ptr, dv.ptr, Hkv * D, pools[0].ptr, pools[1].ptr, pools[2].ptr,
+                                            pools[3].ptr, dtab.ptr, max_pages, 24, dpos.ptr, B, Hkv, D, None) == mi.EINVAL
+    dev.reset_to(mark)
+    wkq, wks, wvq, wvs = bgq.copy(), bgs.copy(), bgq.copy(), bgs.copy()
+    kqo, kso = orc.rotate_quant_rows(k.reshape(-1, D), D)
+    vqo, vso = orc.rotate_quant_rows(v.reshape(-1, D), D)
+    for b in range(B):
+        if pos[b] < max_pages * P:
+            pg, off = table[b, pos[b] // P], pos[b] % P
+            for h in range(Hkv):
+                wkq[pg, h, off], wks[pg, h, off] = kqo[b * Hkv + h], kso[b * Hkv + h]
+                wvq[pg, h, off], wvs[pg, h, off] = vqo[b * Hkv + h], vso[b * Hkv + h]
+    assert np.array_equal(kq, wkq) and np.array_equal(ks, wks)
+    assert np.array_equal(vq, wvq) and np.array_equal(vs, wvs)
