@@ -162,10 +162,29 @@ __global__ __launch_bounds__(1024) void k_moe_dispatch(const int32_t *__restrict
     const int tid = threadIdx.x, nt = blockDim.x;
     const int P = T * topk;
     for (int i = tid; i < E * W; i += nt) bm[i] = 0u;
+    // a thread's pairs stay in registers between the two passes when they are few (one global round trip less)
+    constexpr int KEEP = 8;
+    const bool keep = P <= KEEP * nt;
+    int mine[KEEP];
+    if (keep) {
+#pragma unroll
+        for (int i = 0; i < KEEP; ++i) {
+            const int pr = tid + i * nt;
+            mine[i] = pr < P ? idx[pr] : -1;
+        }
+    }
     __syncthreads();
-    for (int pr = tid; pr < P; pr += nt) {
-        const int e = idx[pr], t = pr / topk;
-        if (e >= 0 && e < E) atomicOr(&bm[e * W + (t >> 5)], 1u << (t & 31));
+    if (keep) {
+#pragma unroll
+        for (int i = 0; i < KEEP; ++i) {
+            const int e = mine[i], t = (tid + i * nt) / topk;
+            if (e >= 0 && e < E) atomicOr(&bm[e * W + (t >> 5)], 1u << (t & 31));
+        }
+    } else {
+        for (int pr = tid; pr < P; pr += nt) {
+            const int e = idx[pr], t = pr / topk;
+            if (e >= 0 && e < E) atomicOr(&bm[e * W + (t >> 5)], 1u << (t & 31));
+        }
     }
     __syncthreads();
     for (int e = tid; e < E; e += nt) {
@@ -177,29 +196,65 @@ __global__ __launch_bounds__(1024) void k_moe_dispatch(const int32_t *__restrict
         seg[e + 1] = c;
     }
     __syncthreads();
-    if (tid == 0) {
-        seg[0] = 0;
-        for (int e = 0; e < E; ++e) seg[e + 1] += seg[e];
+    // exclusive scan of the E counts by one wave: lane l sums its run of ceil(E/64) counts, the wave scans the 64
+    // run totals with shuffles, the lane writes its run back (a serial loop over E through LDS costs a dependent
+    // LDS round trip per expert)
+    if (tid < 64) {
+        const int run = (E + 63) / 64;
+        const int lo = min(tid * run, E), hi = min(lo + run, E);
+        int sum = 0;
+        for (int e = lo; e < hi; ++e) sum += seg[e + 1];
+        int incl = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (tid >= off) incl += v;
+        }
+        int acc = incl - sum;
+        if (tid == 0) seg[0] = 0;
+        for (int e = lo; e < hi; ++e) {
+            acc += seg[e + 1];
+            seg[e + 1] = acc;
+        }
     }
     __syncthreads();
     for (int e = tid; e <= E; e += nt) seg_off[e] = seg[e];
     if (order) {
-        for (int e = tid; e < E; e += nt) {
-            const int c = seg[e + 1] - seg[e];
+        // rank of expert e among the counts (descending, ties by index): 8 lanes share an expert
+        for (int e0 = 0; e0 < E; e0 += nt / 8) {
+            const int e = e0 + (tid >> 3), part = tid & 7;
             int rank = 0;
-            for (int o = 0; o < E; ++o) {
-                const int co = seg[o + 1] - seg[o];
-                rank += (co > c || (co == c && o < e)) ? 1 : 0;
+            if (e < E) {
+                const int c = seg[e + 1] - seg[e];
+                for (int o = part; o < E; o += 8) {
+                    const int co = seg[o + 1] - seg[o];
+                    rank += (co > c || (co == c && o < e)) ? 1 : 0;
+                }
             }
-            order[rank] = e;
+            rank += __shfl_xor(rank, 1, 64);
+            rank += __shfl_xor(rank, 2, 64);
+            rank += __shfl_xor(rank, 4, 64);
+            if (e < E && part == 0) order[rank] = e;
         }
     }
-    for (int pr = tid; pr < P; pr += nt) {
-        const int e = idx[pr], t = pr / topk;
-        if (e < 0 || e >= E) continue;
-        const uint32_t word = bm[e * W + (t >> 5)];
-        const int pos = seg[e] + (int)pre[e * W + (t >> 5)] + __popc(word & ((1u << (t & 31)) - 1u));
-        perm[pos] = pr;
+    if (keep) {
+#pragma unroll
+        for (int i = 0; i < KEEP; ++i) {
+            const int pr = tid + i * nt;
+            const int e = mine[i], t = pr / topk;
+            if (e < 0 || e >= E) continue;
+            const uint32_t word = bm[e * W + (t >> 5)];
+            const int pos = seg[e] + (int)pre[e * W + (t >> 5)] + __popc(word & ((1u << (t & 31)) - 1u));
+            perm[pos] = pr;
+        }
+    } else {
+        for (int pr = tid; pr < P; pr += nt) {
+            const int e = idx[pr], t = pr / topk;
+            if (e < 0 || e >= E) continue;
+            const uint32_t word = bm[e * W + (t >> 5)];
+            const int pos = seg[e] + (int)pre[e * W + (t >> 5)] + __popc(word & ((1u << (t & 31)) - 1u));
+            perm[pos] = pr;
+        }
     }
 }
 
