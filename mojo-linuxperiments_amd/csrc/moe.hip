@@ -443,12 +443,16 @@ __global__ __launch_bounds__(256) void k_moe_expert_gemm(const int8_t *__restric
 // The same contraction with the activation fragments held in registers (possible when a wave's K slice is at
 // most NSMAX steps of 128 bytes): only weights travel through the ring, twice as many of them are in flight
 // for the same LDS, and a workgroup walks several row chunks against one set of activation registers.
-constexpr int RX_RING = 4;
+// stages in flight per wave.  The down projection's workgroups are short (two chunks of 768-byte rows) and pay
+// their set-up (segment -> permutation -> activation rows, two dependent round trips) for little streaming: a ring
+// of two stages lets three of them share a compute unit instead of two (measured 61.5 -> 56 us); gate/up streams
+// six chunks of 2048-byte rows per workgroup and is better off with four stages in flight.
+constexpr int rx_ring(bool down) { return down ? 2 : 4; }
 constexpr int RX_STAGE = 2 * NGRP * 1024;
-constexpr int RX_RING_BYTES = 4 * RX_RING * RX_STAGE;
+constexpr int rx_ring_bytes(bool down) { return 4 * rx_ring(down) * RX_STAGE; }
 constexpr int RX_MT = 3;   // most 16-token fragments per pass
 constexpr int RX_RED_BYTES = NGRP * RX_MT * 4 * 64 * 4;
-constexpr int RX_LDS = RX_RING_BYTES + RX_RED_BYTES + 16 * RX_MT * 8 + 8 * 128 * 4;   // + metadata + scales of <= 8 chunks
+constexpr int rx_lds(bool down) { return rx_ring_bytes(down) + RX_RED_BYTES + 16 * RX_MT * 8 + 8 * 128 * 4; }   // + metadata + scales of <= 8 chunks
 
 template <bool DOWN, int NSMAX, int MTT>
 __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ act,
@@ -472,6 +476,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     // and the segment / permutation lookups are paid once per workgroup.
     constexpr int CHUNK_ROWS = DOWN ? 128 : 16;
     const int n0 = DOWN ? blockIdx.x * nch * 128 + wave * 32 : blockIdx.x * nch * 16;
+    constexpr int RX_RING = rx_ring(DOWN), RX_RING_BYTES = rx_ring_bytes(DOWN);
     char *ring = smem + wave * (RX_RING * RX_STAGE);
     int *s_red = reinterpret_cast<int *>(smem + RX_RING_BYTES);    // [NGRP][MTT][4][64] sums over the four K slices (gate/up)
     // per-pass token metadata and per-chunk weight scales sit in LDS so that the epilogue of a chunk issues no
@@ -860,10 +865,10 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
             MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<false, NS>),        \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::RX_LDS));               \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::rx_lds(false)));        \
             set = true;                                                                                         \
         }                                                                                                       \
-        hipLaunchKernelGGL((moe::k_moe_expert_rx<false, NS>), grid, dim3(256), moe::RX_LDS, s, qx, sx, perm, seg, \
+        hipLaunchKernelGGL((moe::k_moe_expert_rx<false, NS>), grid, dim3(256), moe::rx_lds(false), s, qx, sx, perm, seg, \
                            wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk, nch, order);                   \
     } while (0)
         if (ns_gu <= 2) MI_RX_GU(2);
@@ -889,10 +894,10 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
             MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<true, NS>),         \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::RX_LDS));               \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::rx_lds(true)));         \
             set = true;                                                                                         \
         }                                                                                                       \
-        hipLaunchKernelGGL((moe::k_moe_expert_rx<true, NS>), grid, dim3(256), moe::RX_LDS, s, hq, hs, perm, seg, wd, \
+        hipLaunchKernelGGL((moe::k_moe_expert_rx<true, NS>), grid, dim3(256), moe::rx_lds(true), s, hq, hs, perm, seg, wd, \
                            sd, (const int8_t *)nullptr, (const float *)nullptr, out, (int)I, (int)H, (int)H,    \
                            (int)topk, nch, order);                                                              \
     } while (0)
