@@ -163,6 +163,55 @@ def test_gate_orders_two_streams(mi, ctx):
     mi.check(lib.mi_arena_destroy(a))
 
 
+def test_butterfly_all_reduce_over_eight_pools(mi, ctx):
+    """test_all_reduce (test_linux_threading.mojo:478-553) with a stream pool per "node": log2(N) rounds, in round r
+    node i reads the value of node i ^ (1 << r) into its scratch (phase 1), every pool is waited for, then adds the
+    scratch to its own value (phase 2), every pool is waited for.  Afterwards every node holds 1 + 2 + ... + N."""
+    lib = mi.lib
+    N, L = 8, 4096
+    a = C.c_void_p()
+    mi.check(lib.mi_arena_create(ctx, 1 << 20, 256, C.byref(a)))
+    values = [lib.mi_arena_alloc(a, L * 4) for _ in range(N)]
+    scratch = [lib.mi_arena_alloc(a, L * 4) for _ in range(N)]
+    for i in range(N):
+        host = np.full(L, i + 1, np.float32)
+        mi.check(lib.mi_memcpy_h2d(values[i], host.ctypes.data, host.nbytes, None))
+    mi.check(lib.mi_stream_synchronize(None))
+    pools = []
+    for _ in range(N):
+        p = C.c_void_p()
+        mi.check(lib.mi_stream_pool_create(ctx, 1, C.byref(p)))
+        pools.append(p)
+
+    def launch(node, op):
+        slot = lib.mi_stream_pool_begin(pools[node])
+        assert slot == 0
+        mi.check(op(lib.mi_stream_pool_stream(pools[node], slot)))
+        mi.check(lib.mi_stream_pool_end(pools[node], slot))
+
+    r = 0
+    while (1 << r) < N:
+        for node in range(N):
+            partner = node ^ (1 << r)
+            launch(node, lambda s, n=node, q=partner: lib.mi_memcpy_d2d(scratch[n], values[q], L * 4, s))
+        for p in pools:
+            mi.check(lib.mi_stream_pool_wait_all(p))
+        for node in range(N):
+            launch(node, lambda s, n=node: lib.mi_add_f32(values[n], scratch[n], values[n], L, s))
+        for p in pools:
+            mi.check(lib.mi_stream_pool_wait_all(p))
+        r += 1
+    assert r == 3
+    out = np.empty(L, np.float32)
+    for i in range(N):
+        mi.check(lib.mi_memcpy_d2h(out.ctypes.data, values[i], out.nbytes, None))
+        mi.check(lib.mi_stream_synchronize(None))
+        assert np.all(out == N * (N + 1) // 2)
+    for p in pools:
+        mi.check(lib.mi_stream_pool_destroy(p))
+    mi.check(lib.mi_arena_destroy(a))
+
+
 def test_pinned_host_staging_and_events(mi, ctx):
     lib = mi.lib
     p = lib.mi_host_alloc(1 << 20)
