@@ -163,6 +163,52 @@ def test_gate_orders_two_streams(mi, ctx):
     mi.check(lib.mi_arena_destroy(a))
 
 
+def test_wait_any_returns_slots_in_completion_order(mi, ctx):
+    """test_wait_any (test_linux_threading.mojo:304-357): workers with inverse amounts of work finish in
+    reverse order.  A worker's work is a chain of one-workgroup kernels (1500, 1000, 500 of them) recorded as a graph
+    beforehand, so that the launches leave the host within microseconds of each other and the chains run side by
+    side.  Three workers, not four: a process has four hardware queues here and streams beyond that share one, which
+    serializes them behind each other whatever their length."""
+    lib = mi.lib
+    pool, a = C.c_void_p(), C.c_void_p()
+    mi.check(lib.mi_stream_pool_create(ctx, 3, C.byref(pool)))
+    mi.check(lib.mi_arena_create(ctx, 1 << 20, 256, C.byref(a)))
+    bufs = [lib.mi_arena_alloc(a, 4096) for _ in range(3)]
+    one = lib.mi_arena_alloc(a, 4096)
+    ones = np.ones(1024, np.float32)
+    mi.check(lib.mi_memcpy_h2d(one, ones.ctypes.data, ones.nbytes, None))
+    mi.check(lib.mi_add_f32(one, one, bufs[0], 1024, None))      # first-launch costs paid before the race
+    mi.check(lib.mi_stream_synchronize(None))
+    graphs = []
+    for i in range(3):
+        s = lib.mi_stream_pool_stream(pool, i)
+        mi.check(lib.mi_fill_u32(bufs[i], 0, 1024, s))
+        mi.check(lib.mi_stream_synchronize(s))
+        mi.check(lib.mi_graph_capture_begin(s))
+        for _ in range(500 * (3 - i)):
+            mi.check(lib.mi_add_f32(bufs[i], one, bufs[i], 1024, s))
+        g = C.c_void_p()
+        mi.check(lib.mi_graph_capture_end(s, C.byref(g)))
+        graphs.append(g)
+    for i in range(3):
+        slot = lib.mi_stream_pool_begin(pool)
+        assert slot == i
+        mi.check(lib.mi_graph_launch(graphs[i], lib.mi_stream_pool_stream(pool, slot)))
+        mi.check(lib.mi_stream_pool_end(pool, slot))
+    order = [lib.mi_stream_pool_wait_any(pool) for _ in range(3)]
+    assert order == [2, 1, 0]
+    assert lib.mi_stream_pool_wait_any(pool) == -1
+    out = np.empty(1024, np.float32)
+    for i in range(3):
+        mi.check(lib.mi_memcpy_d2h(out.ctypes.data, bufs[i], out.nbytes, None))
+        mi.check(lib.mi_stream_synchronize(None))
+        assert np.all(out == 500 * (3 - i))                      # every link of the chain ran, in order
+    for g in graphs:
+        mi.check(lib.mi_graph_destroy(g))
+    mi.check(lib.mi_stream_pool_destroy(pool))
+    mi.check(lib.mi_arena_destroy(a))
+
+
 def test_butterfly_all_reduce_over_eight_pools(mi, ctx):
     """test_all_reduce (test_linux_threading.mojo:478-553) with a stream pool per "node": log2(N) rounds, in round r
     node i reads the value of node i ^ (1 << r) into its scratch (phase 1), every pool is waited for, then adds the
