@@ -82,6 +82,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-sub", action="store_true", help="only the headline workload")
+    ap.add_argument("--decode-layer-only", action="store_true",
+                    help="only the decode-layer chain sub-metric (for a kernel trace of that chain alone)")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
@@ -95,6 +97,14 @@ def main():
 
     if args.pmc_probe:
         return pmc_probe(mi, wl)
+    if args.decode_layer_only:
+        dev = mi.Device(arena_bytes=12 << 30)
+        pool = mi.StreamPool(dev, 1)
+        s = pool.stream(0)
+        print(json.dumps(decode_layer_chain(mi, wl, dev, s, Timer(mi, s), reps=20)), flush=True)
+        pool.destroy()
+        dev.close()
+        return
 
     dev = mi.Device(arena_bytes=12 << 30)
     pool = mi.StreamPool(dev, 1)
