@@ -192,6 +192,15 @@ __global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ 
         }
     }
     if constexpr (MODE == 0) {
+        // the norm weights are requested before the reduction: their round trip runs under it
+        float4 gl[C], gh[C];
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            if (t + i * TPB < nchunk) {
+                gl[i] = *reinterpret_cast<const float4 *>(g + base[i]);
+                gh[i] = *reinterpret_cast<const float4 *>(g + base[i] + BLOCK / 2);
+            }
+        }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
         if (lane == 0) s_part[wave] = ss;
@@ -209,12 +218,10 @@ __global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ 
 #pragma unroll
         for (int i = 0; i < C; ++i) {
             if (t + i * TPB < nchunk) {
-                const float4 gl = *reinterpret_cast<const float4 *>(g + base[i]);
-                const float4 gh = *reinterpret_cast<const float4 *>(g + base[i] + BLOCK / 2);
-                v[i][0] = (v[i][0] * r) * gl.x; v[i][1] = (v[i][1] * r) * gl.y;
-                v[i][2] = (v[i][2] * r) * gl.z; v[i][3] = (v[i][3] * r) * gl.w;
-                v[i][4] = (v[i][4] * r) * gh.x; v[i][5] = (v[i][5] * r) * gh.y;
-                v[i][6] = (v[i][6] * r) * gh.z; v[i][7] = (v[i][7] * r) * gh.w;
+                v[i][0] = (v[i][0] * r) * gl[i].x; v[i][1] = (v[i][1] * r) * gl[i].y;
+                v[i][2] = (v[i][2] * r) * gl[i].z; v[i][3] = (v[i][3] * r) * gl[i].w;
+                v[i][4] = (v[i][4] * r) * gh[i].x; v[i][5] = (v[i][5] * r) * gh[i].y;
+                v[i][6] = (v[i][6] * r) * gh[i].z; v[i][7] = (v[i][7] * r) * gh[i].w;
             }
         }
     }
