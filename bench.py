@@ -102,6 +102,7 @@ def main():
         pool = mi.StreamPool(dev, 1)
         s = pool.stream(0)
         print(json.dumps(decode_layer_chain(mi, wl, dev, s, Timer(mi, s), reps=20)), flush=True)
+        print(json.dumps(decode_layer_chain(mi, wl, dev, s, Timer(mi, s), reps=20, batch=1)), flush=True)
         pool.destroy()
         dev.close()
         return
@@ -231,6 +232,7 @@ def main():
         sub.update(moe_layer(mi, wl, dev, s, timer))
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer))
+        sub.update(decode_layer_chain(mi, wl, dev, s, timer, batch=1))
         sub.update(host_staging(mi, wl, dev, s, timer))
     out["sub_metrics"] = sub
     if not args.skip_cpu:
@@ -440,13 +442,15 @@ def cfg0_linear(mi, wl, dev, s, timer, shapes):
                                 "TOPS": round(wl.gemm_ops(M, N, K) / (ms * 1e-3) / 1e12, 2)}}
 
 
-def decode_layer_chain(mi, wl, dev, s, timer, reps=10):
+def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None):
     """A decode step through decoder layers of the cfg1 / cfg2 shapes (hidden 4096, 32/8 heads of 128, FFN 14336,
     16 sequences with 4095 cached tokens each): three layers with their own weights (654 MB) and KV caches
     (417 MB) run one after the other, so that nothing a layer reads is left in the memory-side cache from its
     last turn; the three-layer step is recorded into a graph and replayed."""
     c = wl.ATTN
     B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
+    if batch is not None:
+        B = batch
     H, I = 4096, 14336
     mark = dev.mark()
     inv = 10000.0 ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
@@ -480,7 +484,7 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10):
     wbytes = ((Hq + 2 * Hkv) * D * H + H * Hq * D + 2 * I * H + H * I)
     nbytes = wbytes + wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
     dev.reset_to(mark)
-    return {"decode_layer_b16_t4096": {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10,
+    return {"decode_layer_b%d_t4096" % B: {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10,
                                        "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                        "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                        "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1),

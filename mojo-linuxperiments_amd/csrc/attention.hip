@@ -131,17 +131,18 @@ __device__ __forceinline__ void fold_slots(float (&p)[64], int lane)
     }
 }
 
-#ifndef MI_ATTN_TILES
-#define MI_ATTN_TILES 11
-#endif
-constexpr int WAVE_TILES = MI_ATTN_TILES;   // 16-token tiles per wave: a workgroup covers at most 4 * WAVE_TILES * 16 tokens
-constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each)
+// 16-token tiles per wave: a workgroup covers at most 4 * tiles * 16 tokens.  Every wave runs through all of its
+// tiles (the ones past the end masked), so a workgroup wants a span it can fill: 11 tiles (704 tokens) when there
+// are (batch, kv head) rows enough to occupy the chip with such spans, 4 tiles (256 tokens) when there are few rows
+// and the cache has to be cut finer to give every compute unit work.
+constexpr int TILES_LONG = 11, TILES_SHORT = 4;
+constexpr int RING = 8;           // loads a wave keeps in flight (1 KB each); tiles per wave >= RING / 2
 
 // RAGGED: the span a workgroup can cover runs past the end of the cache and token indices are clamped for the
 // loads; otherwise every address is base + constant.  Tokens past the end of the split are masked in the scores.
 // PAGED: the cache is a pool of pages [page][kv head][P tokens][128]; a 16-token tile lies in one page, so a wave
 // looks up one page per tile (uniform over the wave) and lanes are clamped inside their tile.
-template <bool DUMP, bool RAGGED, bool PAGED = false>
+template <bool DUMP, bool RAGGED, bool PAGED, int WAVE_TILES>
 __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int8_t (&s_q)[4][4][D], float (&s_sq)[4][4],
                                                float (&s_red)[4][4][D], float (&s_sc)[4][WAVE_TILES][16][4],
                                                float (&s_m)[4][4], float (&s_l)[4][4], float (&s_c)[4][4])
@@ -392,7 +393,7 @@ __device__ __forceinline__ void gqa_split_body(const Params &p, const int T, int
     }
 }
 
-template <bool DUMP>
+template <bool DUMP, int WAVE_TILES>
 __global__ __launch_bounds__(256) void k_gqa_split(Params p)
 {
     __shared__ __attribute__((aligned(16))) int8_t s_q[4][4][D];
@@ -418,12 +419,12 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
         }
     }
     if (p.block_table) {
-        gqa_split_body<false, true, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+        gqa_split_body<false, true, true, WAVE_TILES>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
         return;
     }
     const bool full = (tile_lo + 4 * WAVE_TILES) * 16 <= T;
-    if (full) gqa_split_body<DUMP, false>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
-    else gqa_split_body<DUMP, true>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+    if (full) gqa_split_body<DUMP, false, false, WAVE_TILES>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
+    else gqa_split_body<DUMP, true, false, WAVE_TILES>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
 }
 
 // Merge of the splits of one (b, h) row by the 16 lanes that own it (lane j: elements 4j..4j+3 and 64+4j..).
@@ -462,18 +463,36 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ part_o, cons
             v[6] = __builtin_fmaf(hi[s].z, w, v[6]); v[7] = __builtin_fmaf(hi[s].w, w, v[7]);
         }
     } else {
+        // any split count: the maxima first (one round trip), then the partials in batches of eight whose loads all
+        // go out before the first use
         float mx = -INFINITY;
-        for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml0[s * 8 + hl]);
-        for (int s = 0; s < splits; ++s) {
-            const float ms = ml0[s * 8 + hl];
-            const float w = (ms == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);   // empty split
-            l = __builtin_fmaf(ml0[s * 8 + 4 + hl], w, l);
-            const float4 lo = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
-            const float4 hi = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
-            v[0] = __builtin_fmaf(lo.x, w, v[0]); v[1] = __builtin_fmaf(lo.y, w, v[1]);
-            v[2] = __builtin_fmaf(lo.z, w, v[2]); v[3] = __builtin_fmaf(lo.w, w, v[3]);
-            v[4] = __builtin_fmaf(hi.x, w, v[4]); v[5] = __builtin_fmaf(hi.y, w, v[5]);
-            v[6] = __builtin_fmaf(hi.z, w, v[6]); v[7] = __builtin_fmaf(hi.w, w, v[7]);
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float ms[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ms[i] = ml0[min(s0 + i, splits - 1) * 8 + hl];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mx = fmaxf(mx, ms[i]);
+        }
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float ms[8], ls[8];
+            float4 lo[8], hi[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int s = min(s0 + i, splits - 1);
+                ms[i] = ml0[s * 8 + hl];
+                ls[i] = ml0[s * 8 + 4 + hl];
+                lo[i] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
+                hi[i] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float w = (s0 + i >= splits || ms[i] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[i] - mx);
+                l = __builtin_fmaf(ls[i], w, l);
+                v[0] = __builtin_fmaf(lo[i].x, w, v[0]); v[1] = __builtin_fmaf(lo[i].y, w, v[1]);
+                v[2] = __builtin_fmaf(lo[i].z, w, v[2]); v[3] = __builtin_fmaf(lo[i].w, w, v[3]);
+                v[4] = __builtin_fmaf(hi[i].x, w, v[4]); v[5] = __builtin_fmaf(hi[i].y, w, v[5]);
+                v[6] = __builtin_fmaf(hi[i].z, w, v[6]); v[7] = __builtin_fmaf(hi[i].w, w, v[7]);
+            }
         }
     }
     const float rl = l > 0.0f ? 1.0f / l : 0.0f;   // a sequence of length 0 gives a row of zeros
@@ -542,16 +561,25 @@ __global__ __launch_bounds__(1024) void k_gqa_merge_quant(const float *__restric
     }
 }
 
-static int pick_splits(int64_t B, int64_t Hkv, int64_t T)
+struct SplitPlan {
+    int splits, wave_tiles;
+};
+
+static SplitPlan pick_splits(int64_t B, int64_t Hkv, int64_t T)
 {
     const int ntiles = (int)((T + 15) / 16);
     const int cus = compute_units();
-    constexpr int MAX_TILES = 4 * WAVE_TILES;   // 16-token tiles one workgroup can hold in registers
-    int splits = (ntiles + MAX_TILES - 1) / MAX_TILES;
-    // short caches / few heads: more, shorter splits until there are about two workgroups per compute unit
-    while (B * Hkv * splits < 2LL * cus && (ntiles + splits - 1) / splits > 8) splits *= 2;
-    if (splits > ntiles) splits = ntiles;
-    return splits;
+    SplitPlan pl;
+    pl.wave_tiles = TILES_LONG;
+    pl.splits = (ntiles + 4 * TILES_LONG - 1) / (4 * TILES_LONG);
+    if (B * Hkv * pl.splits < cus && ntiles > 4 * TILES_SHORT) {
+        // few rows: spans of 256 tokens, then halves of them while that still doubles the number of busy compute units
+        pl.wave_tiles = TILES_SHORT;
+        pl.splits = (ntiles + 4 * TILES_SHORT - 1) / (4 * TILES_SHORT);
+        while (B * Hkv * pl.splits < cus && (ntiles + pl.splits - 1) / pl.splits > 8) pl.splits *= 2;
+    }
+    if (pl.splits > ntiles) pl.splits = ntiles;
+    return pl;
 }
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -574,7 +602,7 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
 {
     int32_t rc = check_attn(B, Hq, Hkv, D, T);
     if (rc) return rc;
-    const int splits = attn::pick_splits(B, Hkv, T);
+    const int splits = attn::pick_splits(B, Hkv, T).splits;
     return attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256) + attn::align_up(B * Hkv * splits * 8 * 4, 256);
 }
 
@@ -591,7 +619,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     if (!aligned16(q) || !aligned16(kq) || !aligned16(vq) || !aligned4(ks) || !aligned4(vs) || !aligned16(workspace))
         return MI_EINVAL;
     if (workspace_bytes < mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T)) return MI_ENOSPC;
-    const int splits = attn::pick_splits(B, Hkv, T);
+    const attn::SplitPlan plan = attn::pick_splits(B, Hkv, T);
+    const int splits = plan.splits;
     const int ntiles = (int)((T + 15) / 16);
     attn::Params p;
     p.q = q; p.kq = kq; p.ks = ks; p.vq = vq; p.vs = vs;
@@ -606,8 +635,13 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     p.tiles_per_split = (ntiles + splits - 1) / splits;
     p.score_scale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
     const dim3 grid((unsigned)splits, (unsigned)(B * Hkv));
-    if (ddots) hipLaunchKernelGGL(attn::k_gqa_split<true>, grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL(attn::k_gqa_split<false>, grid, dim3(256), 0, s, p);
+    if (plan.wave_tiles == attn::TILES_LONG) {
+        if (ddots) hipLaunchKernelGGL((attn::k_gqa_split<true, attn::TILES_LONG>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((attn::k_gqa_split<false, attn::TILES_LONG>), grid, dim3(256), 0, s, p);
+    } else {
+        if (ddots) hipLaunchKernelGGL((attn::k_gqa_split<true, attn::TILES_SHORT>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((attn::k_gqa_split<false, attn::TILES_SHORT>), grid, dim3(256), 0, s, p);
+    }
     rc = launch_status();
     if (rc) return rc;
     if (oq) {
@@ -621,6 +655,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
         case 4: MI_MERGEQ(4); break;
         case 6: MI_MERGEQ(6); break;
         case 8: MI_MERGEQ(8); break;
+        case 12: MI_MERGEQ(12); break;
+        case 16: MI_MERGEQ(16); break;
         default: MI_MERGEQ(0); break;
         }
 #undef MI_MERGEQ
@@ -638,6 +674,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     case 4: MI_MERGE(4); break;
     case 6: MI_MERGE(6); break;
     case 8: MI_MERGE(8); break;
+    case 12: MI_MERGE(12); break;
+    case 16: MI_MERGE(16); break;
     default: MI_MERGE(0); break;
     }
 #undef MI_MERGE
