@@ -313,6 +313,15 @@ MI_API int32_t mi_rmsnorm_quant_f32_i8(const float *x, const float *residual, co
                                        int64_t M, int64_t H, int32_t block, void *stream);
 MI_API int32_t mi_swiglu_quant_f32_i8(const float *gate_up, float *h_out, int8_t *q, float *scale,
                                       int64_t M, int64_t I, int32_t block, void *stream);
+/* (residual +) RMSNorm + rotate + quantize + W8A8 contraction + dequant as one call: y = linear(rmsnorm(x (+ residual))).
+ * For one token and K in {2048, 4096} (block 128) it is ONE kernel (the GEMV normalizes and quantizes the row
+ * itself); any other shape runs mi_rmsnorm_quant_f32_i8 and the contraction.  workspace as for mi_w8a8_linear_f32
+ * (it receives the codes and the scale); h_out (the residual sum, required with a residual) and xn_out (the
+ * normalized row, optional) as in mi_rmsnorm_quant_f32_i8. */
+MI_API int32_t mi_rmsnorm_linear_f32(const float *x, const float *residual, const float *g, float eps,
+                                     float *h_out, float *xn_out, const int8_t *qw, const float *sw, float *y,
+                                     int64_t M, int64_t N, int64_t K, int32_t block,
+                                     void *workspace, int64_t workspace_bytes, void *stream);
 /* out = a + b over n floats (n % 4 == 0): the residual add that closes the layer. */
 MI_API int32_t mi_add_f32(const float *a, const float *b, float *out, int64_t n, void *stream);
 

@@ -12,6 +12,8 @@ int32_t launch_tiled(const int8_t *, const float *, const int8_t *, const float 
 
 int32_t launch_linear_fused(const float *, const int8_t *, const float *, float *, int8_t *, float *, int64_t, int64_t,
                             int64_t, hipStream_t);
+int32_t launch_norm_linear_fused(const float *, const float *, const float *, float, float *, float *, const int8_t *,
+                                 const float *, float *, int8_t *, float *, int64_t, int64_t, int64_t, hipStream_t);
 
 __global__ void k_dequant(const int32_t *__restrict__ acc, const float *__restrict__ sx,
                           const float *__restrict__ sw, float *__restrict__ y, int64_t M, int64_t N)
@@ -83,6 +85,29 @@ extern "C" int64_t mi_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t 
     (void)N;
     if (M < 0 || K <= 0) return MI_EINVAL;
     return align_up(M * K, 256) + align_up(M * 4, 256);
+}
+
+extern "C" int32_t mi_rmsnorm_linear_f32(const float *x, const float *residual, const float *g, float eps,
+                                         float *h_out, float *xn_out, const int8_t *qw, const float *sw, float *y,
+                                         int64_t M, int64_t N, int64_t K, int32_t block, void *workspace,
+                                         int64_t workspace_bytes, void *stream)
+{
+    if (!workspace || !aligned16(workspace)) return MI_EINVAL;
+    if (workspace_bytes < mi_w8a8_linear_workspace_bytes(M, N, K)) return MI_ENOSPC;
+    int8_t *qx = static_cast<int8_t *>(workspace);
+    float *sx = reinterpret_cast<float *>(qx + align_up(M * K, 256));
+    int32_t rc = check_gemm(qx, qw, y, M, N, K);
+    if (rc) return rc;
+    if (!x || !g || !sw || !aligned16(sw) || !aligned16(x) || !aligned16(g) || !(eps >= 0.0f)) return MI_EINVAL;
+    if (residual && (!h_out || !aligned16(residual) || !aligned16(h_out))) return MI_EINVAL;
+    if (xn_out && !aligned16(xn_out)) return MI_EINVAL;
+    if (M == 1 && block == 128) {
+        rc = launch_norm_linear_fused(x, residual, g, eps, h_out, xn_out, qw, sw, y, qx, sx, M, N, K, as_stream(stream));
+        if (rc != MI_EINVAL) return rc;
+    }
+    rc = mi_rmsnorm_quant_f32_i8(x, residual, g, eps, h_out, xn_out, qx, sx, M, K, block, stream);
+    if (rc) return rc;
+    return gemm_dispatch(qx, sx, qw, sw, nullptr, y, M, N, K, as_stream(stream));
 }
 
 extern "C" int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const float *sw, float *y, int64_t M,

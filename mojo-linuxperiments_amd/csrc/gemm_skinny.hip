@@ -151,11 +151,20 @@ __global__ __launch_bounds__(256) void k_gemv_reg(const int8_t *__restrict__ qx,
 // go out first; while they are in flight the workgroup rotates and quantizes the M activation rows (the same
 // per-chunk code as the stand-alone quantizer, so the codes and scales are bit-identical), parks the codes in
 // LDS and every lane picks up its share.  One launch per linear instead of two.
-template <int MB, int CW, int CQ>
+// NORM: the row is first normalized, v = ((x (+ res)) * r) * g with r = 1 / sqrt(mean((x + res)^2) + eps), the
+// arithmetic of the stand-alone RMSNorm + quantize kernel; workgroup 0 also leaves the residual sum (h_out) and, on
+// request, the normalized row (xn_out) for the caller.
+struct FusedNorm {
+    const float *res, *g;
+    float *h_out, *xn_out;
+    float eps;
+};
+
+template <int MB, int CW, int CQ, bool NORM>
 __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x, const int8_t *__restrict__ qw,
                                                     const float *__restrict__ sw, float *__restrict__ y,
                                                     int8_t *__restrict__ qx_out, float *__restrict__ sx_out, int M,
-                                                    int N, int K, int QW)
+                                                    int N, int K, int QW, FusedNorm nm)
 {
     constexpr int BLOCK = 128, LPB = BLOCK / 8;
     constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);   // rows per wave
@@ -163,8 +172,8 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
     extern __shared__ __attribute__((aligned(16))) char s_dyn[];
     int8_t *s_x = reinterpret_cast<int8_t *>(s_dyn);                       // [MB][K] codes
     float *s_scale = reinterpret_cast<float *>(s_dyn + (size_t)MB * K);    // [MB]
-    float *s_max = s_scale + MB;                                           // [4]
-    int *s_red = reinterpret_cast<int *>(s_max + 4);                       // [4][V]
+    float *s_max = s_scale + MB;                                           // [4] row maxima, then [4] sums of squares
+    int *s_red = reinterpret_cast<int *>(s_max + 8);                       // [4][V]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = wave % QW;                  // which CW-chunk slice of the row
     const int rows_per_wg = (4 / QW) * R;
@@ -202,6 +211,52 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
                 for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
             }
         }
+        const bool keeper = blockIdx.x == 0;   // one workgroup also leaves the codes and scales in the caller's workspace
+        if constexpr (NORM) {
+            float4 gl[CQ], gh[CQ];
+            float ss = 0.0f;
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                if (tid + i * 256 < nchunk) {
+                    gl[i] = *reinterpret_cast<const float4 *>(nm.g + base[i]);
+                    gh[i] = *reinterpret_cast<const float4 *>(nm.g + base[i] + BLOCK / 2);
+                    if (nm.res) {
+                        const float *rr = nm.res + (int64_t)m * K + base[i];
+                        const float4 rl = *reinterpret_cast<const float4 *>(rr), rh = *reinterpret_cast<const float4 *>(rr + BLOCK / 2);
+                        v[i][0] = v[i][0] + rl.x; v[i][1] = v[i][1] + rl.y; v[i][2] = v[i][2] + rl.z; v[i][3] = v[i][3] + rl.w;
+                        v[i][4] = v[i][4] + rh.x; v[i][5] = v[i][5] + rh.y; v[i][6] = v[i][6] + rh.z; v[i][7] = v[i][7] + rh.w;
+                        if (keeper) {
+                            float *ho = nm.h_out + (int64_t)m * K + base[i];
+                            *reinterpret_cast<float4 *>(ho) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+                            *reinterpret_cast<float4 *>(ho + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+                }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            __syncthreads();   // the previous row's sums have been read
+            if (lane == 0) s_max[4 + wave] = ss;
+            __syncthreads();
+            const float total = (s_max[4] + s_max[5]) + (s_max[6] + s_max[7]);
+            const float r = 1.0f / sqrtf(total / (float)K + nm.eps);
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                if (tid + i * 256 < nchunk) {
+                    v[i][0] = (v[i][0] * r) * gl[i].x; v[i][1] = (v[i][1] * r) * gl[i].y;
+                    v[i][2] = (v[i][2] * r) * gl[i].z; v[i][3] = (v[i][3] * r) * gl[i].w;
+                    v[i][4] = (v[i][4] * r) * gh[i].x; v[i][5] = (v[i][5] * r) * gh[i].y;
+                    v[i][6] = (v[i][6] * r) * gh[i].z; v[i][7] = (v[i][7] * r) * gh[i].w;
+                    if (keeper && nm.xn_out) {
+                        float *xo = nm.xn_out + (int64_t)m * K + base[i];
+                        *reinterpret_cast<float4 *>(xo) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+                        *reinterpret_cast<float4 *>(xo + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+                    }
+                }
+            }
+        }
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < CQ; ++i) {
@@ -218,7 +273,6 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
         const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
         if (tid == 0) s_scale[m] = sc;
         int8_t *qrow = s_x + (size_t)m * K;
-        const bool keeper = blockIdx.x == 0;   // one workgroup also leaves the codes and scales in the caller's workspace
         if (keeper && tid == 0) sx_out[m] = sc;
 #pragma unroll
         for (int i = 0; i < CQ; ++i) {
@@ -280,22 +334,23 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
     }
 }
 
-template <int MB, int CW, int CQ>
+template <int MB, int CW, int CQ, bool NORM>
 static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx, int M,
-                            int N, int K, int QW, hipStream_t s)
+                            int N, int K, int QW, const FusedNorm &nm, hipStream_t s)
 {
     constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);
     constexpr int V = pow2_ceil(R * MB);
-    const size_t lds = (size_t)MB * K + (MB + 4) * sizeof(float) + 4 * V * sizeof(int);
+    const size_t lds = (size_t)MB * K + (MB + 8) * sizeof(float) + 4 * V * sizeof(int);
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ>),
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ, NORM>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
         attr_set = true;
     }
     const int rows_per_wg = (4 / QW) * R;
     const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
-    hipLaunchKernelGGL((k_gemv_fused<MB, CW, CQ>), dim3(grid), dim3(256), lds, s, x, qw, sw, y, qx, sx, M, N, K, QW);
+    hipLaunchKernelGGL((k_gemv_fused<MB, CW, CQ, NORM>), dim3(grid), dim3(256), lds, s, x, qw, sw, y, qx, sx, M, N, K,
+                       QW, nm);
     return launch_status();
 }
 
@@ -309,8 +364,23 @@ int32_t launch_linear_fused(const float *x, const int8_t *qw, const float *sw, f
     const int M = (int)M64, N = (int)N64, K = (int)K64;
     if (M != 1 || K % 1024) return MI_EINVAL;
     const int nchunk = K >> 10;
-    if (nchunk == 4) return launch_fused<1, 4, 2>(x, qw, sw, y, qx, sx, M, N, K, 1, s);   // K = 4096
-    if (nchunk == 2) return launch_fused<1, 2, 1>(x, qw, sw, y, qx, sx, M, N, K, 1, s);   // K = 2048
+    const FusedNorm none = {nullptr, nullptr, nullptr, nullptr, 0.0f};
+    if (nchunk == 4) return launch_fused<1, 4, 2, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 4096
+    if (nchunk == 2) return launch_fused<1, 2, 1, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 2048
+    return MI_EINVAL;
+}
+
+// The same with the (residual +) RMSNorm ahead of the quantizer: one launch for norm + quantize + GEMV of one token.
+int32_t launch_norm_linear_fused(const float *x, const float *res, const float *g, float eps, float *h_out,
+                                 float *xn_out, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx,
+                                 int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
+{
+    const int M = (int)M64, N = (int)N64, K = (int)K64;
+    if (M != 1 || K % 1024) return MI_EINVAL;
+    const int nchunk = K >> 10;
+    const FusedNorm nm = {res, g, h_out, xn_out, eps};
+    if (nchunk == 4) return launch_fused<1, 4, 2, true>(x, qw, sw, y, qx, sx, M, N, K, 1, nm, s);
+    if (nchunk == 2) return launch_fused<1, 2, 1, true>(x, qw, sw, y, qx, sx, M, N, K, 1, nm, s);
     return MI_EINVAL;
 }
 

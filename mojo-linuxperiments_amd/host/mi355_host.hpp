@@ -275,7 +275,7 @@ struct PagedKvCache {
     }
 };
 
-// One decoder layer of a decode step (one new token per sequence), chained on one stream, ten launches:
+// One decoder layer of a decode step (one new token per sequence), chained on one stream, ten launches (eight for a single sequence):
 // (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache (split, merge +
 // quantize: the output projection takes the rows in the rotated basis of V) -> O GEMV -> residual + RMSNorm +
 // quantize -> gate|up GEMV -> SwiGLU + quantize -> down GEMV (-> residual).
@@ -290,9 +290,10 @@ struct DecoderLayer {
     // attention (h1), down output (dn); xn / att (rotated basis) / hn / act only when prepare() was asked to trace
     float *h0 = nullptr, *qkv_out = nullptr, *q = nullptr, *ao = nullptr, *h1 = nullptr, *gu = nullptr, *dn = nullptr,
           *xn = nullptr, *att = nullptr, *hn = nullptr, *act = nullptr;
-    // codes of the normalized rows [B,H], of the attention rows [B,Hq*128] and of the activated rows [B,I]
-    int8_t *cx = nullptr, *ca = nullptr, *ci = nullptr;
-    float *sx = nullptr, *sa = nullptr, *si = nullptr;
+    // codes of the attention rows [B,Hq*128] and of the activated rows [B,I] (those of the normalized rows sit in
+    // the workspaces of the QKV and gate|up projections)
+    int8_t *ca = nullptr, *ci = nullptr;
+    float *sa = nullptr, *si = nullptr;
 
     // fp32 weights in device memory: wqkv [(Hq+2Hkv)*128, H], wo [H, Hq*128], wgu [2I, H] (gate rows, then up
     // rows), wd [H, I]; norm weights g1, g2 [H]; rotary tables [T_cap, 64].  false if the arena is exhausted.
@@ -315,10 +316,8 @@ struct DecoderLayer {
         h1 = arena.template alloc<float>(B * H);
         gu = arena.template alloc<float>(B * 2 * I);
         dn = arena.template alloc<float>(B * H);
-        cx = arena.template alloc<int8_t>(B * H);
         ca = arena.template alloc<int8_t>(B * Hq * 128);
         ci = arena.template alloc<int8_t>(B * I);
-        sx = arena.template alloc<float>(B);
         sa = arena.template alloc<float>(B);
         si = arena.template alloc<float>(B);
         if (trace) {
@@ -328,7 +327,7 @@ struct DecoderLayer {
             act = arena.template alloc<float>(B * I);
             ok = ok && xn && att && hn && act;
         }
-        return ok && h0 && qkv_out && q && ao && h1 && gu && dn && cx && ca && ci && sx && sa && si;
+        return ok && h0 && qkv_out && q && ao && h1 && gu && dn && ca && ci && sa && si;
     }
     // x fp32 [B,H], plus residual fp32 [B,H] or nullptr: the layer input is their sum (left in h0).  pos, seq_len
     // int32 [B] in device memory (seq_len = pos + 1 in a plain decode step); t_max bounds seq_len.  out fp32 [B,H],
@@ -337,9 +336,10 @@ struct DecoderLayer {
     int32_t step(const float *x, const float *residual, const int32_t *pos, const int32_t *seq_len, int64_t t_max,
                  float *out, void *stream) const
     {
-        int32_t rc = mi_rmsnorm_quant_f32_i8(x, residual, g1, eps, residual ? h0 : nullptr, xn, cx, sx, B, H, 128, stream);
+        // norm + quantize + projection: one kernel for a single token, two launches otherwise
+        int32_t rc = mi_rmsnorm_linear_f32(x, residual, g1, eps, residual ? h0 : nullptr, xn, qkv.qw, qkv.sw, qkv_out, B,
+                                           qkv.N, H, 128, qkv.workspace, qkv.workspace_bytes, stream);
         const float *xin = residual ? h0 : x;
-        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(cx, sx, qkv.qw, qkv.sw, qkv_out, B, qkv.N, H, stream);
         if (rc == MI_OK)
             rc = mi_rope_kv_append_f32_i8(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, cache.kq, cache.ks,
                                           cache.vq, cache.vs, pos, B, Hq, Hkv, 128, T_cap, stream);
@@ -347,8 +347,9 @@ struct DecoderLayer {
             rc = mi_gqa_decode_attn_cache_quant_i8(q, cache.kq, cache.ks, cache.vq, cache.vs, att, ca, sa, B, Hq, Hkv, 128,
                                                    T_cap, seq_len, t_max, cache.workspace, cache.workspace_bytes, stream);
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
-        if (rc == MI_OK) rc = mi_rmsnorm_quant_f32_i8(ao, xin, g2, eps, h1, hn, cx, sx, B, H, 128, stream);
-        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(cx, sx, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, stream);
+        if (rc == MI_OK)
+            rc = mi_rmsnorm_linear_f32(ao, xin, g2, eps, h1, hn, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, 128,
+                                       gate_up.workspace, gate_up.workspace_bytes, stream);
         if (rc == MI_OK) rc = mi_swiglu_quant_f32_i8(gu, act, ci, si, B, I, 128, stream);
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ci, si, down.qw, down.sw, dn, B, H, I, stream);
         if (rc == MI_OK && out) rc = mi_add_f32(h1, dn, out, B * H, stream);

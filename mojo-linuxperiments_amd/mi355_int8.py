@@ -93,6 +93,7 @@ SIGNATURES = {
     "mi_rope_kv_append_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
     "mi_swiglu_f32": (i32, [vp, vp, i64, i64, vp]),
     "mi_rmsnorm_quant_f32_i8": (i32, [vp, vp, vp, C.c_float, vp, vp, vp, vp, i64, i64, i32, vp]),
+    "mi_rmsnorm_linear_f32": (i32, [vp, vp, vp, C.c_float, vp, vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
     "mi_swiglu_quant_f32_i8": (i32, [vp, vp, vp, vp, i64, i64, i32, vp]),
     "mi_add_f32": (i32, [vp, vp, vp, i64, vp]),
     "mi_gqa_decode_attn_cache_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, vp,
@@ -416,7 +417,7 @@ class DecoderLayer:
         self.xn = dev.empty((B, H), f) if trace else None
         self.hn = dev.empty((B, H), f) if trace else None
         self.act = dev.empty((B, I), f) if trace else None
-        self.cx, self.sx = dev.empty((B, H), np.int8), dev.empty(B, f)        # codes of the normalized rows
+        self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, 2 * I, H), np.uint8)   # codes of the normalized rows
         self.ci, self.si = dev.empty((B, I), np.int8), dev.empty(B, f)        # codes of the activated rows
         self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
 
@@ -426,11 +427,12 @@ class DecoderLayer:
         residual add is left to the next layer (pass x=self.dn, residual=self.h1 to its step)."""
         B, H, Hq, Hkv, I, D, s = self.B, self.H, self.Hq, self.Hkv, self.I, 128, stream
         p = lambda b: b.ptr if b is not None else None
-        check(lib.mi_rmsnorm_quant_f32_i8(x.ptr, p(residual), self.g1.ptr, self.eps,
-                                          self.h0.ptr if residual is not None else None, p(self.xn), self.cx.ptr,
-                                          self.sx.ptr, B, H, self.block, s), "mi_rmsnorm_quant_f32_i8")
+        # norm + quantize + projection: one kernel for a single token, two launches otherwise
+        check(lib.mi_rmsnorm_linear_f32(x.ptr, p(residual), self.g1.ptr, self.eps,
+                                        self.h0.ptr if residual is not None else None, p(self.xn), self.wqkv[0].ptr,
+                                        self.wqkv[1].ptr, self.qkv.ptr, B, self.NQKV, H, self.block, self.lin_ws.ptr,
+                                        self.lin_ws.nbytes, s), "mi_rmsnorm_linear_f32")
         xin = self.h0 if residual is not None else x
-        gemm_dequant(self.cx, self.sx, self.wqkv[0], self.wqkv[1], self.qkv, s)
         check(lib.mi_rope_kv_append_f32_i8(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr,
                                            self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv,
                                            D, self.T_cap, s), "mi_rope_kv_append_f32_i8")
@@ -441,9 +443,9 @@ class DecoderLayer:
                                                     seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
               "mi_gqa_decode_attn_cache_quant_i8")
         gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
-        check(lib.mi_rmsnorm_quant_f32_i8(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
-                                          self.cx.ptr, self.sx.ptr, B, H, self.block, s), "mi_rmsnorm_quant_f32_i8")
-        gemm_dequant(self.cx, self.sx, self.wgu[0], self.wgu[1], self.gu, s)
+        check(lib.mi_rmsnorm_linear_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
+                                        self.wgu[0].ptr, self.wgu[1].ptr, self.gu.ptr, B, 2 * I, H, self.block,
+                                        self.lin_ws.ptr, self.lin_ws.nbytes, s), "mi_rmsnorm_linear_f32")
         check(lib.mi_swiglu_quant_f32_i8(self.gu.ptr, p(self.act), self.ci.ptr, self.si.ptr, B, I, self.block, s),
               "mi_swiglu_quant_f32_i8")
         gemm_dequant(self.ci, self.si, self.wd[0], self.wd[1], self.dn, s)

@@ -174,6 +174,8 @@ def oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=None):
     (4, 1024, 8, 2, 2048, 64, [0, 10, 40, 61]),
     (2, 4096, 32, 8, 14336, 300, [150, 297]),
     (16, 4096, 32, 8, 14336, 128, list(range(100, 116))),
+    (1, 4096, 32, 8, 14336, 600, [500]),          # one sequence: the norm-fused GEMVs and the short attention spans
+    (1, 2048, 8, 2, 1024, 40, [7]),
 ])
 def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, Hq, Hkv, I, T_cap, start):
     mark = dev.mark()
@@ -282,4 +284,44 @@ def test_fused_swiglu_quant_equals_the_two_calls(mi, dev, orc, M, I, block):
     mi.check(mi.lib.mi_swiglu_quant_f32_i8(dgu.ptr, None, dq.ptr, ds.ptr, M, I, block, None))
     assert np.array_equal(dev.download(dq), qo) and np.array_equal(dev.download(ds), so)
     assert mi.lib.mi_swiglu_quant_f32_i8(dgu.ptr, None, dq.ptr, ds.ptr, M, I + 4, block, None) == mi.EINVAL
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (1, 28672, 4096), (1, 272, 2048), (1, 512, 1024), (3, 1024, 4096),
+                                   (16, 512, 14336)])
+def test_rmsnorm_linear_one_call(mi, dev, orc, M, N, K):
+    """One token and K in {2048, 4096}: a single kernel; other shapes: norm + quantize, then the contraction.  Either
+    way the normalized row follows the RMSNorm oracle, the codes are the oracle quantizer's on that row and the
+    output is the oracle's contraction of those codes, exactly."""
+    mark = dev.mark()
+    g = np.random.default_rng(M + N + K)
+    x = workload.activations(71, M, K)
+    r = g.standard_normal((M, K)).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(K)).astype(np.float32)
+    qw = g.integers(-127, 128, (N, K)).astype(np.int8)
+    sw = ((g.random(N) + 0.5) * 0.01).astype(np.float32)
+    dx, dr, dg, dqw, dsw = dev.upload(x), dev.upload(r), dev.upload(w), dev.upload(qw), dev.upload(sw)
+    dh, dxn, dy = dev.empty((M, K), np.float32), dev.empty((M, K), np.float32), dev.empty((M, N), np.float32)
+    ws = dev.empty(mi.lib.mi_w8a8_linear_workspace_bytes(M, N, K), np.uint8)
+    for res in (None, dr):
+        for want_xn in (True, False):
+            mi.check(mi.lib.mi_rmsnorm_linear_f32(dx.ptr, res.ptr if res else None, dg.ptr, 1e-5, dh.ptr if res else None,
+                                                  dxn.ptr if want_xn else None, dqw.ptr, dsw.ptr, dy.ptr, M, N, K, 128,
+                                                  ws.ptr, ws.nbytes, None), "mi_rmsnorm_linear_f32")
+            y = dev.download(dy)
+            xin = x + r if res else x
+            if res:
+                assert np.array_equal(dev.download(dh), xin)
+            if want_xn:
+                xn = dev.download(dxn)
+                ref = orc.rmsnorm(xin, w, 1e-5)
+                assert np.max(np.abs(xn - ref)) <= 2e-6 * np.max(np.abs(ref))
+                want = orc.w8a8_linear(xn, qw, sw, 128)
+                assert np.array_equal(dev.download(ws.offset(0, (M, K), np.int8)), want[1])
+                y_first = y
+                assert np.array_equal(y, want[0])
+            else:
+                assert np.array_equal(y, y_first)          # leaving the fp32 row out changes nothing
+    assert mi.lib.mi_rmsnorm_linear_f32(dx.ptr, dr.ptr, dg.ptr, 1e-5, None, None, dqw.ptr, dsw.ptr, dy.ptr, M, N, K, 128,
+                                        ws.ptr, ws.nbytes, None) == mi.EINVAL     # residual without h_out
     dev.reset_to(mark)
