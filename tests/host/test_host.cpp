@@ -136,8 +136,15 @@ static void test_stream_pool(const Context &ctx)
     uint32_t *big = arena.alloc<uint32_t>(8 << 20);
     int launched = 0;
     bool saw_full = false;
+    // each launch is a run of fills (about a millisecond of device work), so that no slot can finish while the
+    // host is still filling the pool
+    auto long_fill = [&](void *s) {
+        int32_t rc = MI_OK;
+        for (int r = 0; r < 100 && rc == MI_OK; ++r) rc = mi_fill_u32(big, 7u, (int64_t)(8 << 20), s);
+        return rc;
+    };
     for (int i = 0; i < 64; ++i) {
-        if (pool.launch(fill_op, big, 7u, (int64_t)(8 << 20))) ++launched;
+        if (pool.launch(long_fill)) ++launched;
         else { saw_full = true; break; }
     }
     int completed = 0;
