@@ -484,7 +484,7 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None):
     wbytes = ((Hq + 2 * Hkv) * D * H + H * Hq * D + 2 * I * H + H * I)
     nbytes = wbytes + wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
     dev.reset_to(mark)
-    return {"decode_layer_b%d_t4096" % B: {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10,
+    return {"decode_layer_b%d_t4096" % B: {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10 if B > 1 else 8,
                                        "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                        "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                        "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1),
