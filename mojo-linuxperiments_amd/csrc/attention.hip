@@ -576,7 +576,7 @@ static SplitPlan pick_splits(int64_t B, int64_t Hkv, int64_t T)
         // few rows: spans of 256 tokens, then halves of them while that still doubles the number of busy compute units
         pl.wave_tiles = TILES_SHORT;
         pl.splits = (ntiles + 4 * TILES_SHORT - 1) / (4 * TILES_SHORT);
-        while (B * Hkv * pl.splits < cus && (ntiles + pl.splits - 1) / pl.splits > 8) pl.splits *= 2;
+        while (B * Hkv * pl.splits < cus && (ntiles + pl.splits - 1) / pl.splits > 8 && pl.splits * 2 <= 16) pl.splits *= 2;
     }
     if (pl.splits > ntiles) pl.splits = ntiles;
     return pl;
