@@ -73,7 +73,7 @@ def test_linear_random_shapes(mi, dev, orc):
 def test_attention_random_shapes_and_lengths(mi, dev, orc):
     g = np.random.default_rng(6)
     for it in range(16):
-        Hkv, G = int(g.choice([1, 2, 3, 8])), int(g.choice([1, 2, 4]))
+        Hkv, G = int(g.choice([1, 2, 3, 8])), int(g.choice([1, 2, 3, 4]))
         Hq, B, T_cap = Hkv * G, int(g.integers(1, 5)), int(g.integers(1, 1500))
         lens = g.integers(0, T_cap + 1, B).astype(np.int32)
         lens[0] = T_cap
