@@ -462,7 +462,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
                                                          const int8_t *__restrict__ w0, const float *__restrict__ sc0,
                                                          const int8_t *__restrict__ w1, const float *__restrict__ sc1,
                                                          float *__restrict__ out, int Kdim, int Nrows, int Hout,
-                                                         int topk, int nch, int e)
+                                                         int topk, int nch, int e, int bx)
 {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -475,7 +475,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     // loads of the next chunk are already in flight while the partial sums of this one are added and stored,
     // and the segment / permutation lookups are paid once per workgroup.
     constexpr int CHUNK_ROWS = DOWN ? 128 : 16;
-    const int n0 = DOWN ? blockIdx.x * nch * 128 + wave * 32 : blockIdx.x * nch * 16;
+    const int n0 = DOWN ? bx * nch * 128 + wave * 32 : bx * nch * 16;
     constexpr int RX_RING = rx_ring(DOWN), RX_RING_BYTES = rx_ring_bytes(DOWN);
     char *ring = smem + wave * (RX_RING * RX_STAGE);
     int *s_red = reinterpret_cast<int *>(smem + RX_RING_BYTES);    // [NGRP][MTT][4][64] sums over the four K slices (gate/up)
@@ -495,10 +495,10 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
         float v = 0.0f;
         if (o < nch * SCW) {
             if constexpr (DOWN) {
-                const int n = (blockIdx.x * nch + ch) * 128 + nl;
+                const int n = (bx * nch + ch) * 128 + nl;
                 if (n < Nrows) v = sc0[(int64_t)e * Nrows + n];
             } else {
-                const int n = (blockIdx.x * nch + ch) * 16 + (nl & 15);
+                const int n = (bx * nch + ch) * 16 + (nl & 15);
                 if (n < Nrows) v = (nl < 16 ? sc0 : sc1)[(int64_t)e * Nrows + n];
             }
         }
@@ -648,7 +648,7 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
         } else {
             // every wave owns its 32 rows over the whole of K: results leave straight from the accumulators, four
             // consecutive channels of one token per lane; out[pair] in pair order
-            const int nbase = (blockIdx.x * nch + ch) * 128;
+            const int nbase = (bx * nch + ch) * 128;
 #pragma unroll
             for (int a = 0; a < NGRP; ++a) {
                 const int nl = wave * 32 + a * 16 + 4 * g_;
@@ -673,6 +673,10 @@ __device__ __forceinline__ void moe_expert_rx_body(const int8_t *__restrict__ ac
     }
 }
 
+// Grid: one dimension.  The first y_split experts of the size order are cut into workgroups of `nch` row chunks,
+// the rest (the smallest segments, which run last: the launcher takes the last eighth) into workgroups of nch / 2
+// chunks: the work that is left when the kernel runs dry then comes in pieces half as long, and the tail of the
+// kernel with them (cfg4: 210 -> 205 us for the layer; halving a quarter or more of the experts gives it back).
 template <bool DOWN, int NSMAX>
 __global__ __launch_bounds__(256) void k_moe_expert_rx(const int8_t *__restrict__ act,
                                                        const float *__restrict__ act_scale,
@@ -681,18 +685,32 @@ __global__ __launch_bounds__(256) void k_moe_expert_rx(const int8_t *__restrict_
                                                        const int8_t *__restrict__ w0, const float *__restrict__ sc0,
                                                        const int8_t *__restrict__ w1, const float *__restrict__ sc1,
                                                        float *__restrict__ out, int Kdim, int Nrows, int Hout,
-                                                       int topk, int nch, const int32_t *__restrict__ order)
+                                                       int topk, int nch, const int32_t *__restrict__ order,
+                                                       int chunks, int y_split)
 {
     // workgroups are handed out in grid order: the experts with the most tokens go first
-    const int e = order[blockIdx.y];
+    const int wpe = (chunks + nch - 1) / nch;
+    int y, bx, nchl;
+    {
+        const int i = blockIdx.x;
+        if (i < y_split * wpe) {
+            y = i / wpe; bx = i - y * wpe; nchl = nch;
+        } else {
+            nchl = nch > 1 ? nch / 2 : 1;
+            const int wpe2 = (chunks + nchl - 1) / nchl;
+            const int j = i - y_split * wpe;
+            y = y_split + j / wpe2; bx = j - (j / wpe2) * wpe2;
+        }
+    }
+    const int e = order[y];
     // tokens per pass follow the size of the expert's segment: every extra pass streams the weights again
     const int count = seg_off[e + 1] - seg_off[e];
     if (count <= 16)
-        moe_expert_rx_body<DOWN, NSMAX, 1>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+        moe_expert_rx_body<DOWN, NSMAX, 1>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nchl, e, bx);
     else if (count <= 32 || NSMAX > 6)
-        moe_expert_rx_body<DOWN, NSMAX, 2>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+        moe_expert_rx_body<DOWN, NSMAX, 2>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nchl, e, bx);
     else
-        moe_expert_rx_body<DOWN, NSMAX, 3>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nch, e);
+        moe_expert_rx_body<DOWN, NSMAX, 3>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nchl, e, bx);
 }
 
 // y[t, n] = sum over slots in order of w[t, slot] * out[t*topk + slot, n]
@@ -859,7 +877,9 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     const int steps_gu = (int)(H / 128), ns_gu = (steps_gu + 3) / 4;   // K steps per wave (the four waves split K)
     if (ns_gu <= 8) {
         const int nch = pick_nch(I / 16);
-        const dim3 grid((unsigned)((I / 16 + nch - 1) / nch), (unsigned)E);
+        const int chunks = (int)(I / 16), y_split = (int)(E - E / 8);
+        const int wpe = (chunks + nch - 1) / nch, nch2 = nch > 1 ? nch / 2 : 1, wpe2 = (chunks + nch2 - 1) / nch2;
+        const dim3 grid((unsigned)(y_split * wpe + (E - y_split) * wpe2));
 #define MI_RX_GU(NS)                                                                                            \
     do {                                                                                                        \
         static bool set = false;                                                                                \
@@ -869,7 +889,7 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
             set = true;                                                                                         \
         }                                                                                                       \
         hipLaunchKernelGGL((moe::k_moe_expert_rx<false, NS>), grid, dim3(256), moe::rx_lds(false), s, qx, sx, perm, seg, \
-                           wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk, nch, order);                   \
+                           wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk, nch, order, chunks, y_split);  \
     } while (0)
         if (ns_gu <= 2) MI_RX_GU(2);
         else if (ns_gu <= 4) MI_RX_GU(4);
@@ -886,9 +906,10 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     if (rc) return rc;
     const int steps_dn = (int)(I / 128);   // every wave walks the whole of K
     if (steps_dn <= 8) {
-        const int64_t chunks = (H + 127) / 128;
-        const int nch = pick_nch(chunks);
-        const dim3 grid((unsigned)((chunks + nch - 1) / nch), (unsigned)E);
+        const int chunks = (int)((H + 127) / 128);
+        const int nch = pick_nch(chunks), y_split = (int)(E - E / 8);
+        const int wpe = (chunks + nch - 1) / nch, nch2 = nch > 1 ? nch / 2 : 1, wpe2 = (chunks + nch2 - 1) / nch2;
+        const dim3 grid((unsigned)(y_split * wpe + (E - y_split) * wpe2));
 #define MI_RX_DN(NS)                                                                                            \
     do {                                                                                                        \
         static bool set = false;                                                                                \
@@ -899,7 +920,7 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
         }                                                                                                       \
         hipLaunchKernelGGL((moe::k_moe_expert_rx<true, NS>), grid, dim3(256), moe::rx_lds(true), s, hq, hs, perm, seg, wd, \
                            sd, (const int8_t *)nullptr, (const float *)nullptr, out, (int)I, (int)H, (int)H,    \
-                           (int)topk, nch, order);                                                              \
+                           (int)topk, nch, order, chunks, y_split);                                             \
     } while (0)
         if (steps_dn <= 2) MI_RX_DN(2);
         else if (steps_dn <= 4) MI_RX_DN(4);
