@@ -76,6 +76,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
 
 #define ORC_API __attribute__((visibility("default")))
 
@@ -160,9 +163,141 @@ static int32_t orc_dot_i8(const int8_t *a, const int8_t *b, int64_t K)
     return s;
 }
 
+#if defined(__x86_64__)
+/* Blocked AVX-512 VNNI form of the same contraction, taken when the host has
+ * the instruction.  vpdpbusd multiplies unsigned by signed bytes, so the
+ * activation codes are biased by +128 (a byte XOR 0x80) and 128 * sum_k qw[n,k]
+ * is taken off again; every partial sum stays below 14336 * 255 * 127 < 2^31,
+ * so the int32 result is the exact contraction, equal to the scalar loop's.
+ * A register tile of 4 activation rows x 6 weight rows holds 24 accumulators;
+ * a panel of 64 activation rows (x 4096 of K) stays in a core's L2 while the
+ * core walks its share of the weight rows. */
+#define ORC_VNNI __attribute__((target("avx512f,avx512bw,avx512vl,avx512vnni")))
+enum { VN_MR = 4, VN_NR = 6, VN_MP = 64, VN_KC = 4096 };
+
+ORC_VNNI static void vnni_tile(const uint8_t *xu, int64_t ldx, const int8_t *w, int64_t ldw,
+                               int64_t kc, int32_t out[VN_MR][VN_NR])
+{
+    /* 24 named accumulators: an array here is kept in memory by the compiler */
+#define VN_DECL(j) __m512i c0##j = _mm512_setzero_si512(), c1##j = c0##j, c2##j = c0##j, c3##j = c0##j;
+#define VN_STEP(j)                                                                   \
+    {                                                                                \
+        const __m512i b = _mm512_loadu_si512((const void *)(w + (j) * ldw + k));     \
+        c0##j = _mm512_dpbusd_epi32(c0##j, a0, b);                                   \
+        c1##j = _mm512_dpbusd_epi32(c1##j, a1, b);                                   \
+        c2##j = _mm512_dpbusd_epi32(c2##j, a2, b);                                   \
+        c3##j = _mm512_dpbusd_epi32(c3##j, a3, b);                                   \
+    }
+#define VN_OUT(j)                                                                    \
+    out[0][j] = _mm512_reduce_add_epi32(c0##j);                                      \
+    out[1][j] = _mm512_reduce_add_epi32(c1##j);                                      \
+    out[2][j] = _mm512_reduce_add_epi32(c2##j);                                      \
+    out[3][j] = _mm512_reduce_add_epi32(c3##j);
+    VN_DECL(0) VN_DECL(1) VN_DECL(2) VN_DECL(3) VN_DECL(4) VN_DECL(5)
+    for (int64_t k = 0; k < kc; k += 64) {
+        const __m512i a0 = _mm512_loadu_si512((const void *)(xu + k));
+        const __m512i a1 = _mm512_loadu_si512((const void *)(xu + ldx + k));
+        const __m512i a2 = _mm512_loadu_si512((const void *)(xu + 2 * ldx + k));
+        const __m512i a3 = _mm512_loadu_si512((const void *)(xu + 3 * ldx + k));
+        VN_STEP(0) VN_STEP(1) VN_STEP(2) VN_STEP(3) VN_STEP(4) VN_STEP(5)
+    }
+    VN_OUT(0) VN_OUT(1) VN_OUT(2) VN_OUT(3) VN_OUT(4) VN_OUT(5)
+#undef VN_DECL
+#undef VN_STEP
+#undef VN_OUT
+}
+
+ORC_VNNI static int32_t vnni_dot(const uint8_t *xu, const int8_t *w, int64_t kc)
+{
+    __m512i c = _mm512_setzero_si512();
+    for (int64_t k = 0; k < kc; k += 64)
+        c = _mm512_dpbusd_epi32(c, _mm512_loadu_si512((const void *)(xu + k)),
+                                _mm512_loadu_si512((const void *)(w + k)));
+    return _mm512_reduce_add_epi32(c);
+}
+
+ORC_VNNI static int gemm_vnni(const int8_t *qx, const int8_t *qw, int32_t *acc,
+                              int64_t M, int64_t N, int64_t K)
+{
+    const int64_t K64 = K & ~(int64_t)63;
+    uint8_t *xu = (uint8_t *)malloc((size_t)(M * K64) + 64);
+    int32_t *wsum = (int32_t *)malloc((size_t)N * sizeof(int32_t));
+    if (!xu || !wsum) { free(xu); free(wsum); return -2; }
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K64; ++k) xu[m * K64 + k] = (uint8_t)qx[m * K + k] ^ 0x80u;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        int32_t s = 0;
+        for (int64_t k = 0; k < K64; ++k) s += qw[n * K + k];
+        wsum[n] = s;
+    }
+    const int64_t ntiles = (N + VN_NR - 1) / VN_NR;
+#pragma omp parallel
+    {
+        int nth = 1, tid = 0;
+#ifdef _OPENMP
+        extern int omp_get_num_threads(void), omp_get_thread_num(void);
+        nth = omp_get_num_threads();
+        tid = omp_get_thread_num();
+#endif
+        const int64_t t0 = ntiles * tid / nth, t1 = ntiles * (tid + 1) / nth;
+        for (int64_t k0 = 0; k0 < K64; k0 += VN_KC) {
+            const int64_t kc = K64 - k0 < VN_KC ? K64 - k0 : VN_KC;
+            for (int64_t mp = 0; mp < M; mp += VN_MP) {
+                const int64_t mend = mp + VN_MP < M ? mp + VN_MP : M;
+                for (int64_t t = t0; t < t1; ++t) {
+                    const int64_t n0 = t * VN_NR, nr = N - n0 < VN_NR ? N - n0 : VN_NR;
+                    for (int64_t m0 = mp; m0 < mend; m0 += VN_MR) {
+                        const int64_t mr = mend - m0 < VN_MR ? mend - m0 : VN_MR;
+                        int32_t out[VN_MR][VN_NR];
+                        if (mr == VN_MR && nr == VN_NR)
+                            vnni_tile(xu + m0 * K64 + k0, K64, qw + n0 * K + k0, K, kc, out);
+                        else
+                            for (int64_t r = 0; r < mr; ++r)
+                                for (int64_t j = 0; j < nr; ++j)
+                                    out[r][j] = vnni_dot(xu + (m0 + r) * K64 + k0, qw + (n0 + j) * K + k0, kc);
+                        for (int64_t r = 0; r < mr; ++r)
+                            for (int64_t j = 0; j < nr; ++j) {
+                                int32_t *d = acc + (m0 + r) * N + n0 + j;
+                                *d = k0 ? *d + out[r][j] : out[r][j] - 128 * wsum[n0 + j];
+                            }
+                    }
+                }
+            }
+        }
+        if (K64 < K || K64 == 0)                     /* the K tail, and K < 64 as a whole */
+            for (int64_t t = t0; t < t1; ++t)
+                for (int64_t n = t * VN_NR; n < N && n < (t + 1) * VN_NR; ++n)
+                    for (int64_t m = 0; m < M; ++m) {
+                        int32_t s = K64 ? acc[m * N + n] : 0;
+                        for (int64_t k = K64; k < K; ++k) s += (int32_t)qx[m * K + k] * (int32_t)qw[n * K + k];
+                        acc[m * N + n] = s;
+                    }
+    }
+    free(xu);
+    free(wsum);
+    return 0;
+}
+
+static int orc_have_vnni(void)
+{
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") &&
+           __builtin_cpu_supports("avx512vl") && __builtin_cpu_supports("avx512vnni");
+}
+#else
+static int orc_have_vnni(void) { return 0; }
+#endif
+
+/* 1 when orc_gemm_i8_i32 runs its blocked VNNI form on this host, else 0 */
+ORC_API int orc_gemm_uses_vnni(void) { return orc_have_vnni(); }
+
 ORC_API void orc_gemm_i8_i32(const int8_t *qx, const int8_t *qw, int32_t *acc,
                              int64_t M, int64_t N, int64_t K)
 {
+#if defined(__x86_64__)
+    if (M >= VN_MR && orc_have_vnni() && gemm_vnni(qx, qw, acc, M, N, K) == 0) return;
+#endif
 #pragma omp parallel for schedule(static)
     for (int64_t n = 0; n < N; ++n)
         for (int64_t m = 0; m < M; ++m)

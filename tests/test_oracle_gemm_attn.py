@@ -28,6 +28,23 @@ def test_gemm_vs_numpy_int64(orc, M, N, K):
     assert np.array_equal(orc.gemm_i8_i32(qx, qw, scalar=True), got)
 
 
+@pytest.mark.parametrize("M,N,K", [(4, 6, 64), (5, 7, 200), (4, 6, 63), (9, 13, 128), (67, 100, 4096 + 128),
+                                   (130, 50, 14336), (8, 16, 32), (3, 9, 256)])
+def test_gemm_blocked_form_edges(orc, M, N, K):
+    """The blocked form the oracle takes on hosts with byte dot-product instructions (register tiles of 4 x 6,
+    row panels of 64, K chunks of 4096, a scalar K tail, a +128 bias on the activation codes) against the plain
+    loop and numpy int64: tile and panel remainders, several K chunks, K below and off the vector width, and
+    rows of -128 / -127 / 127 that push the biased partial sums to their extremes."""
+    g = np.random.default_rng(M * 131 + N * 7 + K)
+    qx = g.integers(-128, 128, (M, K)).astype(np.int8)
+    qw = g.integers(-128, 128, (N, K)).astype(np.int8)
+    qx[0, :], qw[0, :] = -128, -128
+    qx[M - 1, :], qw[N - 1, :] = 127, -127
+    got = orc.gemm_i8_i32(qx, qw)
+    assert np.array_equal(got, orc.gemm_i8_i32(qx, qw, scalar=True))
+    assert np.array_equal(got.astype(np.int64), qx.astype(np.int64) @ qw.astype(np.int64).T)
+
+
 def test_gemm_extreme_values_do_not_overflow(orc):
     K = 14336
     qx = np.full((2, K), 127, np.int8)
