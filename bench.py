@@ -67,6 +67,20 @@ class Timer:
         self.e1.synchronize()
         return self.e0.elapsed_ms(self.e1) / reps
 
+    def samples(self, fn, n):
+        """n per-call durations (ms): an event before and after every call, all recorded back to back on the
+        launch stream and read only after the last one, so that the chip never idles between the calls."""
+        ev = [self.mi.Event() for _ in range(n + 1)]
+        ev[0].record(self.stream)
+        for i in range(n):
+            fn()
+            ev[i + 1].record(self.stream)
+        ev[n].synchronize()
+        out = [ev[i].elapsed_ms(ev[i + 1]) for i in range(n)]
+        for e in ev:
+            e.destroy()
+        return out
+
     def settle(self, fn, ms=60.0):
         """Untimed: keep fn() running back to back for about `ms` of GPU time.  After any idle spell the
         chip's power control first throttles the matrix pipe hard and then converges, over about 30 ms of
@@ -175,7 +189,7 @@ def main():
     value = step_ops / (ms_step * 1e-3) / 1e12
 
     # ---- the dominant kernel alone: the tiled MFMA GEMM on already-quantized activations
-    gemm_ms = {}
+    gemm_ms, gemm_samples = {}, {}
     qx = {K: dev.empty((M, K), np.int8) for K in (4096, 14336)}
     sx = {K: dev.empty(M, np.float32) for K in (4096, 14336)}
     for K in qx:
@@ -188,6 +202,7 @@ def main():
             mi.check(lib.mi_w8a8_gemm_dequant_f32(qx[K].ptr, sx[K].ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, s))
         timer.settle(one)
         gemm_ms[name] = timer.run(one, max(10, args.steps))
+        gemm_samples[name] = sorted(timer.samples(one, max(10, args.steps)))
     gemm_total_ms = sum(gemm_ms.values())
     gemm_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
     # HBM-side bytes per launch of the tiled GEMM, measured with hardware counters in a separate run
@@ -205,6 +220,10 @@ def main():
         "traffic_unit": "bytes over the four launches (fetched + written), rocprofv3 PMC, calibrated",
         "traffic_per_shape": traffic,
         "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
+        "per_shape_us_median": {k: round(v[len(v) // 2] * 1e3, 2) for k, v in gemm_samples.items()},
+        "per_shape_us_min": {k: round(v[0] * 1e3, 2) for k, v in gemm_samples.items()},
+        "per_shape_samples": "median / min over single launches, each between two event records (the records add "
+                             "1-3 us per launch to these two rows; per_shape_us is one pair of events around the whole run)",
         "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
                            for name, K, N in wl.PROJECTIONS},
     }
