@@ -98,6 +98,9 @@ def main():
     ap.add_argument("--skip-sub", action="store_true", help="only the headline workload")
     ap.add_argument("--decode-layer-only", action="store_true",
                     help="only the decode-layer chain sub-metric (for a kernel trace of that chain alone)")
+    ap.add_argument("--decode-stack", type=int, default=0, metavar="L",
+                    help="only a decode step through a stack of L decoder layers (e.g. 32: 11.4 GB of weights and "
+                         "caches), each with its own weights and KV cache, as one graph")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
@@ -111,6 +114,16 @@ def main():
 
     if args.pmc_probe:
         return pmc_probe(mi, wl)
+    if args.decode_stack:
+        dev = mi.Device(arena_bytes=(2 << 30) + args.decode_stack * (400 << 20))
+        pool = mi.StreamPool(dev, 1)
+        s = pool.stream(0)
+        for b in (None, 1):
+            print(json.dumps(decode_layer_chain(mi, wl, dev, s, Timer(mi, s), reps=5, batch=b,
+                                                nlayers=args.decode_stack)), flush=True)
+        pool.destroy()
+        dev.close()
+        return
     if args.decode_layer_only:
         dev = mi.Device(arena_bytes=12 << 30)
         pool = mi.StreamPool(dev, 1)
@@ -121,7 +134,7 @@ def main():
         dev.close()
         return
 
-    dev = mi.Device(arena_bytes=12 << 30)
+    dev = mi.Device(arena_bytes=20 << 30)
     pool = mi.StreamPool(dev, 1)
     s = pool.stream(0)
     timer = Timer(mi, s)
@@ -252,6 +265,9 @@ def main():
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer, batch=1))
+        # the whole stack as one graph: 32 layers, each with its own weights and cache (11.4 GB)
+        sub.update(decode_layer_chain(mi, wl, dev, s, timer, reps=5, nlayers=32))
+        sub.update(decode_layer_chain(mi, wl, dev, s, timer, reps=5, batch=1, nlayers=32))
         sub.update(host_staging(mi, wl, dev, s, timer))
     out["sub_metrics"] = sub
     if not args.skip_cpu:
@@ -461,11 +477,13 @@ def cfg0_linear(mi, wl, dev, s, timer, shapes):
                                 "TOPS": round(wl.gemm_ops(M, N, K) / (ms * 1e-3) / 1e12, 2)}}
 
 
-def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None):
+def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None, nlayers=3):
     """A decode step through decoder layers of the cfg1 / cfg2 shapes (hidden 4096, 32/8 heads of 128, FFN 14336,
     16 sequences with 4095 cached tokens each): three layers with their own weights (654 MB) and KV caches
     (417 MB) run one after the other, so that nothing a layer reads is left in the memory-side cache from its
-    last turn; the three-layer step is recorded into a graph and replayed."""
+    last turn; the three-layer step is recorded into a graph and replayed.  With nlayers > 3 (a whole stack: 32
+    layers hold 7 GB of weights and 4.4 GB of caches) every layer still has its own weights and cache at its own
+    address; the fp32 sources of the weights repeat with period three."""
     c = wl.ATTN
     B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
     if batch is not None:
@@ -477,14 +495,19 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None):
     cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
     g1 = np.ones(H, np.float32)
     layers = []
-    for li in range(3):
-        w = [wl.weights(500 + li, n, k, i) for i, (n, k) in
-             enumerate((((Hq + 2 * Hkv) * D, H), (H, Hq * D), (2 * I, H), (H, I)))]
+    wsrc, csrc = {}, {}
+    for li in range(nlayers):
+        if li % 3 not in wsrc:
+            wsrc[li % 3] = [wl.weights(500 + li, n, k, i) for i, (n, k) in
+                            enumerate((((Hq + 2 * Hkv) * D, H), (H, Hq * D), (2 * I, H), (H, I)))]
+            csrc[li % 3] = wl.normal(600 + li, (B * Hkv * T, D), 0)
+        w = wsrc[li % 3]
         L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, w[0], w[1], w[2], w[3], g1, g1, cos, sin)
-        del w
+        if li + 3 >= nlayers:
+            wsrc[li % 3] = None
         # a cache of real rows: rotate + quantize N(0,1) keys and values
         m2 = dev.mark()
-        src = dev.upload(wl.normal(600 + li, (B * Hkv * T, D), 0))
+        src = dev.upload(csrc[li % 3])
         mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.kq.ptr, L.ks.ptr, B * Hkv * T, D, D, s))
         mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.vq.ptr, L.vs.ptr, B * Hkv * T, D, D, s))
         dev.sync(s)
@@ -497,18 +520,22 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None):
     def step():
         # inside the stack a layer's closing residual add is done by the next layer's first kernel
         layers[0].step(x, dpos, dlen, T, None, s)
-        layers[1].step(layers[0].dn, dpos, dlen, T, None, s, residual=layers[0].h1)
-        layers[2].step(layers[1].dn, dpos, dlen, T, out, s, residual=layers[1].h1)
+        for li in range(1, nlayers):
+            layers[li].step(layers[li - 1].dn, dpos, dlen, T, out if li == nlayers - 1 else None, s,
+                            residual=layers[li - 1].h1)
     ms = graph_time(mi, dev, s, timer, [step], reps) / len(layers)
     wbytes = ((Hq + 2 * Hkv) * D * H + H * Hq * D + 2 * I * H + H * I)
     nbytes = wbytes + wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
     dev.reset_to(mark)
-    return {"decode_layer_b%d_t4096" % B: {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10 if B > 1 else 8,
-                                       "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                                       "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1),
-                                       "tokens_per_s_32_layers": round(B / (32 * ms * 1e-3), 1),
-                                       "algorithmic_bytes": nbytes}}
+    res = {"us_per_layer": round(ms * 1e3, 2), "kernels_per_layer": 10 if B > 1 else 8, "layers_in_graph": nlayers,
+           "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+           "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes}
+    if nlayers == 3:
+        res["tokens_per_s_32_layers"] = round(B / (32 * ms * 1e-3), 1)        # extrapolated from three layers
+        return {"decode_layer_b%d_t4096" % B: res}
+    res["us_per_step"] = round(ms * 1e3 * nlayers, 1)                           # measured: the stack is one graph
+    res["tokens_per_s"] = round(B / (nlayers * ms * 1e-3), 1)
+    return {"decode_stack_%d_layers_b%d_t4096" % (nlayers, B): res}
 
 
 def host_staging(mi, wl, dev, s, timer):
