@@ -6,7 +6,7 @@
 // :70-80, :103-121).  No Mojo toolchain exists where this is built, so the same
 // surface is written in C++: DeviceArena mirrors NumaArena, StreamPool mirrors
 // ThreadPool, Gate mirrors MutexGate, and QuantLinear / DecodeAttention /
-// KvCache / DecoderLayer / MoeFfn are the quantize / linear / attention / MoE call surface that a Mojo
+// KvCache / DecoderLayer / DecoderStack / MoeFfn are the quantize / linear / attention / MoE call surface that a Mojo
 // host would hold as structs over the same handles.  Nothing here throws.
 #pragma once
 #include <cstdint>
@@ -354,6 +354,61 @@ struct DecoderLayer {
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ci, si, down.qw, down.sw, dn, B, H, I, stream);
         if (rc == MI_OK && out) rc = mi_add_f32(h1, dn, out, B * H, stream);
         return rc;
+    }
+};
+
+// A recorded sequence of launches, replayed as one (mi_graph_*).  Record with
+//   Graph g; g.begin(stream); ...enqueue on stream...; g.end(stream);   then   g.launch(stream)
+// after one eager run of the same calls (the first call of a kernel sets its attributes).  Move-only.
+class Graph {
+public:
+    Graph() = default;
+    Graph(const Graph &) = delete;
+    Graph &operator=(const Graph &) = delete;
+    Graph(Graph &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    ~Graph() { if (h_) mi_graph_destroy(h_); }
+    explicit operator bool() const { return h_ != nullptr; }
+    int32_t begin(void *stream) { return mi_graph_capture_begin(stream); }
+    int32_t end(void *stream)
+    {
+        if (h_) { mi_graph_destroy(h_); h_ = nullptr; }
+        return mi_graph_capture_end(stream, &h_);
+    }
+    int32_t launch(void *stream) const { return h_ ? mi_graph_launch(h_, stream) : MI_EINVAL; }
+
+private:
+    mi_graph *h_ = nullptr;
+};
+
+// A stack of decoder layers for one decode step: layer l+1 takes x = dn and residual = h1 of layer l, so that the
+// closing residual add of a layer happens inside the first kernel of the next one; only the last layer writes `out`.
+// Capacity is a compile-time parameter like the reference's pool sizes; nothing is allocated outside the arena.
+template <int MaxLayers = 128>
+struct DecoderStack {
+    DecoderLayer layers[MaxLayers];
+    int count = 0;
+
+    // appends a layer (arguments as DecoderLayer::prepare); false when the stack or the arena is full
+    template <typename Arena, typename... Args>
+    bool add(Arena &arena, Args &&...args)
+    {
+        if (count >= MaxLayers) return false;
+        if (!layers[count].prepare(arena, std::forward<Args>(args)...)) return false;
+        ++count;
+        return true;
+    }
+    // one new token per sequence through every layer; the first failing call's status is returned
+    int32_t step(const float *x, const int32_t *pos, const int32_t *seq_len, int64_t t_max, float *out, void *stream) const
+    {
+        if (count <= 0 || !out) return MI_EINVAL;
+        const float *xin = x, *res = nullptr;
+        for (int l = 0; l < count; ++l) {
+            const int32_t rc = layers[l].step(xin, res, pos, seq_len, t_max, l + 1 == count ? out : nullptr, stream);
+            if (rc != MI_OK) return rc;
+            xin = layers[l].dn;
+            res = layers[l].h1;
+        }
+        return MI_OK;
     }
 };
 

@@ -399,6 +399,69 @@ static void test_decoder_layer(const Context &ctx)
     report("decoder_layer_vs_oracle", good);
 }
 
+// Three small layers as a DecoderStack: the stack's step equals the same layers chained by hand with explicit
+// residual adds between them only where the arithmetic is the same (the sum h1 + dn is formed once either way),
+// and a recorded step replayed twice gives the same bits as the eager one (the caches are rewritten with the
+// same rows at the same positions, so a replay is idempotent).
+static void test_decoder_stack(const Context &ctx)
+{
+    const int64_t B = 2, H = 256, Hq = 2, Hkv = 1, I = 256, T_cap = 16, D = 128, NQ = (Hq + 2 * Hkv) * D;
+    DeviceArena<256> arena(ctx, 256 << 20);
+    Rng rng{11};
+    auto gauss = [&](int64_t n, float s) { std::vector<float> v((size_t)n); for (auto &e : v) e = s * rng.normal(); return v; };
+    std::vector<float> cs((size_t)(T_cap * 64)), sn((size_t)(T_cap * 64));
+    for (int64_t t = 0; t < T_cap; ++t)
+        for (int64_t i = 0; i < 64; ++i) {
+            const double a = (double)t * std::pow(10000.0, -2.0 * (double)i / 128.0);
+            cs[t * 64 + i] = (float)std::cos(a);
+            sn[t * 64 + i] = (float)std::sin(a);
+        }
+    float *dcs = upload(arena, cs), *dsn = upload(arena, sn);
+    DecoderStack<4> stack;
+    DecoderLayer solo[3];
+    bool ok = dcs && dsn;
+    for (int l = 0; l < 3 && ok; ++l) {
+        std::vector<float> wqkv = gauss(NQ * H, 0.05f), wo = gauss(H * Hq * D, 0.05f), wgu = gauss(2 * I * H, 0.05f),
+                           wd = gauss(H * I, 0.05f), g1 = gauss(H, 0.1f), g2 = gauss(H, 0.1f);
+        for (auto &e : g1) e += 1.0f;
+        for (auto &e : g2) e += 1.0f;
+        float *a = upload(arena, wqkv), *b = upload(arena, wo), *c = upload(arena, wgu), *d = upload(arena, wd),
+              *e = upload(arena, g1), *f = upload(arena, g2);
+        ok = a && b && c && d && e && f &&
+             stack.add(arena, B, H, Hq, Hkv, I, T_cap, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr) &&
+             solo[l].prepare(arena, B, H, Hq, Hkv, I, T_cap, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr);
+    }
+    std::vector<float> x = gauss(B * H, 1.0f);
+    const std::vector<int32_t> pos = {0, 5}, len = {1, 6};
+    int32_t *dpos = upload(arena, pos), *dlen = upload(arena, len);
+    float *dx = upload(arena, x), *dout = arena.alloc<float>(B * H), *dref = arena.alloc<float>(B * H),
+          *dmid = arena.alloc<float>(B * H);
+    ok = ok && dpos && dlen && dx && dout && dref && dmid && stack.count == 3;
+    const bool refuses = ok && [&] { DecoderStack<1> one; one.count = 1; return !one.add(arena, B, H, Hq, Hkv, I, T_cap, dx, dx, dx, dx, dx, dx, dcs, dsn, 1e-5f, nullptr); }();
+    if (!ok) { report("decoder_stack", false, "set-up failed"); return; }
+    // by hand: every layer closes with its own residual add, the next one starts from that sum
+    bool good = solo[0].step(dx, nullptr, dpos, dlen, T_cap, dmid, nullptr) == MI_OK &&
+                solo[1].step(dmid, nullptr, dpos, dlen, T_cap, dref, nullptr) == MI_OK &&
+                solo[2].step(dref, nullptr, dpos, dlen, T_cap, dmid, nullptr) == MI_OK;
+    const std::vector<float> want = download(dmid, (size_t)(B * H));
+    good = good && stack.step(dx, dpos, dlen, T_cap, dout, nullptr) == MI_OK;
+    const std::vector<float> eager = download(dout, (size_t)(B * H));
+    good = good && eager == want;
+    // the same step recorded and replayed
+    StreamPool pool(ctx, 1);
+    void *s = pool.stream(0);
+    Graph g;
+    good = good && g.begin(s) == MI_OK;
+    const int32_t rc_step = stack.step(dx, dpos, dlen, T_cap, dout, s);
+    good = (g.end(s) == MI_OK) && good && rc_step == MI_OK && (bool)g;
+    for (int rep = 0; rep < 2 && good; ++rep) {
+        good = mi_fill_u32(dout, 0u, B * H, s) == MI_OK && g.launch(s) == MI_OK && mi_stream_synchronize(s) == MI_OK;
+        good = good && download(dout, (size_t)(B * H)) == want;
+    }
+    good = good && refuses && stack.step(dx, dpos, dlen, T_cap, nullptr, nullptr) == MI_EINVAL;
+    report("decoder_stack", good);
+}
+
 int main()
 {
     Context ctx(0);
@@ -411,6 +474,7 @@ int main()
     test_decode_attention(ctx);
     test_kv_cache(ctx);
     test_decoder_layer(ctx);
+    test_decoder_stack(ctx);
     std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;
 }
