@@ -96,6 +96,16 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
     if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float readlane_f(float v, int l)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+
 // one wave per token: k rounds of (wave-wide max, lowest index among the lanes that hold it); lane l holds
 // experts l, l+64, l+128, l+192.  Ties go to the lower expert index; picks come out by descending logit.
 __global__ __launch_bounds__(256) void k_moe_topk(const float *__restrict__ logits, int32_t *__restrict__ idx,
@@ -113,9 +123,14 @@ __global__ __launch_bounds__(256) void k_moe_topk(const float *__restrict__ logi
     float top[MAX_TOPK];
     int pick_lane = 0;       // lane s keeps pick s
     for (int s = 0; s < topk; ++s) {
+        // wave-wide maximum: four DPP steps leave every 16-lane row with its own maximum, four scalar reads join the
+        // rows (a chain of cross-lane permutes costs five times as many cycles, and this loop is all latency)
         float v = fmaxf(fmaxf(mine[0], mine[1]), fmaxf(mine[2], mine[3]));
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+        v = fmaxf(v, dpp_f<0xB1>(v));    // quad_perm [1,0,3,2]
+        v = fmaxf(v, dpp_f<0x4E>(v));    // quad_perm [2,3,0,1]
+        v = fmaxf(v, dpp_f<0x124>(v));   // row_ror:4
+        v = fmaxf(v, dpp_f<0x128>(v));   // row_ror:8
+        v = fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
         // lowest expert index holding v: experts of slot u are 64u .. 64u+63, so the first non-empty ballot wins
         int win = -1;
 #pragma unroll
@@ -132,15 +147,19 @@ __global__ __launch_bounds__(256) void k_moe_topk(const float *__restrict__ logi
         for (int q = 0; q < MAX_TOPK; ++q)
             if (q == s) top[q] = v;
     }
+    // lane s evaluates e_s = expf(l_s - l_0) once; the sum runs over the picks in pick order, as the oracle's does
+    float mine_top = top[0];
+#pragma unroll
+    for (int q = 1; q < MAX_TOPK; ++q)
+        if (q == lane) mine_top = top[q];
+    const float e = lane < topk ? expf(mine_top - top[0]) : 0.0f;
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < MAX_TOPK; ++q)
+        if (q < topk) sum = sum + readlane_f(e, q);
     if (lane < topk) {
         idx[(int64_t)t * topk + lane] = pick_lane;
-        float sum = 0.0f;
-        for (int s = 0; s < topk; ++s) sum = sum + expf(top[s] - top[0]);
-        float mine_top = top[0];
-#pragma unroll
-        for (int q = 1; q < MAX_TOPK; ++q)
-            if (q == lane) mine_top = top[q];
-        w[(int64_t)t * topk + lane] = expf(mine_top - top[0]) / sum;
+        w[(int64_t)t * topk + lane] = e / sum;
     }
 }
 
