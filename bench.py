@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--decode-stack", type=int, default=0, metavar="L",
                     help="only a decode step through a stack of L decoder layers (e.g. 32: 11.4 GB of weights and "
                          "caches), each with its own weights and KV cache, as one graph")
+    ap.add_argument("--skip-stack", action="store_true", help="no 32-layer decode stack leg (it takes 15 GB more)")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
@@ -134,7 +135,7 @@ def main():
         dev.close()
         return
 
-    dev = mi.Device(arena_bytes=20 << 30)
+    dev = mi.Device(arena_bytes=12 << 30)
     pool = mi.StreamPool(dev, 1)
     s = pool.stream(0)
     timer = Timer(mi, s)
@@ -265,9 +266,17 @@ def main():
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer, batch=1))
-        # the whole stack as one graph: 32 layers, each with its own weights and cache (11.4 GB)
-        sub.update(decode_layer_chain(mi, wl, dev, s, timer, reps=5, nlayers=32))
-        sub.update(decode_layer_chain(mi, wl, dev, s, timer, reps=5, batch=1, nlayers=32))
+        if not args.skip_stack:
+            # the whole stack as one graph: 32 layers, each with its own weights and cache (11.4 GB), in an arena
+            # of its own that lives only for this measurement
+            sdev = mi.Device(arena_bytes=15 << 30)
+            spool = mi.StreamPool(sdev, 1)
+            ss = spool.stream(0)
+            stimer = Timer(mi, ss)
+            sub.update(decode_layer_chain(mi, wl, sdev, ss, stimer, reps=5, nlayers=32))
+            sub.update(decode_layer_chain(mi, wl, sdev, ss, stimer, reps=5, batch=1, nlayers=32))
+            spool.destroy()
+            sdev.close()
         sub.update(host_staging(mi, wl, dev, s, timer))
     out["sub_metrics"] = sub
     if not args.skip_cpu:
