@@ -1,0 +1,39 @@
+"""The bench line keeps its contract: one JSON object on stdout with the driver's fields, the roofline and (when asked
+for) the CPU baseline; more than one GPU is refused with a message."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.gpu
+def test_bench_line_fields():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--steps", "2", "--warmup", "1",
+                          "--skip-sub", "--skip-cpu"], capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [l for l in out.stdout.strip().splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    b = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in b, key
+    assert b["n_gpus"] == 1 and b["steps"] == 2 and b["warmup"] == 1 and b["higher_is_better"] is True
+    assert b["unit"] == "TOPS" and b["dtype"] == "int8" and b["data"] == "synthetic" and b["vs_baseline"] is None
+    assert "workload" in b["config"] and "model" not in b["config"]
+    r = b["roofline"]
+    assert r["bound"] == "mfma" and r["unit"] == "TOP/s" and r["peak"] == 5000.0
+    assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
+    assert 0.05 < r["frac"] < 1.0 and b["value"] > 100.0
+    # value is ops per step over the step time
+    assert abs(b["value"] - b["config"]["ops_per_step"] / (b["ms_per_step"] * 1e-3) / 1e12) < 0.01 * b["value"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120, cwd=ROOT)
+    assert out.returncode != 0
+    assert "ONE GPU" in (out.stderr + out.stdout)
