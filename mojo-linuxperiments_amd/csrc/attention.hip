@@ -582,6 +582,21 @@ static SplitPlan pick_splits(int64_t B, int64_t Hkv, int64_t T)
     return pl;
 }
 
+// the largest split count pick_splits returns for any length in [1, T]
+static int max_splits(int64_t B, int64_t Hkv, int64_t T)
+{
+    const int ntiles = (int)((T + 15) / 16);
+    int best = (ntiles + 4 * TILES_LONG - 1) / (4 * TILES_LONG);   // long spans: monotone in T
+    if (B * Hkv < compute_units()) {
+        // short spans are possible for some length: ceil(n / 16) splits, doubled at most up to 16
+        int s = (ntiles + 4 * TILES_SHORT - 1) / (4 * TILES_SHORT);
+        if (s < 16) s = 16;
+        if (s > ntiles) s = ntiles;
+        if (s > best) best = s;
+    }
+    return best;
+}
+
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace attn
@@ -602,7 +617,9 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
 {
     int32_t rc = check_attn(B, Hq, Hkv, D, T);
     if (rc) return rc;
-    const int splits = attn::pick_splits(B, Hkv, T).splits;
+    // an upper bound over every length up to T, so that a workspace sized for the capacity of a cache serves every
+    // decode step: the plan is not monotone in T (a shorter sequence may be cut into more, shorter spans)
+    const int splits = attn::max_splits(B, Hkv, T);
     return attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256) + attn::align_up(B * Hkv * splits * 8 * 4, 256);
 }
 

@@ -47,3 +47,19 @@ def test_status_strings_and_argument_checks_without_gpu(mi):
     assert lib.mi_w8a8_linear_workspace_bytes(32, 4096, 4096) >= 32 * 4096 + 32 * 4
     assert lib.mi_gqa_decode_workspace_bytes(16, 32, 8, 64, 4096) == mi.EINVAL      # head_dim must be 128
     assert lib.mi_gqa_decode_workspace_bytes(16, 32, 6, 128, 4096) == mi.EINVAL     # Hq % Hkv
+
+
+def test_attention_workspace_bound_covers_every_shorter_length(mi):
+    """A workspace sized for the capacity of a cache must serve every decode step: the split plan is not monotone
+    in the length (a shorter sequence may be cut into more, shorter spans), the size query is."""
+    lib = mi.lib
+    for rows, hkv in ((128, 8), (64, 8), (32, 8), (16, 8), (8, 8), (1, 1), (3, 1)):
+        B = rows // hkv if rows >= hkv else rows
+        for t_cap in (48, 1000, 2048, 4096, 16384):
+            cap = lib.mi_gqa_decode_workspace_bytes(B, 4 * hkv, hkv, 128, t_cap)
+            assert cap > 0
+            prev = 0
+            for t in list(range(1, min(t_cap, 600))) + list(range(600, t_cap + 1, 37)) + [t_cap]:
+                need = lib.mi_gqa_decode_workspace_bytes(B, 4 * hkv, hkv, 128, t)
+                assert prev <= need <= cap, (rows, t_cap, t)
+                prev = need
