@@ -178,6 +178,19 @@ MI_API int64_t mi_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 MI_API int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const float *sw, float *y,
                                   int64_t M, int64_t N, int64_t K, int32_t block,
                                   void *workspace, int64_t workspace_bytes, void *stream);
+/* The same linear without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart upstream.  The activation
+ * codes and scales live in a static device array of 8 MiB + 32 KiB that every device the library runs on holds
+ * until the process ends; mi_ctx_create looks its address up for the context's device (otherwise the first call on
+ * a device does).  Limits: M <= mi_w8a8_linear_noalloc_max_rows() = 8192 and M * K <=
+ * mi_w8a8_linear_noalloc_max_codes() = 8 Mi, beyond them MI_ERANGE.  The call allocates and frees nothing.  All
+ * calls on one device share the one array: two calls may not overlap on a device (different streams, or two
+ * threads) - they would race on the codes; calls on one stream are ordered and safe.  Results are bit-identical to
+ * mi_w8a8_linear_f32 (the same kernels run). */
+MI_API int32_t mi_w8a8_linear_f32_noalloc(const float *x, const int8_t *qw, const float *sw, float *y,
+                                          int64_t M, int64_t N, int64_t K, int32_t block, void *stream);
+MI_API int64_t mi_w8a8_linear_noalloc_max_rows(void);
+MI_API int64_t mi_w8a8_linear_noalloc_max_codes(void);
 
 /* ---- a8: grouped-query decode attention over an int8 KV cache
  * q fp32 [B,Hq,D] (unrotated); kq,vq int8 [B,Hkv,T,D]; ks,vs fp32 [B,Hkv,T];

@@ -1,5 +1,7 @@
 // C ABI of the W8A8 contraction: argument checks and the choice between the
 // skinny weight-streaming kernel (M <= 64) and the LDS-tiled MFMA kernel.
+#include <atomic>
+
 #include "common.h"
 
 namespace mi {
@@ -110,14 +112,10 @@ extern "C" int32_t mi_rmsnorm_linear_f32(const float *x, const float *residual, 
     return gemm_dispatch(qx, sx, qw, sw, nullptr, y, M, N, K, as_stream(stream));
 }
 
-extern "C" int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const float *sw, float *y, int64_t M,
-                                      int64_t N, int64_t K, int32_t block, void *workspace,
-                                      int64_t workspace_bytes, void *stream)
+// The linear once its activation codes (qx) and scales (sx) have a home: the caller's workspace or the static array.
+static int32_t linear_with(const float *x, const int8_t *qw, const float *sw, float *y, int64_t M, int64_t N,
+                           int64_t K, int32_t block, int8_t *qx, float *sx, void *stream)
 {
-    if (!workspace || !aligned16(workspace)) return MI_EINVAL;
-    if (workspace_bytes < mi_w8a8_linear_workspace_bytes(M, N, K)) return MI_ENOSPC;
-    int8_t *qx = static_cast<int8_t *>(workspace);
-    float *sx = reinterpret_cast<float *>(qx + align_up(M * K, 256));
     int32_t rc = check_gemm(qx, qw, y, M, N, K);
     if (rc) return rc;
     if (!x || !sw || !aligned16(sw)) return MI_EINVAL;
@@ -129,4 +127,64 @@ extern "C" int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const fl
     rc = mi_fwht_quant_f32_i8(x, qx, sx, M, K, block, stream);
     if (rc) return rc;
     return gemm_dispatch(qx, sx, qw, sw, nullptr, y, M, N, K, as_stream(stream));
+}
+
+extern "C" int32_t mi_w8a8_linear_f32(const float *x, const int8_t *qw, const float *sw, float *y, int64_t M,
+                                      int64_t N, int64_t K, int32_t block, void *workspace,
+                                      int64_t workspace_bytes, void *stream)
+{
+    if (!workspace || !aligned16(workspace)) return MI_EINVAL;
+    if (workspace_bytes < mi_w8a8_linear_workspace_bytes(M, N, K)) return MI_ENOSPC;
+    int8_t *qx = static_cast<int8_t *>(workspace);
+    float *sx = reinterpret_cast<float *>(qx + align_up(M * K, 256));
+    return linear_with(x, qw, sw, y, M, N, K, block, qx, sx, stream);
+}
+
+// ---- the same linear for callers that cannot allocate (code under graph capture, serving loops, harnesses that
+// forbid hipMalloc): the activation codes and scales live in a static device array instead of a caller workspace.
+// Every device the library runs on holds its own copy of the array, at its own address, until the process ends.
+static constexpr int64_t NOALLOC_CODE_BYTES = 8ll << 20;   // M * K activation codes
+static constexpr int64_t NOALLOC_MAX_ROWS = 8192;          // M scales
+static constexpr int64_t NOALLOC_BYTES = NOALLOC_CODE_BYTES + NOALLOC_MAX_ROWS * 4;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_BYTES];
+
+// In host code `scratch` is only a handle for the symbol: the array's device address is asked for once per device,
+// with that device current, and every later use goes through the pointer kept here.
+static constexpr int NOALLOC_MAX_DEVICES = 64;
+static std::atomic<unsigned char *> g_scratch_ptr[NOALLOC_MAX_DEVICES];
+
+namespace mi {
+int32_t linear_scratch_bind(int device, unsigned char **out)   // `device` must be the current device
+{
+    if (device < 0 || device >= NOALLOC_MAX_DEVICES) return MI_ERANGE;
+    unsigned char *p = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        void *sym = nullptr;
+        MI_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)));
+        if (!sym) return MI_EIO;
+        p = static_cast<unsigned char *>(sym);
+        g_scratch_ptr[device].store(p, std::memory_order_release);   // a race stores the same address twice
+    }
+    if (out) *out = p;
+    return MI_OK;
+}
+}  // namespace mi
+
+extern "C" int64_t mi_w8a8_linear_noalloc_max_codes(void) { return NOALLOC_CODE_BYTES; }
+extern "C" int64_t mi_w8a8_linear_noalloc_max_rows(void) { return NOALLOC_MAX_ROWS; }
+
+extern "C" int32_t mi_w8a8_linear_f32_noalloc(const float *x, const int8_t *qw, const float *sw, float *y, int64_t M,
+                                              int64_t N, int64_t K, int32_t block, void *stream)
+{
+    if (M < 0 || K <= 0) return MI_EINVAL;
+    if (M > NOALLOC_MAX_ROWS || K > NOALLOC_CODE_BYTES || M * K > NOALLOC_CODE_BYTES) return MI_ERANGE;
+    int device = -1;
+    MI_HIP(hipGetDevice(&device));
+    unsigned char *base = nullptr;
+    int32_t rc = linear_scratch_bind(device, &base);   // already bound when a context was created on this device
+    if (rc) return rc;
+    int8_t *qx = reinterpret_cast<int8_t *>(base);
+    float *sx = reinterpret_cast<float *>(base + NOALLOC_CODE_BYTES);
+    // nothing in the array has to start at zero: the quantizer writes every code and scale the contraction reads
+    return linear_with(x, qw, sw, y, M, N, K, block, qx, sx, stream);
 }

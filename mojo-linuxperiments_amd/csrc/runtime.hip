@@ -28,6 +28,8 @@ int32_t compute_units()
     return cached[dev];
 }
 
+int32_t linear_scratch_bind(int device, unsigned char **out);   // gemm.hip: address of the static scratch array
+
 __global__ void k_fill_u32(uint32_t *dst, uint32_t value, int64_t count)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -111,6 +113,10 @@ int32_t mi_ctx_create(int32_t device, mi_ctx **out)
     hipDeviceProp_t prop;
     MI_HIP(hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MI_ENODEV;
+    // the library's set-up call: look up this device's copy of the static scratch array now, so that
+    // mi_w8a8_linear_f32_noalloc never has to on a caller's critical path
+    int32_t rc = linear_scratch_bind(device, nullptr);
+    if (rc) return rc;
     mi_ctx *c = new (std::nothrow) mi_ctx;
     if (!c) return MI_ENOMEM;
     c->device = device;

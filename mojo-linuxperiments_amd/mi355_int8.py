@@ -86,6 +86,9 @@ SIGNATURES = {
     "mi_dequant_i32_f32": (i32, [vp, vp, vp, vp, i64, i64, vp]),
     "mi_w8a8_linear_workspace_bytes": (i64, [i64, i64, i64]),
     "mi_w8a8_linear_f32": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
+    "mi_w8a8_linear_f32_noalloc": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "mi_w8a8_linear_noalloc_max_rows": (i64, []),
+    "mi_w8a8_linear_noalloc_max_codes": (i64, []),
     "mi_gqa_decode_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
     "mi_gqa_decode_attn": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp]),
     "mi_gqa_decode_attn_cache": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64, vp]),
