@@ -82,6 +82,14 @@ extern "C" int32_t mi_dequant_i32_f32(const int32_t *acc, const float *sx, const
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// do the byte ranges [a, a + bytes) and [b, b + bytes) share a byte (null = no range)
+static bool overlaps(const void *a, const void *b, int64_t bytes)
+{
+    if (!a || !b) return false;
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return pa < pb + (uintptr_t)bytes && pb < pa + (uintptr_t)bytes;
+}
+
 extern "C" int64_t mi_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     (void)N;
@@ -103,7 +111,13 @@ extern "C" int32_t mi_rmsnorm_linear_f32(const float *x, const float *residual, 
     if (!x || !g || !sw || !aligned16(sw) || !aligned16(x) || !aligned16(g) || !(eps >= 0.0f)) return MI_EINVAL;
     if (residual && (!h_out || !aligned16(residual) || !aligned16(h_out))) return MI_EINVAL;
     if (xn_out && !aligned16(xn_out)) return MI_EINVAL;
-    if (M == 1 && block == 128) {
+    // The one-kernel form reads x and residual in every workgroup while one of them writes h_out / xn_out: a caller
+    // that updates its residual stream in place (h_out or xn_out overlapping x or residual) takes the two-kernel
+    // form, whose row operator reads each element before it writes it.
+    const int64_t row_bytes = M * K * 4;
+    const bool in_place = overlaps(h_out, x, row_bytes) || overlaps(h_out, residual, row_bytes) ||
+                          overlaps(xn_out, x, row_bytes) || overlaps(xn_out, residual, row_bytes);
+    if (M == 1 && block == 128 && !in_place) {
         rc = launch_norm_linear_fused(x, residual, g, eps, h_out, xn_out, qw, sw, y, qx, sx, M, N, K, as_stream(stream));
         if (rc != MI_EINVAL) return rc;
     }
