@@ -318,8 +318,10 @@ MI_API int32_t mi_rope_kv_append_f32_i8(const float *qkv, int64_t row_stride, co
 MI_API int32_t mi_swiglu_f32(const float *gate_up, float *h, int64_t M, int64_t I, void *stream);
 /* The two row operators above fused with the rotate + quantize prologue (mi_fwht_quant_f32_i8) of the linear that
  * consumes them: codes int8 [M,H] (resp. [M,I]) and scales fp32 [M] go straight to mi_w8a8_gemm_dequant_f32.
- * The arithmetic per element is that of the separate calls in the same order (codes are bit-identical to
- * quantizing the fp32 row the separate call writes).  y_out / h_out of the activated row are optional (NULL: the
+ * The arithmetic per element is that of the separate calls in the same order, and the sum of squares is taken in
+ * an order that depends on the row alone: one token gives the same codes whatever M it is batched in, here and in
+ * mi_rmsnorm_linear_f32, and they are the codes mi_fwht_quant_f32_i8 gives on the row y_out receives.
+ * (mi_rmsnorm_f32 sums the squares in another order: its row may differ from y_out in the last bit.)  y_out / h_out of the activated row are optional (NULL: the
  * fp32 row is never written); with a residual, h_out (the sum) is required as above.  H, I % block == 0. */
 MI_API int32_t mi_rmsnorm_quant_f32_i8(const float *x, const float *residual, const float *g, float eps,
                                        float *h_out, float *y_out, int8_t *q, float *scale,

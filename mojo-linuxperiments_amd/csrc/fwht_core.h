@@ -72,6 +72,38 @@ __device__ __forceinline__ float abs8(const float (&v)[8])
     return a;
 }
 
+// Sum of squares of a row in an order that depends on the row alone and not on how many threads share it, so that
+// a kernel of 256 threads and one of 1024 produce the same bits: the eight squares of a chunk are added in element
+// order, the 64 chunks of a group (chunk index / 64, one wave's worth) by a xor butterfly (every lane ends with
+// the same bits, a + b being b + a), and the groups pairwise in index order (tree_sum; absent groups count as 0,
+// which changes nothing).
+__device__ __forceinline__ float chunk_sumsq(const float (&v)[8])
+{
+    float s = v[0] * v[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) s += v[e] * v[e];
+    return s;
+}
+__device__ __forceinline__ float group_sum(float s)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
+    return s;
+}
+template <int G>
+__device__ __forceinline__ float tree_sum(const float *part)   // part[0 .. G-1], any G >= 1
+{
+    constexpr int P = G <= 1 ? 1 : 1 << (32 - __builtin_clz(G - 1));
+    float t[P];
+#pragma unroll
+    for (int w = 0; w < P; ++w) t[w] = w < G ? part[w] : 0.0f;
+#pragma unroll
+    for (int n = P; n > 1; n >>= 1)
+#pragma unroll
+        for (int w = 0; w < n / 2; ++w) t[w] = t[2 * w] + t[2 * w + 1];
+    return t[0];
+}
+
 __device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d, float inv)
 {
     const int i0 = (int)fminf(fmaxf(rintf(a * inv), -127.0f), 127.0f);

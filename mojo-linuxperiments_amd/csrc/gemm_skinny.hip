@@ -172,8 +172,8 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
     extern __shared__ __attribute__((aligned(16))) char s_dyn[];
     int8_t *s_x = reinterpret_cast<int8_t *>(s_dyn);                       // [MB][K] codes
     float *s_scale = reinterpret_cast<float *>(s_dyn + (size_t)MB * K);    // [MB]
-    float *s_max = s_scale + MB;                                           // [4] row maxima, then [4] sums of squares
-    int *s_red = reinterpret_cast<int *>(s_max + 8);                       // [4][V]
+    float *s_max = s_scale + MB;                                           // [4] row maxima, then [4 * CQ] sums of squares
+    int *s_red = reinterpret_cast<int *>(s_max + 4 + 4 * CQ);              // [4][V]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = wave % QW;                  // which CW-chunk slice of the row
     const int rows_per_wg = (4 / QW) * R;
@@ -214,9 +214,10 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
         const bool keeper = blockIdx.x == 0;   // one workgroup also leaves the codes and scales in the caller's workspace
         if constexpr (NORM) {
             float4 gl[CQ], gh[CQ];
-            float ss = 0.0f;
+            float ss[CQ];   // per chunk, then per group of 64 chunks (group wave + 4 * i): the order of fwht_core.h
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
+                ss[i] = 0.0f;
                 if (tid + i * 256 < nchunk) {
                     gl[i] = *reinterpret_cast<const float4 *>(nm.g + base[i]);
                     gh[i] = *reinterpret_cast<const float4 *>(nm.g + base[i] + BLOCK / 2);
@@ -231,16 +232,18 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
                             *reinterpret_cast<float4 *>(ho + BLOCK / 2) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
                         }
                     }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+                    ss[i] = chunk_sumsq(v[i]);
                 }
             }
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            for (int i = 0; i < CQ; ++i) ss[i] = group_sum(ss[i]);
             __syncthreads();   // the previous row's sums have been read
-            if (lane == 0) s_max[4 + wave] = ss;
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < CQ; ++i) s_max[4 + wave + 4 * i] = ss[i];
+            }
             __syncthreads();
-            const float total = (s_max[4] + s_max[5]) + (s_max[6] + s_max[7]);
+            const float total = tree_sum<4 * CQ>(s_max + 4);
             const float r = 1.0f / sqrtf(total / (float)K + nm.eps);
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
@@ -340,7 +343,7 @@ static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, f
 {
     constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);
     constexpr int V = pow2_ceil(R * MB);
-    const size_t lds = (size_t)MB * K + (MB + 8) * sizeof(float) + 4 * V * sizeof(int);
+    const size_t lds = (size_t)MB * K + (MB + 4 + 4 * CQ) * sizeof(float) + 4 * V * sizeof(int);
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ, NORM>),

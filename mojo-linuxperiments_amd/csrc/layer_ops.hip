@@ -148,16 +148,17 @@ __global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ 
 {
     constexpr int LPB = BLOCK / 8;
     constexpr int NW = TPB / 64;
-    __shared__ float s_part[NW], s_max[NW];
+    __shared__ float s_part[C * NW], s_max[NW];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int j = t % LPB;
     const int nchunk = K / 8;
     const int64_t row = blockIdx.x;
     float v[C][8];
     int base[C];
-    float ss = 0.0f;
+    float ss[C];   // sums of squares per chunk, then per group of 64 chunks (group wave + i * NW)
 #pragma unroll
     for (int i = 0; i < C; ++i) {
+        ss[i] = 0.0f;
         const int c = t + i * TPB;
         base[i] = (c / LPB) * BLOCK + 4 * j;
         if (c < nchunk) {
@@ -175,8 +176,7 @@ __global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ 
                 }
                 v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
                 v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+                ss[i] = chunk_sumsq(v[i]);
             } else {
                 const float *gr = x + row * 2 * (int64_t)K + base[i];
                 const float4 gl = *reinterpret_cast<const float4 *>(gr), gh = *reinterpret_cast<const float4 *>(gr + BLOCK / 2);
@@ -202,18 +202,12 @@ __global__ __launch_bounds__(TPB) void k_row_op_quant(const float *__restrict__ 
             }
         }
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
-        if (lane == 0) s_part[wave] = ss;
+        for (int i = 0; i < C; ++i) {
+            ss[i] = group_sum(ss[i]);
+            if (lane == 0) s_part[wave + i * NW] = ss[i];
+        }
         __syncthreads();
-        // pairwise over the waves' partial sums (a fixed order)
-        float part[NW];
-#pragma unroll
-        for (int w = 0; w < NW; ++w) part[w] = s_part[w];
-#pragma unroll
-        for (int n = NW; n > 1; n >>= 1)
-#pragma unroll
-            for (int w = 0; w < n / 2; ++w) part[w] = part[2 * w] + part[2 * w + 1];
-        const float total = part[0];
+        const float total = tree_sum<C * NW>(s_part);   // the order of fwht_core.h: the same bits whatever TPB is
         const float r = 1.0f / sqrtf(total / (float)K + eps);
 #pragma unroll
         for (int i = 0; i < C; ++i) {

@@ -325,3 +325,67 @@ def test_rmsnorm_linear_one_call(mi, dev, orc, M, N, K):
     assert mi.lib.mi_rmsnorm_linear_f32(dx.ptr, dr.ptr, dg.ptr, 1e-5, None, None, dqw.ptr, dsw.ptr, dy.ptr, M, N, K, 128,
                                         ws.ptr, ws.nbytes, None) == mi.EINVAL     # residual without h_out
     dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (1, 272, 2048), (4, 512, 4096)])
+@pytest.mark.parametrize("target", ["residual", "x"])
+def test_rmsnorm_linear_residual_stream_updated_in_place(mi, dev, orc, M, N, K, target):
+    """h_out written over the residual (or over x), the way a decoder updates its residual stream: the one-kernel
+    form reads both rows in every workgroup, so such a call has to give what separate buffers give."""
+    mark = dev.mark()
+    g = np.random.default_rng(5 * M + N + K)
+    x = workload.activations(72, M, K)
+    r = g.standard_normal((M, K)).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(K)).astype(np.float32)
+    qw = g.integers(-127, 128, (N, K)).astype(np.int8)
+    sw = ((g.random(N) + 0.5) * 0.01).astype(np.float32)
+    dx, dr, dg, dqw, dsw = dev.upload(x), dev.upload(r), dev.upload(w), dev.upload(qw), dev.upload(sw)
+    dh, dy, dy2 = dev.empty((M, K), np.float32), dev.empty((M, N), np.float32), dev.empty((M, N), np.float32)
+    ws = dev.empty(mi.lib.mi_w8a8_linear_workspace_bytes(M, N, K), np.uint8)
+    mi.check(mi.lib.mi_rmsnorm_linear_f32(dx.ptr, dr.ptr, dg.ptr, 1e-5, dh.ptr, None, dqw.ptr, dsw.ptr, dy.ptr, M, N, K,
+                                          128, ws.ptr, ws.nbytes, None), "separate buffers")
+    y_sep, h_sep = dev.download(dy), dev.download(dh)
+    codes_sep = dev.download(ws.offset(0, (M, K), np.int8))
+    for _ in range(3):   # the race needs workgroups to start after the keeper has written: several tries, each from fresh rows
+        mi.check(mi.lib.mi_memcpy_h2d(dx.ptr, x.ctypes.data, x.nbytes, None))
+        mi.check(mi.lib.mi_memcpy_h2d(dr.ptr, r.ctypes.data, r.nbytes, None))
+        dev.sync()
+        dst = dr if target == "residual" else dx
+        mi.check(mi.lib.mi_rmsnorm_linear_f32(dx.ptr, dr.ptr, dg.ptr, 1e-5, dst.ptr, None, dqw.ptr, dsw.ptr, dy2.ptr, M, N,
+                                              K, 128, ws.ptr, ws.nbytes, None), "in place")
+        assert np.array_equal(dev.download(dst), h_sep)
+        assert np.array_equal(dev.download(ws.offset(0, (M, K), np.int8)), codes_sep)
+        assert np.array_equal(dev.download(dy2), y_sep)
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("K", [2048, 4096])
+def test_one_token_gets_the_same_codes_alone_and_in_a_batch(mi, dev, K):
+    """The one-kernel form (M = 1) and the row operator (M > 1) sum the squares in the same order: a token's
+    normalized row, codes and scale do not depend on the batch it arrives in."""
+    mark = dev.mark()
+    N = 256
+    g = np.random.default_rng(K)
+    x = workload.activations(73, 3, K)
+    r = g.standard_normal((3, K)).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(K)).astype(np.float32)
+    qw = g.integers(-127, 128, (N, K)).astype(np.int8)
+    sw = ((g.random(N) + 0.5) * 0.01).astype(np.float32)
+    dg, dqw, dsw = dev.upload(w), dev.upload(qw), dev.upload(sw)
+    ws = dev.empty(mi.lib.mi_w8a8_linear_workspace_bytes(3, N, K), np.uint8)
+
+    def run(rows):
+        M = len(rows)
+        dx, dr = dev.upload(x[rows]), dev.upload(r[rows])
+        dh, dxn, dy = dev.empty((M, K), np.float32), dev.empty((M, K), np.float32), dev.empty((M, N), np.float32)
+        mi.check(mi.lib.mi_rmsnorm_linear_f32(dx.ptr, dr.ptr, dg.ptr, 1e-5, dh.ptr, dxn.ptr, dqw.ptr, dsw.ptr, dy.ptr, M, N,
+                                              K, 128, ws.ptr, ws.nbytes, None), "mi_rmsnorm_linear_f32")
+        sx_off = (M * K + 255) // 256 * 256
+        return (dev.download(dxn), dev.download(ws.offset(0, (M, K), np.int8)),
+                dev.download(ws.offset(sx_off, (M,), np.float32)), dev.download(dy))
+    batch = run([0, 1, 2])
+    for m in range(3):
+        alone = run([m])
+        for a, b in zip(alone, batch):
+            assert np.array_equal(a[0], b[m])
+    dev.reset_to(mark)
