@@ -371,7 +371,10 @@ def decode_gemv(mi, wl, dev, pool, s, timer, shapes, next_w):
 
 
 def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
-    """cfg2: B=16, 32/8 heads, D=128, T=4096; three KV sets (402 MB) in rotation."""
+    """cfg2: B=16, 32/8 heads, D=128, T=4096; three KV sets in rotation (402 MB per layout).  The headline is the
+    cache in the matrix-pipe layouts (keys in 16-token tiles, values in transposed 64-token blocks: the layouts the
+    decode chain keeps its cache in); the row-major cache [T, 128] is timed beside it, dense, with the append in
+    front, and paged."""
     lib = mi.lib
     c = wl.ATTN
     B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
@@ -382,31 +385,41 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
     for i in range(3):
         kq, ks = dev.empty((B, Hkv, T, D), np.int8), dev.empty((B, Hkv, T), np.float32)
         vq, vs = dev.empty((B, Hkv, T, D), np.int8), dev.empty((B, Hkv, T), np.float32)
+        kt, vt = dev.empty((B, Hkv, T, D), np.int8), dev.empty((B, Hkv, T, D), np.int8)
         mi.check(lib.mi_fwht_quant_f32_i8(src.ptr, kq.ptr, ks.ptr, rows, D, D, s))
         mi.check(lib.mi_fwht_quant_f32_i8(src.ptr, vq.ptr, vs.ptr, rows, D, D, s))
-        sets.append((kq, ks, vq, vs))
+        mi.check(lib.mi_kv_tiled_from_rows_i8(kq.ptr, vq.ptr, kt.ptr, vt.ptr, B * Hkv, T, T, T, s))
+        sets.append((kq, ks, vq, vs, kt, vt))
     dq = dev.upload(wl.normal(88, (B, Hq, D), 1))
     do = dev.empty((B, Hq, D), np.float32)
     ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T), np.uint8)
-    calls = [(lambda k=k: mi.gqa_decode(dq, k[0], k[1], k[2], k[3], do, False, ws, stream=s)) for k in sets]
-    ms = graph_time(mi, dev, s, timer, calls, reps) if graph else eager_time(dev, s, timer, calls)
+    run = (lambda calls: graph_time(mi, dev, s, timer, calls, reps)) if graph else (lambda calls: eager_time(dev, s, timer, calls))
     nbytes = wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
-    # the same step as a decode loop runs it: the new token's K and V heads are appended (rotate + quantize + write
-    # at position T-1 of every sequence), then attention reads the cache through per-sequence lengths
     knew = dev.upload(wl.normal(88, (B, Hkv, D), 2))
     vnew = dev.upload(wl.normal(88, (B, Hkv, D), 3))
     dpos = dev.upload(np.full(B, T - 1, np.int32))
     dlen = dev.upload(np.full(B, T, np.int32))
+
+    def tiled(k, append):
+        # as a decode loop runs it: the new token's K and V heads are appended (rotate + quantize + write at
+        # position T-1 of every sequence), then attention reads the cache through per-sequence lengths
+        if append:
+            mi.check(lib.mi_kv_append_tiled_f32_i8(knew.ptr, vnew.ptr, Hkv * D, k[4].ptr, k[1].ptr, k[5].ptr, k[3].ptr,
+                                                   dpos.ptr, B, Hkv, D, T, s))
+        mi.check(lib.mi_gqa_decode_attn_tiled(dq.ptr, k[4].ptr, k[1].ptr, k[5].ptr, k[3].ptr, do.ptr, B, Hq, Hkv, D, T,
+                                              dlen.ptr if append else None, T, 0, ws.ptr, ws.nbytes, s))
+    ms = run([(lambda k=k: tiled(k, False)) for k in sets])
+    ms_app = run([(lambda k=k: tiled(k, True)) for k in sets])
+    ms_rows = run([(lambda k=k: mi.gqa_decode(dq, k[0], k[1], k[2], k[3], do, False, ws, stream=s)) for k in sets])
 
     def cached(k):
         mi.check(lib.mi_kv_append_f32_i8(knew.ptr, vnew.ptr, Hkv * D, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr,
                                          dpos.ptr, B, Hkv, D, T, s))
         mi.check(lib.mi_gqa_decode_attn_cache(dq.ptr, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr, do.ptr, B, Hq, Hkv, D,
                                               T, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
-    calls2 = [(lambda k=k: cached(k)) for k in sets]
-    ms2 = graph_time(mi, dev, s, timer, calls2, reps) if graph else eager_time(dev, s, timer, calls2)
-    # the same caches read as pools of 16-token pages under a shuffled block table (the rows a pool holds are the
-    # same bytes; which token sits where does not change the time)
+    ms_rows_app = run([(lambda k=k: cached(k)) for k in sets])
+    # the row-major caches read as pools of 16-token pages under a shuffled block table (the rows a pool holds are
+    # the same bytes; which token sits where does not change the time)
     P = 16
     max_pages = T // P
     table = np.random.default_rng(3).permutation(B * max_pages).astype(np.int32).reshape(B, max_pages)
@@ -415,14 +428,16 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
     def paged(k):
         mi.check(lib.mi_gqa_decode_attn_paged(dq.ptr, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr, do.ptr, dtab.ptr,
                                               max_pages, P, B, Hq, Hkv, D, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
-    calls3 = [(lambda k=k: paged(k)) for k in sets]
-    ms3 = graph_time(mi, dev, s, timer, calls3, reps) if graph else eager_time(dev, s, timer, calls3)
+    ms_paged = run([(lambda k=k: paged(k)) for k in sets])
     dev.reset_to(mark)
     return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                       "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes,
-                                      "with_kv_append_us": round(ms2 * 1e3, 2),
-                                      "paged_16_token_pages_us": round(ms3 * 1e3, 2)}}
+                                      "cache_layout": "keys in 16-token tiles, values in transposed 64-token blocks",
+                                      "with_kv_append_us": round(ms_app * 1e3, 2),
+                                      "row_major_cache_us": round(ms_rows * 1e3, 2),
+                                      "row_major_with_kv_append_us": round(ms_rows_app * 1e3, 2),
+                                      "row_major_paged_16_token_pages_us": round(ms_paged * 1e3, 2)}}
 
 
 def eager_time(dev, s, timer, calls):
@@ -517,8 +532,7 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None, nlayers=3):
         # a cache of real rows: rotate + quantize N(0,1) keys and values
         m2 = dev.mark()
         src = dev.upload(csrc[li % 3])
-        mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.kq.ptr, L.ks.ptr, B * Hkv * T, D, D, s))
-        mi.check(mi.lib.mi_fwht_quant_f32_i8(src.ptr, L.vq.ptr, L.vs.ptr, B * Hkv * T, D, D, s))
+        L.fill_cache_from_rows(src, T, s)
         dev.sync(s)
         dev.reset_to(m2)
         layers.append(L)

@@ -248,6 +248,44 @@ MI_API int32_t mi_kv_append_paged_f32_i8(const float *k_new, const float *v_new,
 MI_API int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
                                    int8_t *kq, float *ks, int8_t *vq, float *vs, const int32_t *pos,
                                    int64_t B, int64_t Hkv, int64_t D, int64_t T_cap, void *stream);
+/* ---- the same attention over a cache stored in the two layouts the int8 matrix instruction loads straight from
+ * memory (1 KB contiguous per wave instruction, nothing converted or transposed on the way):
+ *   kt int8 [B, Hkv, T_cap/16, 8, 16, 16]  tile of 16 tokens: byte (c, t % 16, e) = code 16*c + e of token t
+ *   vt int8 [B, Hkv, T_cap/64, 8, 4, 16, 16]  block of 64 tokens, transposed, in 16 x 16 pieces:
+ *                                          byte (d / 16, (t % 64) / 16, d % 16, t % 16) = code d of token t
+ * ks, vs fp32 [B, Hkv, T_cap] as above (16-byte aligned); T_cap % 64 == 0.  Both products of the attention run on
+ * the int8 matrix pipe (the softmax weights times the V scales enter as 28-bit fixed-point numbers, finer than
+ * fp32's mantissa, so the result is that of the fp32 accumulation to within rounding): the fast layout, and the one
+ * the decode-layer chain uses.  seq_len may be NULL (every sequence holds T_max tokens).  Workspace:
+ * mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max) (one query serves both layouts).  Bytes that belong to tokens
+ * at or past a sequence's length are never used (they may hold anything).  No upstream counterpart. */
+MI_API int32_t mi_gqa_decode_attn_tiled(const float *q, const int8_t *kt, const float *ks,
+                                        const int8_t *vt, const float *vs, float *o,
+                                        int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                        const int32_t *seq_len, int64_t T_max, int32_t out_rotated,
+                                        void *workspace, int64_t workspace_bytes, void *stream);
+/* ... with the merge fused with the output projection's row quantizer, as mi_gqa_decode_attn_cache_quant_i8. */
+MI_API int32_t mi_gqa_decode_attn_tiled_quant_i8(const float *q, const int8_t *kt, const float *ks,
+                                                 const int8_t *vt, const float *vs, float *o_rot,
+                                                 int8_t *oq, float *oscale,
+                                                 int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                                 const int32_t *seq_len, int64_t T_max,
+                                                 void *workspace, int64_t workspace_bytes, void *stream);
+/* Row-major codes [rows, src_stride tokens, 128] (rows = B*Hkv) -> the tiled layouts, first T tokens of every row
+ * (the rest of the last 64-token block touched is zero-filled); either pair (kq, kt) / (vq, vt) may be NULL.  For
+ * caches that were quantized in one go (prefill) with mi_fwht_quant_f32_i8. */
+MI_API int32_t mi_kv_tiled_from_rows_i8(const int8_t *kq, const int8_t *vq, int8_t *kt, int8_t *vt,
+                                        int64_t rows, int64_t T, int64_t src_stride, int64_t T_cap, void *stream);
+/* mi_kv_append_f32_i8 and mi_rope_kv_append_f32_i8 for these layouts (same arithmetic, same codes and scales, at
+ * the tiled places of token pos[b]). */
+MI_API int32_t mi_kv_append_tiled_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                         int8_t *kt, float *ks, int8_t *vt, float *vs, const int32_t *pos,
+                                         int64_t B, int64_t Hkv, int64_t D, int64_t T_cap, void *stream);
+MI_API int32_t mi_rope_kv_append_tiled_f32_i8(const float *qkv, int64_t row_stride, const float *rope_cos,
+                                              const float *rope_sin, float *q_out, int8_t *kt, float *ks,
+                                              int8_t *vt, float *vs, const int32_t *pos,
+                                              int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                              void *stream);
 /* Gate helper: runs the same split kernel and also writes out the int8 query
  * codes [B,Hq,D], their scales [B,Hq] and the raw int32 scores [B,Hq,T] it
  * works from (no merge, no o). */

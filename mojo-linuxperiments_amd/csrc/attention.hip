@@ -10,13 +10,10 @@
 // tokens of one KV head once and serves the G = Hq/Hkv <= 4 query heads that
 // share it.  A second small kernel merges the splits.
 //
-// Both passes load 16 bytes per lane in token-major order (lane l: token l/8
-// of an 8-token group, bytes 16*(l%8)..+15), i.e. 1 KB contiguous per wave
-// instruction, eight instructions in flight per wave.
-// Pass 1 (scores).  Each lane runs v_dot4_i32_i8 of its 16 key bytes against
-// the matching 16 query-code bytes of the G heads; the 8 lanes of a token add
-// their int32 partial sums (lane xor 1, 2, 4).  Scores (already in log2 units)
-// go to LDS, the running max stays in registers.
+// Pass 1 (scores).  Keys are loaded straight in MFMA operand layout (lane l: token l%16 of a 16-token tile,
+// 16-byte chunk l/16 of each half of the head dimension); two v_mfma_i32_16x16x64_i8 per tile against the
+// query codes of the G heads give the exact int32 dot products (lane l < 16: token l, register r: head r).
+// Scores (already in log2 units) go to LDS, the running max stays in registers.
 // Pass 2 (P.V).  v_mfma_f32_4x4x1_16B_f32 treats each aligned group of
 // four lanes as one 4x4 outer product: the four lanes share a token, lane
 // l%4 = i supplies p(token, head i) * vs(token) as the A value and one V
@@ -28,9 +25,13 @@
 //
 // Bound: HBM.  Algorithmic bytes = K and V codes (2*B*Hkv*T*D) + their scales
 // (8*B*Hkv*T) + q and o (8*B*Hq*D).
-#include "common.h"
+#include "fwht_core.h"
 
 namespace mi {
+
+namespace avt {
+int max_splits(int64_t B, int64_t Hkv, int64_t T);   // attention_tiled.hip: the block-transposed V layout's own plan
+}
 
 namespace attn {
 
@@ -48,43 +49,7 @@ __device__ __forceinline__ float lane_xor(float v)
     return __int_as_float(r);
 }
 
-// normalized 128-point Hadamard over 16 lanes x 8 values, stage order h = 1, 2, ..., 64
-__device__ __forceinline__ void fwht128(float (&v)[8], int j)
-{
-#pragma unroll
-    for (int b = 0; b < 8; b += 4) {
-        float a0 = v[b] + v[b + 1], a1 = v[b] - v[b + 1];
-        float a2 = v[b + 2] + v[b + 3], a3 = v[b + 2] - v[b + 3];
-        v[b] = a0 + a2; v[b + 2] = a0 - a2;
-        v[b + 1] = a1 + a3; v[b + 3] = a1 - a3;
-    }
-#define MI_STAGE(MASK)                                                                              \
-    {                                                                                               \
-        const unsigned neg = (j & MASK) ? 0x80000000u : 0u;                                         \
-        _Pragma("unroll") for (int e = 0; e < 8; ++e)                                               \
-        {                                                                                           \
-            const float other = lane_xor<MASK>(v[e]);                                               \
-            v[e] = other + __int_as_float(__float_as_int(v[e]) ^ neg);                              \
-        }                                                                                           \
-    }
-    MI_STAGE(1) MI_STAGE(2) MI_STAGE(4) MI_STAGE(8)
-#undef MI_STAGE
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float lo = v[e] + v[e + 4], hi = v[e] - v[e + 4];
-        v[e] = lo * 0.08838834764831845f;
-        v[e + 4] = hi * 0.08838834764831845f;
-    }
-}
-
-__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d, float inv)
-{
-    const int i0 = (int)fminf(fmaxf(rintf(a * inv), -127.0f), 127.0f);
-    const int i1 = (int)fminf(fmaxf(rintf(b * inv), -127.0f), 127.0f);
-    const int i2 = (int)fminf(fmaxf(rintf(c * inv), -127.0f), 127.0f);
-    const int i3 = (int)fminf(fmaxf(rintf(d * inv), -127.0f), 127.0f);
-    return (uint32_t)(i0 & 0xff) | ((uint32_t)(i1 & 0xff) << 8) | ((uint32_t)(i2 & 0xff) << 16) | ((uint32_t)i3 << 24);
-}
+__device__ __forceinline__ void fwht128(float (&v)[8], int j) { fwht_chunk<D>(v, j); }   // fwht_core.h
 
 struct Params {
     const float *q;
@@ -597,6 +562,49 @@ static int max_splits(int64_t B, int64_t Hkv, int64_t T)
     return best;
 }
 
+// Merge of the splits' partial results [B*Hkv, splits, 4, 128] / [B*Hkv, splits, 2, 4].  oq: one workgroup per token
+// merges its Hq rows and quantizes them for the output projection (o then optionally receives the fp32 row in the
+// rotated basis); otherwise 16 rows per workgroup into o.
+int32_t launch_merge(const float *part_o, const float *part_ml, float *o, int8_t *oq, float *oscale, int64_t B,
+                     int64_t Hq, int64_t Hkv, int splits, int out_rotated, hipStream_t s)
+{
+    const int G = (int)(Hq / Hkv);
+    if (oq) {
+#define MI_MERGEQ(SP)                                                                                           \
+    hipLaunchKernelGGL(k_gqa_merge_quant<SP>, dim3((unsigned)B), dim3((unsigned)(Hq * 16)), 0, s, part_o, part_ml, \
+                       o, oq, oscale, (int)Hq, (int)Hkv, G, splits)
+        switch (splits) {
+        case 1: MI_MERGEQ(1); break;
+        case 2: MI_MERGEQ(2); break;
+        case 4: MI_MERGEQ(4); break;
+        case 6: MI_MERGEQ(6); break;
+        case 8: MI_MERGEQ(8); break;
+        case 12: MI_MERGEQ(12); break;
+        case 16: MI_MERGEQ(16); break;
+        default: MI_MERGEQ(0); break;
+        }
+#undef MI_MERGEQ
+        return launch_status();
+    }
+    const int rows = (int)(B * Hq);
+    const dim3 mgrid((unsigned)((rows + 15) / 16));
+#define MI_MERGE(SP)                                                                                              \
+    hipLaunchKernelGGL(k_gqa_merge<SP>, mgrid, dim3(256), 0, s, part_o, part_ml, o, rows, (int)Hq, (int)Hkv, G, \
+                       splits, out_rotated)
+    switch (splits) {
+    case 1: MI_MERGE(1); break;
+    case 2: MI_MERGE(2); break;
+    case 4: MI_MERGE(4); break;
+    case 6: MI_MERGE(6); break;
+    case 8: MI_MERGE(8); break;
+    case 12: MI_MERGE(12); break;
+    case 16: MI_MERGE(16); break;
+    default: MI_MERGE(0); break;
+    }
+#undef MI_MERGE
+    return launch_status();
+}
+
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace attn
@@ -619,7 +627,9 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
     if (rc) return rc;
     // an upper bound over every length up to T, so that a workspace sized for the capacity of a cache serves every
     // decode step: the plan is not monotone in T (a shorter sequence may be cut into more, shorter spans)
-    const int splits = attn::max_splits(B, Hkv, T);
+    int splits = attn::max_splits(B, Hkv, T);
+    const int splits_vt = avt::max_splits(B, Hkv, T);   // one query serves both cache layouts
+    if (splits_vt > splits) splits = splits_vt;
     return attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256) + attn::align_up(B * Hkv * splits * 8 * 4, 256);
 }
 
@@ -661,42 +671,8 @@ static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const
     }
     rc = launch_status();
     if (rc) return rc;
-    if (oq) {
-        // one workgroup per token merges its Hq rows and quantizes them for the output projection
-#define MI_MERGEQ(SP)                                                                                              \
-    hipLaunchKernelGGL(attn::k_gqa_merge_quant<SP>, dim3((unsigned)B), dim3((unsigned)(Hq * 16)), 0, s, p.part_o, \
-                       p.part_ml, o, oq, oscale, (int)Hq, (int)Hkv, p.G, splits)
-        switch (splits) {
-        case 1: MI_MERGEQ(1); break;
-        case 2: MI_MERGEQ(2); break;
-        case 4: MI_MERGEQ(4); break;
-        case 6: MI_MERGEQ(6); break;
-        case 8: MI_MERGEQ(8); break;
-        case 12: MI_MERGEQ(12); break;
-        case 16: MI_MERGEQ(16); break;
-        default: MI_MERGEQ(0); break;
-        }
-#undef MI_MERGEQ
-        return launch_status();
-    }
-    if (!o) return rc;
-    const int rows = (int)(B * Hq);
-    const dim3 mgrid((unsigned)((rows + 15) / 16));
-#define MI_MERGE(SP)                                                                                        \
-    hipLaunchKernelGGL(attn::k_gqa_merge<SP>, mgrid, dim3(256), 0, s, p.part_o, p.part_ml, o, rows, (int)Hq, \
-                       (int)Hkv, p.G, splits, out_rotated)
-    switch (splits) {
-    case 1: MI_MERGE(1); break;
-    case 2: MI_MERGE(2); break;
-    case 4: MI_MERGE(4); break;
-    case 6: MI_MERGE(6); break;
-    case 8: MI_MERGE(8); break;
-    case 12: MI_MERGE(12); break;
-    case 16: MI_MERGE(16); break;
-    default: MI_MERGE(0); break;
-    }
-#undef MI_MERGE
-    return launch_status();
+    if (!o && !oq) return rc;
+    return attn::launch_merge(p.part_o, p.part_ml, o, oq, oscale, B, Hq, Hkv, splits, out_rotated, s);
 }
 
 extern "C" int32_t mi_gqa_decode_attn(const float *q, const int8_t *kq, const float *ks, const int8_t *vq,

@@ -86,16 +86,6 @@ __device__ __forceinline__ void dma16(const int8_t *sbase, unsigned voff, unsign
                  : "v"(voff), "s"(sbase), "s"(ldsaddr)
                  : "memory", "m0");
 }
-template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>)
-{
-    (f(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&f)
-{
-    static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
-}
 // how many second-half activation fragments are fetched during group g of the first half
 template <int TM, int TN>
 constexpr int xb1_count(int g)

@@ -105,6 +105,12 @@ SIGNATURES = {
                                        vp]),
     "mi_kv_append_paged_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
+    "mi_gqa_decode_attn_tiled": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64, vp]),
+    "mi_gqa_decode_attn_tiled_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, vp, i64,
+                                             vp]),
+    "mi_kv_tiled_from_rows_i8": (i32, [vp, vp, vp, vp, i64, i64, i64, i64, vp]),
+    "mi_kv_append_tiled_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
+    "mi_rope_kv_append_tiled_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_moe_route_workspace_bytes": (i64, [i64, i64]),
     "mi_moe_route": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
@@ -381,6 +387,30 @@ def moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, topk, ws, stream=None):
                            T, H, I, E, topk, ws.ptr, ws.nbytes, stream), "mi_moe_layer")
 
 
+# ---- the matrix-pipe cache layouts restated in numpy (test and bench plumbing: what goes where) ----
+
+def kv_rows_to_tiled(kq, vq, T_cap):
+    """row-major codes [B,Hkv,T,128] -> kt [B,Hkv,T_cap/16,8,16,16] (chunk, token, byte) and
+    vt [B,Hkv,T_cap/64,8,4,16,16] (dim piece, token chunk, dim, token); tokens past T are zero."""
+    B, Hkv, T, D = kq.shape
+
+    def pad(a):
+        out = np.zeros((B, Hkv, T_cap, D), np.int8)
+        out[:, :, :T] = a
+        return out
+    kt = np.ascontiguousarray(pad(kq).reshape(B, Hkv, T_cap // 16, 16, 8, 16).transpose(0, 1, 2, 4, 3, 5))
+    vt = np.ascontiguousarray(pad(vq).reshape(B, Hkv, T_cap // 64, 4, 16, 8, 16).transpose(0, 1, 2, 5, 3, 6, 4))
+    return kt, vt
+
+
+def kv_tiled_to_rows(kt, vt):
+    B, Hkv = kt.shape[:2]
+    T_cap = kt.size // (B * Hkv * 128)
+    kq = np.ascontiguousarray(kt.reshape(B, Hkv, T_cap // 16, 8, 16, 16).transpose(0, 1, 2, 4, 3, 5)).reshape(B, Hkv, T_cap, 128)
+    vq = np.ascontiguousarray(vt.reshape(B, Hkv, T_cap // 64, 8, 4, 16, 16).transpose(0, 1, 2, 4, 6, 3, 5)).reshape(B, Hkv, T_cap, 128)
+    return kq, vq
+
+
 class DecoderLayer:
     """One decoder layer of a decode step, chained from the C-ABI entry points on one stream:
     (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + KV-cache append -> attention over the cache (split,
@@ -390,8 +420,10 @@ class DecoderLayer:
     (xn, att, hn, act) so that a test can gate every stage."""
 
     def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
-                 block=128, trace=False):
+                 block=128, trace=False, tiled=None):
         D = 128
+        # the cache lives in the matrix-pipe layouts whenever its capacity allows (a multiple of 64 tokens)
+        self.tiled = (T_cap % 64 == 0) if tiled is None else bool(tiled)
         self.dev, self.B, self.H, self.Hq, self.Hkv, self.I, self.T_cap, self.eps, self.block = \
             dev, B, H, Hq, Hkv, I, T_cap, eps, block
         self.NQKV = (Hq + 2 * Hkv) * D
@@ -436,15 +468,15 @@ class DecoderLayer:
                                         self.wqkv[1].ptr, self.qkv.ptr, B, self.NQKV, H, self.block, self.lin_ws.ptr,
                                         self.lin_ws.nbytes, s), "mi_rmsnorm_linear_f32")
         xin = self.h0 if residual is not None else x
-        check(lib.mi_rope_kv_append_f32_i8(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr,
-                                           self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv,
-                                           D, self.T_cap, s), "mi_rope_kv_append_f32_i8")
+        append = lib.mi_rope_kv_append_tiled_f32_i8 if self.tiled else lib.mi_rope_kv_append_f32_i8
+        check(append(self.qkv.ptr, self.NQKV, self.cos.ptr, self.sin.ptr, self.q.ptr, self.kq.ptr, self.ks.ptr,
+                     self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv, D, self.T_cap, s), "mi_rope_kv_append")
         # attention output stays in the rotated basis of V and is quantized by the merge itself: the O weights were
         # rotated with block 128 = head_dim along K, so their GEMV takes these codes as they are
-        check(lib.mi_gqa_decode_attn_cache_quant_i8(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
-                                                    p(self.att), self.ca.ptr, self.sa.ptr, B, Hq, Hkv, D, self.T_cap,
-                                                    seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
-              "mi_gqa_decode_attn_cache_quant_i8")
+        attend = lib.mi_gqa_decode_attn_tiled_quant_i8 if self.tiled else lib.mi_gqa_decode_attn_cache_quant_i8
+        check(attend(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, p(self.att), self.ca.ptr,
+                     self.sa.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
+              "mi_gqa_decode_attn_quant_i8")
         gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
         check(lib.mi_rmsnorm_linear_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
                                         self.wgu[0].ptr, self.wgu[1].ptr, self.gu.ptr, B, 2 * I, H, self.block,
@@ -454,3 +486,33 @@ class DecoderLayer:
         gemm_dequant(self.ci, self.si, self.wd[0], self.wd[1], self.dn, s)
         if out is not None:
             check(lib.mi_add_f32(self.h1.ptr, self.dn.ptr, out.ptr, B * H, s), "mi_add_f32")
+
+    # the cache as row-major arrays [B,Hkv,T_cap,128] / [B,Hkv,T_cap], whatever layout the layer keeps it in
+    def set_cache_rows(self, kq, ks, vq, vs):
+        if self.tiled:
+            kq, vq = kv_rows_to_tiled(kq, vq, self.T_cap)
+        for buf, a in ((self.kq, kq), (self.ks, ks), (self.vq, vq), (self.vs, vs)):
+            a = np.ascontiguousarray(a)
+            check(lib.mi_memcpy_h2d(buf.ptr, a.ctypes.data, a.nbytes, None), "mi_memcpy_h2d")
+        self.dev.sync()
+
+    def get_cache_rows(self):
+        kq, ks, vq, vs = (self.dev.download(b) for b in (self.kq, self.ks, self.vq, self.vs))
+        if self.tiled:
+            kq, vq = kv_tiled_to_rows(kq, vq)
+        return kq, ks, vq, vs
+
+    def fill_cache_from_rows(self, src, T, stream=None):
+        """rotate + quantize fp32 rows [B*Hkv*T, 128] (device) into both halves of the cache (bench set-up)"""
+        B, Hkv, D = self.B, self.Hkv, 128
+        if not self.tiled:
+            check(lib.mi_fwht_quant_f32_i8(src.ptr, self.kq.ptr, self.ks.ptr, B * Hkv * T, D, D, stream))
+            check(lib.mi_fwht_quant_f32_i8(src.ptr, self.vq.ptr, self.vs.ptr, B * Hkv * T, D, D, stream))
+            return
+        mark = self.dev.mark()
+        rows = self.dev.empty((B * Hkv * T, D), np.int8)
+        check(lib.mi_fwht_quant_f32_i8(src.ptr, rows.ptr, self.ks.ptr, B * Hkv * T, D, D, stream))
+        check(lib.mi_memcpy_d2d(self.vs.ptr, self.ks.ptr, B * Hkv * T * 4, stream))
+        check(lib.mi_kv_tiled_from_rows_i8(rows.ptr, rows.ptr, self.kq.ptr, self.vq.ptr, B * Hkv, T, T, self.T_cap, stream))
+        self.dev.sync(stream)
+        self.dev.reset_to(mark)

@@ -199,11 +199,16 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
              g.integers(-127, 128, (B, Hkv, T_cap, D)).astype(np.int8),
              ((g.random((B, Hkv, T_cap)) + 0.5) * 0.03).astype(np.float32)]
     free = [c.copy() for c in cache]
-    for buf, ref in zip((layer.kq, layer.ks, layer.vq, layer.vs), cache):
-        mi.check(mi.lib.mi_memcpy_h2d(buf.ptr, ref.ctypes.data, ref.nbytes, None))
+    assert layer.tiled == (T_cap % 64 == 0)      # capacities of 64 and 128 tokens run the matrix-pipe layouts
+    layer.set_cache_rows(*cache)
     dpos, dlen = dev.empty(B, np.int32), dev.empty(B, np.int32)
     dx, dout = dev.empty((B, H), np.float32), dev.empty((B, H), np.float32)
-    names = ("xn", "qkv", "q", "att", "ca", "sa", "ao", "h1", "hn", "gu", "act", "dn", "kq", "ks", "vq", "vs")
+    names = ("xn", "qkv", "q", "att", "ca", "sa", "ao", "h1", "hn", "gu", "act", "dn")
+
+    def snapshot():
+        got = {n: dev.download(getattr(layer, n)) for n in names}
+        got["kq"], got["ks"], got["vq"], got["vs"] = layer.get_cache_rows()
+        return got
     for step in range(3):
         pos = (start + step).astype(np.int32)
         lens = (pos + 1).astype(np.int32)
@@ -212,7 +217,7 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
             mi.check(mi.lib.mi_memcpy_h2d(d.ptr, a.ctypes.data, a.nbytes, None))
         layer.step(dx, dpos, dlen, int(lens.max()), dout)
         out = dev.download(dout)
-        gpu = {n: dev.download(getattr(layer, n)) for n in names}
+        gpu = snapshot()
         gpu["q"] = gpu["q"].reshape(B, Hq, D)
         # stage by stage, each stage fed what the GPU fed it: integer stages bit-exact
         staged = oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=gpu)
@@ -230,7 +235,7 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
     for d, a in ((dpos, pos), (dlen, lens)):
         mi.check(mi.lib.mi_memcpy_h2d(d.ptr, a.ctypes.data, a.nbytes, None))
     layer.step(d_dn, dpos, dlen, int(lens.max()), None, residual=d_h1)
-    gpu = {n: dev.download(getattr(layer, n)) for n in names}
+    gpu = snapshot()
     gpu["q"] = gpu["q"].reshape(B, Hq, D)
     x_in = prev_dn + prev_h1
     assert np.array_equal(dev.download(layer.h0), x_in)
