@@ -224,6 +224,29 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
         for (int i = 0; i < TM; ++i) acc[j][i] = (v4i){0, 0, 0, 0};
     v4i xb0[TM], xb1[TM], wa[R];
 
+    // The scales of the epilogue are requested before the first stage: a load issued between the stores would wait
+    // for every store before it (the memory counter is shared and counts in order), and one issued after the loop
+    // would put a memory round trip between the last MFMA and the first store.  28 registers for the whole loop.
+    const bool lo = r < 8;
+    float sxA[TM], sxB[TM], sxO[TM];
+    float4 swP[(TN + 1) / 2];
+    if constexpr (DEQ) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mrow = m0 + (wm * TM + i) * 16;
+            const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7), mO = mrow + r;
+            sxA[i] = sx[mA < M ? mA : M - 1];
+            sxB[i] = sx[mB < M ? mB : M - 1];
+            if constexpr (TN & 1) sxO[i] = sx[mO < M ? mO : M - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j += 2) {
+            int n = n0 + (wn * TN + j) * 16 + ((!lo && j + 1 < TN) ? 16 : 0) + 4 * g_;
+            if (n > N - 4) n = N - 4;
+            swP[j / 2] = *reinterpret_cast<const float4 *>(sw + n);
+        }
+    }
+
     const int nk = K >> 7;
     // stage s lives in activation buffer s % 2 and weight buffer s % NWB; the offsets rotate with the stage
     unsigned xcur = 0, xnxt = XSTAGE;
@@ -321,29 +344,8 @@ __global__ __launch_bounds__(256) void k_w8a8_tiled(const int8_t *__restrict__ q
     // drain the trailing fragment reads; 2 x 16 wait states cover the longest MFMA-result -> VALU-read hazard
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
 
-    // epilogue: lane holds channels nb + 4*g_ .. +3 of token mrow + r for each (i, j).  Every scale is
-    // fetched before the first store: the memory counter is shared by loads and stores and counts in
-    // order, so a load issued between stores would wait for all stores before it
-    const bool lo = r < 8;
-    float sxA[TM], sxB[TM], sxO[TM];
-    float4 swP[(TN + 1) / 2];
-    if constexpr (DEQ) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int mrow = m0 + (wm * TM + i) * 16;
-            const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7), mO = mrow + r;
-            sxA[i] = sx[mA < M ? mA : M - 1];
-            sxB[i] = sx[mB < M ? mB : M - 1];
-            if constexpr (TN & 1) sxO[i] = sx[mO < M ? mO : M - 1];
-        }
-#pragma unroll
-        for (int j = 0; j < TN; j += 2) {
-            int n = n0 + (wn * TN + j) * 16 + ((!lo && j + 1 < TN) ? 16 : 0) + 4 * g_;
-            if (n > N - 4) n = N - 4;
-            swP[j / 2] = *reinterpret_cast<const float4 *>(sw + n);
-        }
-    }
-    // interior tiles take a branch-free path: with divergent branches between the stores the compiler
+    // epilogue: lane holds channels nb + 4*g_ .. +3 of token mrow + r for each (i, j); interior tiles take a
+    // branch-free path: with divergent branches between the stores the compiler
     // can no longer count how many are in flight and falls back to waiting for each one
     auto emit = [&](auto CHECKED) {
         constexpr bool checked = decltype(CHECKED)::value;
