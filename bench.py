@@ -175,11 +175,20 @@ def main():
         counters[(K, N)] = (counters[(K, N)] + 1) % len(bufs)
         return bufs[counters[(K, N)]]
 
+    # One cfg3 step = the four projections of a decoder layer's prefill.  gate and up read the same activation
+    # matrix (as they do in the layer), so its rotate + quantize prologue runs once and both contractions take the
+    # codes; qkv and down each quantize their own input.  Three prologues and four GEMM launches per step.
+    qx_ws = {K: (dev.empty((M, K), np.int8), dev.empty(M, np.float32)) for K in (4096, 14336)}
+
     def prefill_step():
+        last_quantized = None
         for name, K, N in wl.PROJECTIONS:
             qw, sw = next_w(K, N)
-            mi.check(lib.mi_w8a8_linear_f32(acts[K].ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, wl.HADAMARD_BLOCK,
-                                            lin_ws.ptr, lin_ws.nbytes, s))
+            cx, cs = qx_ws[K]
+            if not (name == "up" and last_quantized == "gate"):
+                mi.fwht_quant(acts[K], cx, cs, wl.HADAMARD_BLOCK, stream=s)
+            last_quantized = name
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(cx.ptr, cs.ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, s))
 
     log("headline: prefill step x%d (+%d warm-up)" % (args.steps, args.warmup))
     timer.settle(prefill_step)
@@ -190,15 +199,16 @@ def main():
     ms_eager = timer.run(prefill_step, args.steps)
     dev.sync(s)
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    # the same K steps recorded once into a graph (the weight rotation is baked in) and replayed as one launch:
-    # exactly K steps inside the timed region, no host work between kernels
+    # The declared method: the same K steps recorded once into a graph (the weight rotation is baked in) and
+    # replayed as one launch, exactly K steps inside the timed region and no host work between kernels.  The eager
+    # figure is reported beside it and never picked.
     with mi.Graph.capture(s) as g:
         for _ in range(args.steps):
             prefill_step()
     timer.settle(lambda: g.launch())
     ms_graph = timer.run(lambda: g.launch(), 1) / args.steps
     g.destroy()
-    ms_step = min(ms_eager, ms_graph)
+    ms_step = ms_graph
     step_ops = sum(wl.gemm_ops(M, N, K) for _, K, N in wl.PROJECTIONS)
     value = step_ops / (ms_step * 1e-3) / 1e12
 
@@ -221,7 +231,7 @@ def main():
     gemm_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
     # HBM-side bytes per launch of the tiled GEMM, measured with hardware counters in a separate run
     traffic, traffic_total = None, None
-    tpath = os.path.join(os.path.dirname(os.path.abspath(mi.__file__)), "hbm_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as fh:
             per = json.load(fh)["tiled_gemm_bytes_per_launch"]
@@ -232,6 +242,8 @@ def main():
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_total,
         "traffic_unit": "bytes over the four launches (fetched + written), rocprofv3 PMC, calibrated",
+        "traffic_source": "profiles/hbm_traffic_pmc.md (a separate rocprofv3 --pmc run of bench.py --pmc-probe, "
+                          "not this run)",
         "traffic_per_shape": traffic,
         "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
         "per_shape_us_median": {k: round(v[len(v) // 2] * 1e3, 2) for k, v in gemm_samples.items()},
@@ -247,10 +259,13 @@ def main():
         "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "cfg3 prefill: 4 rotated W8A8 linears (4096->6144, 4096->14336 x2, 14336->4096) "
-                               "at M=2048, Hadamard block 128, rotate+quant prologue included; the K steps are recorded into one "
-                               "HIP graph and replayed (eager launches from Python also reported); about 60 ms of the same "
-                               "steps run untimed before the W warm-up steps so that timing starts at the sustained clock",
+        "config": {"workload": "cfg3 prefill: the 4 rotated W8A8 projections of a layer (4096->6144, 4096->14336 x2, "
+                               "14336->4096) at M=2048, Hadamard block 128, rotate+quant prologues included; gate and up share "
+                               "one input, which is rotated and quantized once (3 prologues + 4 GEMMs per step); all four "
+                               "write one 117 MB output buffer (it stays in the memory-side cache; weights rotate through "
+                               ">256 MB of copies); the K steps are recorded into one HIP graph and replayed - the timed "
+                               "method; eager launches from Python are reported beside it; about 60 ms of the same steps "
+                               "run untimed before the W warm-up steps so that timing starts at the sustained clock",
                    "tokens": M, "ops_per_step": step_ops, "tokens_per_s": round(M / (ms_step * 1e-3), 1),
                    "wall_ms_per_step": round(wall_ms, 4),
                    "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph": round(ms_graph, 4)},
@@ -581,46 +596,159 @@ def host_staging(mi, wl, dev, s, timer):
                                       "d2h_us": round(ms_out * 1e3, 1), "d2h_GBps": round(nout / (ms_out * 1e-3) / 1e9, 1)}}
 
 
+def node_cpu_lists():
+    """{node: [cpus]} from /sys/devices/system/node/node*/cpulist, the files the upstream NumaInfo parses
+    (numa/numa.mojo:107-115), restricted to the CPUs this process may run on."""
+    allowed = os.sched_getaffinity(0)
+    nodes = {}
+    base = "/sys/devices/system/node"
+    try:
+        names = sorted(n for n in os.listdir(base) if n.startswith("node") and n[4:].isdigit())
+    except OSError:
+        names = []
+    for n in names:
+        try:
+            txt = open(os.path.join(base, n, "cpulist")).read().strip()
+        except OSError:
+            continue
+        cpus = []
+        for part in filter(None, txt.split(",")):
+            lo, _, hi = part.partition("-")
+            cpus.extend(range(int(lo), int(hi or lo) + 1))
+        cpus = [c for c in cpus if c in allowed]
+        if cpus:
+            nodes[int(n[4:])] = cpus
+    if not nodes:
+        nodes[0] = sorted(allowed)
+    return nodes
+
+
 def cpu_baseline(wl):
-    """The CPU oracle (a builder-written port; upstream has no CPU kernels for this path) on the host cores, on the
-    headline workload itself: the four cfg3 linears at M = 2048 (rotate + quantize, int8 GEMM, dequant), repeated
-    until about 12 s of CPU work have been timed."""
+    """The CPU oracle (a builder-written port; upstream has no CPU kernels for this path) on the host cores, one
+    OpenMP thread per core, each pinned to a CPU of its NUMA node as the upstream pool pins its workers
+    (threading/linux_threading.mojo:89-91).  The headline workload (the four cfg3 linears at M = 2048: rotate +
+    quantize, int8 GEMM, dequant) runs for about 6 s; cfg0, cfg1, cfg2 and cfg4 follow on bounded samples (a few
+    calls each), about 20 s in all."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import ctypes as C
     import cpu_oracle as orc
+    nodes = node_cpu_lists()
+    nth = orc.num_threads()
+    # threads are dealt to the nodes in turn, inside a node to its CPUs in turn
+    order, depth = [], 0
+    while len(order) < nth:
+        took = False
+        for n in sorted(nodes):
+            if depth < len(nodes[n]) and len(order) < nth:
+                order.append(nodes[n][depth])
+                took = True
+        depth += 1
+        if not took:
+            depth = 0
+            if not any(nodes.values()):
+                break
+    pinned = orc.pin_threads(order) if order else 0
     M = wl.PREFILL_M
     g = np.random.default_rng(3)
+    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+    lib = orc.lib()
+
+    def linear_call(x, qw, sw, bufs):
+        Mx, K = x.shape
+        N = qw.shape[0]
+        y, qx, sx, acc = bufs
+        rc = lib.orc_w8a8_linear(ptr(x), ptr(qw), ptr(sw), ptr(y), C.c_int64(Mx), C.c_int64(N), C.c_int64(K),
+                                 C.c_int(128), ptr(qx), ptr(sx), ptr(acc))
+        assert rc == 0
+
+    def bufs_for(Mx, N, K):   # outputs allocated and touched once, as a resident caller's are
+        return (np.zeros((Mx, N), np.float32), np.zeros((Mx, K), np.int8), np.zeros(Mx, np.float32),
+                np.zeros((Mx, N), np.int32))
+
+    def timed(fn, budget_s, max_calls=10000):
+        fn()   # first touch
+        n, dt = 0, 0.0
+        while dt < budget_s and n < max_calls:
+            t0 = time.perf_counter()
+            fn()
+            dt += time.perf_counter() - t0
+            n += 1
+        return dt / n, n
+
     xs = {K: wl.activations(1, M, K, stream=K) for K in (4096, 14336)}
     ws = {}
     for name, K, N in wl.PROJECTIONS:
         if (K, N) not in ws:
-            ws[(K, N)] = (g.integers(-127, 128, (N, K)).astype(np.int8), np.full(N, 0.001, np.float32))
+            ws[(K, N)] = (g.integers(-127, 128, (N, K), dtype=np.int8), np.full(N, 0.001, np.float32))
     orc.rotate_quant_rows(xs[4096][:64], 128)          # load the library, spin up the OpenMP team
-    import ctypes as C
-    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
-    outs = {}                                          # outputs allocated and touched once, as a resident caller's are
-    for name, K, N in wl.PROJECTIONS:
-        if (K, N) not in outs:
-            outs[(K, N)] = (np.zeros((M, N), np.float32), np.zeros((M, K), np.int8), np.zeros(M, np.float32),
-                            np.zeros((M, N), np.int32))
-    ops, dt, passes = 0, 0.0, 0
-    while dt < 12.0 and passes < 400:
+    outs = {(K, N): bufs_for(M, N, K) for _, K, N in wl.PROJECTIONS}
+
+    def cfg3_step():
         for name, K, N in wl.PROJECTIONS:
-            qw, sw = ws[(K, N)]
-            y, qx, sx, acc = outs[(K, N)]
-            t0 = time.perf_counter()
-            rc = orc.lib().orc_w8a8_linear(ptr(xs[K]), ptr(qw), ptr(sw), ptr(y), C.c_int64(M), C.c_int64(N),
-                                           C.c_int64(K), C.c_int(128), ptr(qx), ptr(sx), ptr(acc))
-            dt += time.perf_counter() - t0
-            assert rc == 0
-            ops += wl.gemm_ops(M, N, K)
-        passes += 1
+            linear_call(xs[K], ws[(K, N)][0], ws[(K, N)][1], outs[(K, N)])
+    per_step, passes = timed(cfg3_step, 6.0, 400)
+    step_ops = sum(wl.gemm_ops(M, N, K) for _, K, N in wl.PROJECTIONS)
+    per = {}
+    # cfg1: decode GEMV sweep (rotate + quantize + contraction + dequant per call; bytes = the GPU leg's)
+    cfg1 = {}
+    for Mx in wl.DECODE_BATCHES:
+        row = {}
+        for name, K, N in wl.PROJECTIONS:
+            x = np.ascontiguousarray(xs[K][:Mx])
+            b = bufs_for(Mx, N, K)
+            sec, n = timed(lambda: linear_call(x, ws[(K, N)][0], ws[(K, N)][1], b), 0.25, 50)
+            row[name] = {"us": round(sec * 1e6, 1), "GBps": round(wl.linear_algorithmic_bytes(Mx, N, K) / sec / 1e9, 1)}
+        cfg1["M%d" % Mx] = row
+    per["cfg1_decode_gemv"] = cfg1
+    outs = None
+    # cfg0: the single rotated linear at M = 32
+    K0 = N0 = 4096
+    x0, b0 = np.ascontiguousarray(xs[4096][:32]), bufs_for(32, N0, K0)
+    w0 = (g.integers(-127, 128, (N0, K0), dtype=np.int8), np.full(N0, 0.001, np.float32))
+    sec, n = timed(lambda: linear_call(x0, w0[0], w0[1], b0), 1.0, 200)
+    per["cfg0_linear_m32"] = {"us": round(sec * 1e6, 1),
+                              "GBps": round(wl.linear_algorithmic_bytes(32, N0, K0) / sec / 1e9, 1),
+                              "TOPS": round(wl.gemm_ops(32, N0, K0) / sec / 1e12, 3)}
+    # cfg2: decode attention over an int8 cache (codes straight from the generator: the time does not depend on them)
+    c = wl.ATTN
+    B, Hq, Hkv, D, T = c["B"], c["Hq"], c["Hkv"], c["D"], c["T"]
+    kq = g.integers(-127, 128, (B, Hkv, T, D), dtype=np.int8)
+    vq = g.integers(-127, 128, (B, Hkv, T, D), dtype=np.int8)
+    ks = np.full((B, Hkv, T), 0.03, np.float32)
+    q = wl.normal(88, (B, Hq, D), 1)
+    sec, n = timed(lambda: orc.gqa_decode(q, kq, ks, vq, ks), 1.5, 50)
+    nbytes = wl.attention_algorithmic_bytes(B, Hq, Hkv, D, T)
+    per["cfg2_decode_attention"] = {"us": round(sec * 1e6, 1), "GBps": round(nbytes / sec / 1e9, 1),
+                                    "tokens_per_s": round(B / sec, 1)}
+    kq = vq = None
+    # cfg4: the MoE layer (router + dispatch + grouped expert FFN)
+    mc = wl.MOE
+    Tm, H, E, topk, I = mc["T"], mc["H"], mc["E"], mc["topk"], mc["I"]
+    xm = wl.activations(5, Tm, H)
+    wr = (0.02 * g.standard_normal((E, H))).astype(np.float32)
+    wg, wu = g.integers(-127, 128, (E, I, H), dtype=np.int8), g.integers(-127, 128, (E, I, H), dtype=np.int8)
+    wd = g.integers(-127, 128, (E, H, I), dtype=np.int8)
+    sg, sd = np.full((E, I), 0.001, np.float32), np.full((E, H), 0.001, np.float32)
+
+    def moe_call():
+        idx, w = orc.moe_route(xm, wr, topk)
+        orc.moe_ffn(xm, idx, w, wg, sg, wu, sg, wd, sd, 128, 256)
+    sec, n = timed(moe_call, 2.0, 20)
+    wbytes = wl.moe_weight_bytes(E, H, I)
+    per["cfg4_moe_layer"] = {"us": round(sec * 1e6, 1), "GBps": round(wbytes / sec / 1e9, 1),
+                             "TOPS": round(wl.moe_ops(Tm, topk, H, I) / sec / 1e12, 3),
+                             "tokens_per_s": round(Tm / sec, 1)}
     topo = host_topology()
-    return {"value": round(ops / dt / 1e12, 4), "unit": "TOPS", "cores": orc.num_threads(), "kind": "port",
-            "numa_nodes": topo["numa_nodes"],
+    return {"value": round(step_ops / per_step / 1e12, 4), "unit": "TOPS", "cores": nth, "kind": "port",
+            "numa_nodes": topo["numa_nodes"], "threads_pinned": pinned,
+            "pinning": "one OpenMP thread per core, dealt to the NUMA nodes in turn and pinned to a CPU of its node "
+                       "(node CPU lists from /sys/devices/system/node/node*/cpulist)",
             "sample": "the cfg3 step (four rotated W8A8 linears at M=2048: rotate+quant, int8 GEMM, dequant) x %d, "
-                      "%.1f s, OpenMP C, int8 GEMM %s" % (
-                          passes, dt, "blocked AVX-512 VNNI (4x6 register tiles)" if orc.lib().orc_gemm_uses_vnni()
-                          else "auto-vectorized dot products")}
+                      "%.1f s, OpenMP C, int8 GEMM %s; per_config: a few calls of each other config (0.25 - 2 s each)" % (
+                          passes, per_step * passes,
+                          "blocked AVX-512 VNNI (4x6 register tiles)" if lib.orc_gemm_uses_vnni()
+                          else "auto-vectorized dot products"),
+            "per_config": per}
 
 
 if __name__ == "__main__":

@@ -151,7 +151,11 @@ MI_API int32_t mi_event_elapsed_ms(mi_event *start, mi_event *stop, float *ms);
  * all-zero row gives scale 1 and codes 0.  The same call prepares activations
  * (per token), weights [N,K] (per output channel) and KV-cache rows
  * [B*Hkv*T, D] (per token-head, block = D).  K % block == 0, K <= 32768.
- * Codes and scales are bit-exact against the CPU restatement. */
+ * Codes and scales are bit-exact against the CPU restatement.
+ * Rows are meant to be finite (the rotation spreads one non-finite input over its whole block).  What the
+ * quantizer does with a non-finite rotated value is fixed all the same, by IEEE max / min semantics: a NaN takes no
+ * part in the absmax and gets the code -127; a row holding +-Inf gets scale Inf, code 0 for its finite values and
+ * -127 for the infinite ones. */
 MI_API int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale,
                                     int64_t M, int64_t K, int32_t block, void *stream);
 /* a1 alone: out fp32 [M,K] = rotated rows (out may alias x). */

@@ -238,3 +238,9 @@ def swiglu(gate_up):
 
 def num_threads():
     return int(lib().orc_num_threads())
+
+
+def pin_threads(cpus):
+    """thread t of the OpenMP team -> cpus[t]; returns how many threads were pinned"""
+    a = np.ascontiguousarray(cpus, dtype=np.int32)
+    return int(lib().orc_pin_threads(_p(a), C.c_int(a.size)))

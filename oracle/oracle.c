@@ -71,8 +71,18 @@
  *      token are quantized as one row by D2 with no further rotation, and the
  *      projection weights are rotated along K with block D as for any linear
  *      ((x.H) . (W.H)^T = x . W^T for the orthonormal H).
+ *  D14 Rows are meant to be finite; what a non-finite element does is fixed
+ *      all the same, by IEEE fmax / fmin (a NaN operand is ignored): a NaN
+ *      takes no part in the absmax and gets the code -127 (its product with
+ *      inv is NaN, which max(.., -127) turns into -127); a row holding +-Inf
+ *      has a = Inf, scale Inf and inv 0, so its finite elements get code 0
+ *      and the infinite ones -127; a row of NaNs and zeros only has a = 0,
+ *      scale 1, inv 0: zeros give 0, NaNs -127.  Nothing is undefined and
+ *      the GPU does the same.
  */
+#define _GNU_SOURCE   /* sched_setaffinity, cpu_set_t */
 #include <math.h>
+#include <sched.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -119,17 +129,11 @@ ORC_API void orc_quant_row(const float *xr, int64_t K, int8_t *q, float *scale)
         float v = fabsf(xr[k]);
         if (v > a) a = v;
     }
-    if (a == 0.0f) {
-        *scale = 1.0f;
-        memset(q, 0, (size_t)K);
-        return;
-    }
-    *scale = a / 127.0f;
-    const float inv = 127.0f / a;
+    *scale = (a == 0.0f) ? 1.0f : a / 127.0f;
+    const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
     for (int64_t k = 0; k < K; ++k) {
-        float r = rintf(xr[k] * inv);
-        if (r > 127.0f) r = 127.0f;
-        if (r < -127.0f) r = -127.0f;
+        /* fmaxf / fminf return the other operand when one is NaN (C11 F.10.9.2): never a cast of NaN (D14) */
+        const float r = fminf(fmaxf(rintf(xr[k] * inv), -127.0f), 127.0f);
         q[k] = (int8_t)r;
     }
 }
@@ -599,6 +603,32 @@ ORC_API int orc_swiglu(const float *gate_up, float *h, int64_t M, int64_t I)
             h[m * I + n] = (g / (1.0f + expf(-g))) * u;
         }
     return 0;
+}
+
+/* Pins OpenMP thread t of the team to cpu_of_thread[t] (t < n), the way the upstream pool pins its workers to
+ * the CPUs of one NUMA node (threading/linux_threading.mojo:89-91, :130-158).  Used by the benchmark's CPU leg
+ * only; the caller reads the nodes' CPU lists from sysfs as upstream does (numa/numa.mojo:107-115).
+ * Returns the number of threads that were pinned. */
+ORC_API int orc_pin_threads(const int32_t *cpu_of_thread, int n)
+{
+    int pinned = 0;
+#ifdef _OPENMP
+#pragma omp parallel reduction(+ : pinned)
+    {
+        extern int omp_get_thread_num(void);
+        const int t = omp_get_thread_num();
+        if (t < n) {
+            cpu_set_t set;
+            CPU_ZERO(&set);
+            CPU_SET(cpu_of_thread[t], &set);
+            if (sched_setaffinity(0, sizeof(set), &set) == 0) pinned = 1;
+        }
+    }
+#else
+    (void)cpu_of_thread;
+    (void)n;
+#endif
+    return pinned;
 }
 
 ORC_API int orc_num_threads(void)

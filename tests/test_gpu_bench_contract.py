@@ -28,8 +28,36 @@ def test_bench_line_fields():
     assert r["bound"] == "mfma" and r["unit"] == "TOP/s" and r["peak"] == 5000.0
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
     assert 0.05 < r["frac"] < 1.0 and b["value"] > 100.0
-    # value is ops per step over the step time
+    # value is ops per step over the step time, and the step time is the declared method's (graph replay)
     assert abs(b["value"] - b["config"]["ops_per_step"] / (b["ms_per_step"] * 1e-3) / 1e12) < 0.01 * b["value"]
+    assert b["ms_per_step"] == b["config"]["ms_per_step_graph"] and "ms_per_step_eager" in b["config"]
+    # the HBM traffic figure says where it comes from: a separate counter run, not this one
+    assert r["traffic"] is None or "profiles/" in r["traffic_source"]
+
+
+def test_cpu_baseline_leg_pins_its_threads_per_numa_node():
+    """The CPU leg without a GPU: node CPU lists come from sysfs and lie inside the process's affinity mask, every
+    OpenMP thread gets pinned, and the record carries a figure for every config."""
+    sys.path.insert(0, ROOT)
+    sys.path.insert(0, os.path.join(ROOT, "mojo-linuxperiments_amd"))
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import bench
+    import cpu_oracle as orc
+    nodes = bench.node_cpu_lists()
+    allowed = os.sched_getaffinity(0)
+    assert nodes and all(cpus and set(cpus) <= allowed for cpus in nodes.values())
+    assert sum(len(c) for c in nodes.values()) <= len(allowed)
+    first = sorted(nodes)[0]
+    try:
+        assert orc.pin_threads(nodes[first][:1] * orc.num_threads()) == orc.num_threads()
+    finally:
+        # give the team its CPUs back for the tests that follow
+        every = sorted(allowed)
+        orc.pin_threads([every[i % len(every)] for i in range(orc.num_threads())])
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    for key in ("cfg0_linear_m32", "cfg1_decode_gemv", "cfg2_decode_attention", "cfg4_moe_layer", "per_config",
+                "threads_pinned"):
+        assert '"%s"' % key in src[src.index("def cpu_baseline"):], key
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -63,6 +63,26 @@ def test_zero_rows_ties_and_extremes(mi, dev, orc):
     assert np.array_equal(s, so) and np.array_equal(q, qo)
 
 
+@pytest.mark.parametrize("M,K,block", [(9, 512, 128), (1030, 256, 128), (40, 128, 128), (5, 768, 256)])
+def test_non_finite_rows_follow_the_oracle(mi, dev, orc, M, K, block):
+    """NaN and +-Inf inputs (which the rotation spreads over their block) quantize the same way on both sides, in
+    each of the three kernels (a workgroup per row, a wave per row, 16 lanes per row): nothing is undefined."""
+    x = workload.activations(6, M, K)
+    x[1, 3] = np.nan
+    x[2, K - 1] = np.inf
+    x[3, 0], x[3, block // 2] = np.inf, -np.inf
+    x[4] = np.nan
+    x[M - 1, K // 2] = -np.inf
+    with np.errstate(invalid="ignore"):
+        q, s = run_quant(mi, dev, x, block)
+        qo, so = orc.rotate_quant_rows(x, block)
+    assert np.array_equal(q, qo)
+    assert np.array_equal(s, so, equal_nan=True)
+    assert s[4] == 1.0 and np.all(q[4] == -127)           # a row of NaNs: absmax 0, every product NaN
+    assert np.all(q[1, :block] == -127)                    # the NaN's block
+    assert np.array_equal(q[0], orc.rotate_quant_rows(x[:1], block)[0][0])
+
+
 @pytest.mark.parametrize("M,K,block", [(7, 4096, 128), (3, 768, 256), (33, 128, 128), (1027, 512, 256)])
 def test_rotation_only_bit_exact_and_in_place(mi, dev, orc, M, K, block):
     x = workload.normal(3, (M, K))

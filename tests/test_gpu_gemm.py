@@ -95,7 +95,7 @@ def test_whole_linear(mi, dev, orc, M, N, K):
 
 
 @pytest.mark.parametrize("name,K,N", workload.PROJECTIONS)
-@pytest.mark.parametrize("M", [16, 2048])
+@pytest.mark.parametrize("M", [1, 4, 16, 2048])
 def test_full_size_projections(mi, dev, orc, name, K, N, M):
     """cfg1 / cfg3 shapes: sampled rows against the oracle plus a linearity
     checksum over every row: sum_n acc[m,n] == qx[m,:] . (sum_n qw[n,:])."""
@@ -107,6 +107,35 @@ def test_full_size_projections(mi, dev, orc, name, K, N, M):
     assert np.array_equal(acc.astype(np.int64).sum(axis=0), qw.astype(np.int64) @ rowsum)
     rows = sorted(set([0, M - 1] + list(np.random.default_rng(M).integers(0, M, 6))))
     assert np.array_equal(acc[rows], orc.gemm_i8_i32(qx[rows], qw))
+
+
+@pytest.mark.parametrize("name,K,N", [workload.PROJECTIONS[0], workload.PROJECTIONS[3]])
+def test_whole_prefill_linear_end_to_end(mi, dev, orc, name, K, N):
+    """cfg3, one projection per K: the whole mi_w8a8_linear_f32 at M = 2048 (rotate + quantize, tiled GEMM, dequant)
+    against the oracle's linear on sampled rows (the oracle quantizes a row on its own, so a row of y depends on
+    that row of x alone), and the activation codes of every row."""
+    M = workload.PREFILL_M
+    x = workload.activations(21, M, K)
+    w = workload.weights(22, N, K)
+    mark = dev.mark()
+    dqw, dsw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+    keep = dev.mark()
+    mi.fwht_quant(dev.upload(w), dqw, dsw, 128)
+    dev.sync()
+    dev.reset_to(keep)
+    ws = dev.empty(mi.lib.mi_w8a8_linear_workspace_bytes(M, N, K), np.uint8)
+    dy = dev.empty((M, N), np.float32)
+    mi.linear(dev.upload(x), dqw, dsw, dy, 128, ws)
+    y = dev.download(dy)
+    qx = dev.download(ws.offset(0, (M, K), np.int8))
+    qw, sw = dev.download(dqw), dev.download(dsw)
+    dev.reset_to(mark)
+    assert np.array_equal(qx, orc.rotate_quant_rows(x, 128)[0])
+    rows = sorted(set([0, 255, 256, M - 1] + list(np.random.default_rng(K).integers(0, M, 8))))
+    yo = orc.w8a8_linear(x[rows], qw, sw, 128)[0]
+    assert np.linalg.norm(y[rows].astype(np.float64) - yo) <= 1e-3 * np.linalg.norm(yo.astype(np.float64))
+    assert np.array_equal(y[rows], yo)
+    assert np.all(np.isfinite(y))
 
 
 def test_argument_errors(mi, dev):

@@ -142,3 +142,17 @@ def test_rotate_quant_rows_is_composition(orc):
     q2, s2 = orc.rotate_quant_rows(x2, 256)
     assert np.array_equal(np.delete(q2, 3, 0), np.delete(q, 3, 0))
     assert s2[3] == s[3] * 8 and np.array_equal(q2[3], q[3])
+
+
+def test_quant_non_finite_values_are_defined(orc):
+    """D14: a NaN takes no part in the absmax and gets -127; +-Inf makes the scale Inf, finite values 0 and the
+    infinite ones -127; NaNs among zeros only: scale 1."""
+    row = np.array([1.0, -2.0, np.nan, 0.5], np.float32)
+    q, s = orc.quant_row(row)
+    assert s == np.float32(2.0) / np.float32(127.0) and list(q) == [64, -127, -127, 32]
+    row = np.array([1.0, np.inf, -np.inf, -3.0, 0.0], np.float32)
+    q, s = orc.quant_row(row)
+    assert np.isinf(s) and s > 0 and list(q) == [0, -127, -127, 0, 0]
+    row = np.array([0.0, np.nan, -0.0], np.float32)
+    q, s = orc.quant_row(row)
+    assert s == 1.0 and list(q) == [0, -127, 0]
