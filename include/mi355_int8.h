@@ -93,6 +93,9 @@ MI_API int32_t mi_host_arena_create(mi_ctx *ctx, int64_t size_bytes, int64_t ali
  * begin never blocks and reports a full pool as MI_EBUSY, as launch returns
  * False (linux_threading.mojo:103-121). */
 typedef struct mi_stream_pool mi_stream_pool;
+/* capacity <= 1024.  A process has four hardware queues on this part (HIP's default): the first three slots run
+ * beside each other and beside the null stream; a fourth and later slot shares a queue with an earlier one and
+ * its work waits behind that slot's. */
 MI_API int32_t mi_stream_pool_create(mi_ctx *ctx, int32_t capacity, mi_stream_pool **out); /* linux_threading.mojo:56-66, :130-158 */
 MI_API int32_t mi_stream_pool_destroy(mi_stream_pool *p);      /* linux_threading.mojo:70-77: MI_EBUSY (pool kept) instead of abort() when work is in flight */
 MI_API int32_t mi_stream_pool_capacity(const mi_stream_pool *p);         /* linux_threading.mojo:85-86 */

@@ -4,17 +4,21 @@
 // Bound: HBM.  Algorithmic bytes per call = N*K (weights) + M*K (codes)
 // + 4*M*N (output) + 4*(M+N) (scales).
 //
-// Two kernels, chosen by M:
+// Kernels, chosen by M and K (launch_skinny):
 //
-//  k_gemv_dot4 (M <= 4).  One workgroup per compute unit owns a contiguous span
-//  of weight rows; the activation codes (M*K bytes) sit in LDS.  A wave streams
-//  one weight row at a time with 128-bit loads, 1 KB contiguous per wave
-//  instruction (eight whole 128-byte lines), double buffered in registers, and
-//  each lane feeds its 16 bytes to v_dot4_i32_i8 against the matching 16 bytes
-//  of every token.  The 64 partial int32 sums of a row meet in a DPP / swizzle
-//  wave reduction.  Exact: integer sums are order independent.
+//  k_gemv_reg (M = 1, and M <= 4 on K < 8192).  A lane always works on the same byte offsets of a weight row, so
+//  its share of the activation codes lives in registers for the whole kernel: no LDS and no barrier in the
+//  streaming part, 16 x 1 KB weight loads in flight per wave, v_dot4_i32_i8, one transposed butterfly per wave.
+//  k_gemv_fused is the same kernel with the rotate + quantize prologue (and optionally the RMSNorm) inside, for
+//  one token and K <= 4096.
 //
-//  k_skinny_ring (4 < M <= 64).  v_mfma_i32_16x16x64_i8 wants 16 rows x 64
+//  k_gemv_dot4 (M <= 4, K that the register kernel cannot split evenly).  One workgroup per compute unit owns a
+//  contiguous span of weight rows; the activation codes (M*K bytes) sit in LDS.  A wave streams one weight row
+//  at a time with 128-bit loads, 1 KB contiguous per wave instruction, double buffered in registers, and each
+//  lane feeds its 16 bytes to v_dot4_i32_i8 against the matching 16 bytes of every token.  The 64 partial int32
+//  sums of a row meet in a DPP / swizzle wave reduction.  Exact: integer sums are order independent.
+//
+//  k_skinny_ring (4 < M <= 64, and M = 2..4 on K >= 8192).  v_mfma_i32_16x16x64_i8 wants 16 rows x 64
 //  bytes per operand, but a load shaped like that touches 16 different lines
 //  per quarter wave and runs at a third of the bandwidth of a load that takes
 //  8 rows x 128 bytes.  So every wave owns a private ring of LDS stages, fills

@@ -204,17 +204,22 @@ struct DecodeAttention {
 // An int8 KV cache of fixed capacity held in an arena: the decode loop appends one token per sequence at its own
 // position and attends over what each sequence holds.  Positions and lengths are int32 [B] arrays in device memory
 // (the loop that produces them runs on the device side of the stream, not on the host).
+// tiled: the codes live in the layouts the int8 matrix instruction loads straight from memory (keys in 16-token
+// tiles, values in transposed 64-token blocks; capacity a multiple of 64 tokens): the fast attention path.
+// Otherwise both halves are row-major [B, Hkv, T_cap, 128].  Same arithmetic, same codes, same scales.
 struct KvCache {
     int64_t B = 0, Hq = 0, Hkv = 0, D = 128, T_cap = 0;
+    bool tiled = false;
     int8_t *kq = nullptr, *vq = nullptr;
     float *ks = nullptr, *vs = nullptr;
     void *workspace = nullptr;
     int64_t workspace_bytes = 0;
 
     template <typename Arena>
-    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t_cap)
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t_cap, bool use_tiled_layouts)
     {
-        B = b; Hq = hq; Hkv = hkv; T_cap = t_cap;
+        B = b; Hq = hq; Hkv = hkv; T_cap = t_cap; tiled = use_tiled_layouts;
+        if (tiled && T_cap % 64) return false;
         workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap);
         if (workspace_bytes <= 0) return false;
         kq = arena.template alloc<int8_t>(B * Hkv * T_cap * D);
@@ -224,17 +229,52 @@ struct KvCache {
         workspace = arena.template alloc<uint8_t>(workspace_bytes);
         return kq && vq && ks && vs && workspace;
     }
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t_cap)
+    {
+        return prepare(arena, b, hq, hkv, t_cap, t_cap % 64 == 0);
+    }
     explicit operator bool() const { return workspace != nullptr; }
     // k_new / v_new: head h of sequence b at + b*row_stride + h*128 floats (slices of a fused QKV row are fine)
     int32_t append(const float *k_new, const float *v_new, int64_t row_stride, const int32_t *pos, void *stream) const
     {
-        return mi_kv_append_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, pos, B, Hkv, D, T_cap, stream);
+        return tiled ? mi_kv_append_tiled_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, pos, B, Hkv, D, T_cap, stream)
+                     : mi_kv_append_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, pos, B, Hkv, D, T_cap, stream);
     }
-    // t_max bounds every entry of seq_len (<= T_cap); a tighter bound launches fewer splits
+    // a fused QKV row per sequence: rotary embedding on query and key heads, queries out, keys and values appended
+    int32_t rope_append(const float *qkv, int64_t row_stride, const float *rope_cos, const float *rope_sin, float *q_out,
+                        const int32_t *pos, void *stream) const
+    {
+        return tiled ? mi_rope_kv_append_tiled_f32_i8(qkv, row_stride, rope_cos, rope_sin, q_out, kq, ks, vq, vs, pos, B, Hq,
+                                                      Hkv, D, T_cap, stream)
+                     : mi_rope_kv_append_f32_i8(qkv, row_stride, rope_cos, rope_sin, q_out, kq, ks, vq, vs, pos, B, Hq, Hkv, D,
+                                                T_cap, stream);
+    }
+    // t_max bounds every entry of seq_len (<= T_cap); the workspace serves every t_max up to the capacity
     int32_t attend(const float *q, float *o, const int32_t *seq_len, int64_t t_max, bool out_rotated, void *stream) const
     {
-        return mi_gqa_decode_attn_cache(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_cap, seq_len, t_max,
-                                        out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+        return tiled ? mi_gqa_decode_attn_tiled(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_cap, seq_len, t_max,
+                                                out_rotated ? 1 : 0, workspace, workspace_bytes, stream)
+                     : mi_gqa_decode_attn_cache(q, kq, ks, vq, vs, o, B, Hq, Hkv, D, T_cap, seq_len, t_max,
+                                                out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+    }
+    // the same with the merge fused with the output projection's row quantizer (rows stay in the rotated basis of V)
+    int32_t attend_quant(const float *q, float *o_rot, int8_t *oq, float *oscale, const int32_t *seq_len, int64_t t_max,
+                         void *stream) const
+    {
+        return tiled ? mi_gqa_decode_attn_tiled_quant_i8(q, kq, ks, vq, vs, o_rot, oq, oscale, B, Hq, Hkv, D, T_cap, seq_len,
+                                                         t_max, workspace, workspace_bytes, stream)
+                     : mi_gqa_decode_attn_cache_quant_i8(q, kq, ks, vq, vs, o_rot, oq, oscale, B, Hq, Hkv, D, T_cap, seq_len,
+                                                         t_max, workspace, workspace_bytes, stream);
+    }
+    // a cache quantized in one go (prefill): row-major codes [B*Hkv, T, 128] (rows src_stride tokens apart) into this
+    // cache's layout, first T tokens of every row; the scales are the caller's to copy into ks / vs
+    int32_t load_rows(const int8_t *kq_rows, const int8_t *vq_rows, int64_t T, int64_t src_stride, void *stream) const
+    {
+        if (tiled) return mi_kv_tiled_from_rows_i8(kq_rows, vq_rows, kq, vq, B * Hkv, T, src_stride, T_cap, stream);
+        if (src_stride != T_cap) return MI_EINVAL;
+        int32_t rc = mi_memcpy_d2d(kq, kq_rows, B * Hkv * T_cap * D, stream);
+        return rc == MI_OK ? mi_memcpy_d2d(vq, vq_rows, B * Hkv * T_cap * D, stream) : rc;
     }
 };
 
@@ -340,12 +380,8 @@ struct DecoderLayer {
         int32_t rc = mi_rmsnorm_linear_f32(x, residual, g1, eps, residual ? h0 : nullptr, xn, qkv.qw, qkv.sw, qkv_out, B,
                                            qkv.N, H, 128, qkv.workspace, qkv.workspace_bytes, stream);
         const float *xin = residual ? h0 : x;
-        if (rc == MI_OK)
-            rc = mi_rope_kv_append_f32_i8(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, cache.kq, cache.ks,
-                                          cache.vq, cache.vs, pos, B, Hq, Hkv, 128, T_cap, stream);
-        if (rc == MI_OK)
-            rc = mi_gqa_decode_attn_cache_quant_i8(q, cache.kq, cache.ks, cache.vq, cache.vs, att, ca, sa, B, Hq, Hkv, 128,
-                                                   T_cap, seq_len, t_max, cache.workspace, cache.workspace_bytes, stream);
+        if (rc == MI_OK) rc = cache.rope_append(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, pos, stream);
+        if (rc == MI_OK) rc = cache.attend_quant(q, att, ca, sa, seq_len, t_max, stream);
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
         if (rc == MI_OK)
             rc = mi_rmsnorm_linear_f32(ao, xin, g2, eps, h1, hn, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, 128,

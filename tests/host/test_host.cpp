@@ -223,9 +223,20 @@ static void test_decode_attention(const Context &ctx)
 
 // three decode steps through KvCache: append at per-sequence positions, attend over per-sequence lengths; the
 // cache rows follow the oracle quantizer bit for bit and the output follows the oracle on each sequence's prefix
-static void test_kv_cache(const Context &ctx)
+// key codes of a tiled cache [rows, T_cap/16, 8 chunks, 16 tokens, 16 bytes] back in token-major order
+static std::vector<int8_t> key_tiles_to_rows(const std::vector<int8_t> &kt, int64_t rows, int64_t T_cap)
 {
-    const int64_t B = 2, Hq = 8, Hkv = 2, D = 128, T_cap = 40;
+    std::vector<int8_t> out(kt.size());
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t t = 0; t < T_cap; ++t)
+            for (int64_t d = 0; d < 128; ++d)
+                out[(r * T_cap + t) * 128 + d] = kt[(r * T_cap + (t & ~15)) * 128 + (d >> 4) * 256 + (t & 15) * 16 + (d & 15)];
+    return out;
+}
+
+static void test_kv_cache(const Context &ctx, int64_t T_cap, const char *name)
+{
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 128;
     DeviceArena<256> arena(ctx, 64 << 20);
     KvCache cache;
     bool ok = cache.prepare(arena, B, Hq, Hkv, T_cap) && (bool)cache;
@@ -284,9 +295,10 @@ static void test_kv_cache(const Context &ctx)
         }
     }
     std::vector<int8_t> hkq = download(cache.kq, (size_t)(B * Hkv * T_cap * D));
+    if (cache.tiled) hkq = key_tiles_to_rows(hkq, B * Hkv, T_cap);
     std::vector<float> hvs = download(cache.vs, (size_t)(B * Hkv * T_cap));
-    ok = ok && hkq == rkq && hvs == rvs;
-    report("kv_cache_append_attend_vs_oracle", ok && err <= 2e-3f, "max-abs " + std::to_string(err));
+    ok = ok && hkq == rkq && hvs == rvs && cache.tiled == (T_cap % 64 == 0);
+    report(name, ok && err <= 2e-3f, "max-abs " + std::to_string(err));
 }
 
 // DecoderLayer::step against the oracle's operators chained in the same order, every stage fed what the device
@@ -472,7 +484,8 @@ int main()
     test_stream_pool(ctx);
     test_quant_linear(ctx);
     test_decode_attention(ctx);
-    test_kv_cache(ctx);
+    test_kv_cache(ctx, 40, "kv_cache_append_attend_vs_oracle");
+    test_kv_cache(ctx, 64, "kv_cache_tiled_layouts_append_attend_vs_oracle");
     test_decoder_layer(ctx);
     test_decoder_stack(ctx);
     std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");

@@ -63,3 +63,19 @@ def test_attention_workspace_bound_covers_every_shorter_length(mi):
                 need = lib.mi_gqa_decode_workspace_bytes(B, 4 * hkv, hkv, 128, t)
                 assert prev <= need <= cap, (rows, t_cap, t)
                 prev = need
+
+
+MOJO = os.path.join(ROOT, "mojo-linuxperiments_amd", "host", "mi355.mojo")
+
+
+def test_mojo_host_surface_binds_only_exported_symbols_and_all_of_them():
+    """host/mi355.mojo cannot be compiled here (no Mojo toolchain); what can be held to the library is its symbol
+    list: every name it looks up is exported, and it binds every entry point the header declares."""
+    text = open(MOJO).read()
+    names = set(re.findall(r'\("(mi_\w+)"\)', text))
+    assert len(names) >= 60
+    lib = ctypes.CDLL(LIB)
+    missing = sorted(n for n in names if not hasattr(lib, n))
+    assert not missing, missing
+    unbound = sorted(set(declared_symbols()) - names)
+    assert not unbound, unbound
