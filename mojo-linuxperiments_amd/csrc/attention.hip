@@ -26,7 +26,6 @@
 // Bound: HBM.  Algorithmic bytes = K and V codes (2*B*Hkv*T*D) + their scales
 // (8*B*Hkv*T) + q and o (8*B*Hq*D).
 #include "fwht_core.h"
-#include "attention_merge.h"
 
 namespace mi {
 
@@ -393,6 +392,79 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
     else gqa_split_body<DUMP, true, false, WAVE_TILES>(p, T, s_q, s_sq, s_red, s_sc, s_m, s_l, s_c);
 }
 
+// Merge of the splits of one (b, h) row by the 16 lanes that own it (lane j: elements 4j..4j+3 and 64+4j..).
+// SP > 0: the split count is known at compile time and every load of the row goes out before the first use (one
+// memory round trip).  Returns the normalized row in the rotated basis of V.
+template <int SP>
+__device__ __forceinline__ void merge_row(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                          int splits_rt, int64_t bkv, int hl, int j, float (&v)[8])
+{
+    const int splits = SP > 0 ? SP : splits_rt;
+    const float *ml0 = part_ml + bkv * splits * 8;
+    const float *po0 = part_o + (bkv * splits * 4 + hl) * attn::D;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    float l = 0.0f;
+    if constexpr (SP > 0) {
+        float ms[SP], ls[SP];
+        float4 lo[SP], hi[SP];
+#pragma unroll
+        for (int s = 0; s < SP; ++s) {
+            ms[s] = ml0[s * 8 + hl];
+            ls[s] = ml0[s * 8 + 4 + hl];
+            lo[s] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
+            hi[s] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
+        }
+        float mx = ms[0];
+#pragma unroll
+        for (int s = 1; s < SP; ++s) mx = fmaxf(mx, ms[s]);
+#pragma unroll
+        for (int s = 0; s < SP; ++s) {
+            const float w = (ms[s] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[s] - mx);   // empty split
+            l = __builtin_fmaf(ls[s], w, l);
+            v[0] = __builtin_fmaf(lo[s].x, w, v[0]); v[1] = __builtin_fmaf(lo[s].y, w, v[1]);
+            v[2] = __builtin_fmaf(lo[s].z, w, v[2]); v[3] = __builtin_fmaf(lo[s].w, w, v[3]);
+            v[4] = __builtin_fmaf(hi[s].x, w, v[4]); v[5] = __builtin_fmaf(hi[s].y, w, v[5]);
+            v[6] = __builtin_fmaf(hi[s].z, w, v[6]); v[7] = __builtin_fmaf(hi[s].w, w, v[7]);
+        }
+    } else {
+        // any split count: the maxima first (one round trip), then the partials in batches of eight whose loads all
+        // go out before the first use
+        float mx = -INFINITY;
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float ms[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ms[i] = ml0[min(s0 + i, splits - 1) * 8 + hl];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mx = fmaxf(mx, ms[i]);
+        }
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float ms[8], ls[8];
+            float4 lo[8], hi[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int s = min(s0 + i, splits - 1);
+                ms[i] = ml0[s * 8 + hl];
+                ls[i] = ml0[s * 8 + 4 + hl];
+                lo[i] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 4 * j);
+                hi[i] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float w = (s0 + i >= splits || ms[i] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[i] - mx);
+                l = __builtin_fmaf(ls[i], w, l);
+                v[0] = __builtin_fmaf(lo[i].x, w, v[0]); v[1] = __builtin_fmaf(lo[i].y, w, v[1]);
+                v[2] = __builtin_fmaf(lo[i].z, w, v[2]); v[3] = __builtin_fmaf(lo[i].w, w, v[3]);
+                v[4] = __builtin_fmaf(hi[i].x, w, v[4]); v[5] = __builtin_fmaf(hi[i].y, w, v[5]);
+                v[6] = __builtin_fmaf(hi[i].z, w, v[6]); v[7] = __builtin_fmaf(hi[i].w, w, v[7]);
+            }
+        }
+    }
+    const float rl = l > 0.0f ? 1.0f / l : 0.0f;   // a sequence of length 0 gives a row of zeros
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= rl;
+}
+
 // merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row
 template <int SP>
 __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ part_o,
@@ -406,7 +478,7 @@ __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ par
     const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
     const int64_t bkv = (int64_t)b * Hkv + kvh;
     float v[8];
-    merge_row<SP, false>(part_o, part_ml, splits_rt, bkv, hl, j, v);
+    merge_row<SP>(part_o, part_ml, splits_rt, bkv, hl, j, v);
     if (!out_rotated) fwht128(v, j);  // whole workgroup takes the same branch
     if (live) {
         float *orow = o + (int64_t)row * attn::D;
@@ -431,7 +503,7 @@ __global__ __launch_bounds__(1024) void k_gqa_merge_quant(const float *__restric
     const int b = blockIdx.x, h = tid >> 4;
     const int kvh = h / G, hl = h % G;
     float v[8];
-    merge_row<SP, false>(part_o, part_ml, splits_rt, (int64_t)b * Hkv + kvh, hl, j, v);
+    merge_row<SP>(part_o, part_ml, splits_rt, (int64_t)b * Hkv + kvh, hl, j, v);
     float a = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) a = fmaxf(a, fabsf(v[e]));
@@ -558,10 +630,7 @@ extern "C" int64_t mi_gqa_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t 
     int splits = attn::max_splits(B, Hkv, T);
     const int splits_vt = avt::max_splits(B, Hkv, T);   // one query serves both cache layouts
     if (splits_vt > splits) splits = splits_vt;
-    // partial outputs, partial (max, sum) pairs, and one fp32 row per query head for the kernels that merge and
-    // quantize a token's rows without a second launch
-    return attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256) + attn::align_up(B * Hkv * splits * 8 * 4, 256) +
-           attn::align_up(B * Hq * attn::D * 4, 256);
+    return attn::align_up(B * Hkv * splits * 4 * attn::D * 4, 256) + attn::align_up(B * Hkv * splits * 8 * 4, 256);
 }
 
 static int32_t run_attn(const float *q, const int8_t *kq, const float *ks, const int8_t *vq, const float *vs,

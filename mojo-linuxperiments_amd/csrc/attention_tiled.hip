@@ -27,11 +27,6 @@
 // The partial results have the layout the merge kernels of attention.hip take.
 //
 // Bound: HBM (the K and V codes, 2 * B * Hkv * T * 128 bytes, + 8 bytes of scales per token-head).
-#include <stdlib.h>
-
-#include <atomic>
-
-#include "attention_merge.h"
 #include "fwht_core.h"
 
 namespace mi {
@@ -62,14 +57,6 @@ struct Params {
     float score_scale;        // log2(e) / sqrt(D)
     float *o;                 // DIRECT kernels: the output rows [B, Hq, 128]
     int out_rotated;
-    int rows, splits;         // B * Hkv cache rows, workgroups per row
-    // FUSED kernels: the last workgroup of a row to finish merges the row's splits (and, with oq, the last row of a
-    // token quantizes the token's rows), so that no second kernel has to be launched
-    unsigned *row_ctr, *tok_ctr;   // arrival counters, zero between calls
-    int group;                     // consecutive rows that share an XCD: 1, or Hkv when tokens are quantized
-    float *rows_out;               // merged rows [B, Hq, 128]: o, o_rot or an area of the workspace
-    int8_t *oq;
-    float *oscale;
 };
 
 template <int MASK>
@@ -78,90 +65,10 @@ __device__ __forceinline__ float fmax_xor(float v)
     return fmaxf(v, xor_lane<MASK>(v));
 }
 
-// What a workgroup of a FUSED kernel does once its partial result is stored.  Ordering rests on three facts, none of
-// which needs a cache-wide operation: stores leave the vector L1 at once (it writes through) and are complete in
-// the XCD's L2 when the memory counter has run out; atomics execute in that L2; agent-scope atomic loads do not hit
-// in the vector L1.  All workgroups involved run on one XCD (see the kernel), so that L2 is the one they share.
-// The counters live in a static device array (zero when the library is loaded) and are put back to zero by the
-// workgroup that finds them full.
-template <int NW>
-__device__ __forceinline__ void fused_tail(const Params &p, int bkv, int b, int kvh)
-{
-    __shared__ int s_last[2];
-    __shared__ float s_amax[NW];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's part of the partial result is in L2
-    __syncthreads();
-    if (tid == 0) {
-        unsigned *c = p.row_ctr + bkv;
-        const unsigned old = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = old == (unsigned)(p.splits - 1);
-        if (last) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last[0] = last;
-    }
-    __syncthreads();
-    if (!s_last[0]) return;
-    // the row's last workgroup: merge the splits, 16 lanes per head row as the merge kernels do
-    if (tid < 64) {
-        const int hr = lane >> 4, jj = lane & 15;
-        if (hr < p.G) {
-            float v[8];
-            attn::merge_row<0, true>(p.part_o, p.part_ml, p.splits, bkv, hr, jj, v);
-            if (!p.oq && !p.out_rotated) fwht_chunk<D>(v, jj);
-            float *orow = p.rows_out + ((int64_t)b * p.Hq + kvh * p.G + hr) * D;
-            *reinterpret_cast<float4 *>(orow + 4 * jj) = make_float4(v[0], v[1], v[2], v[3]);
-            *reinterpret_cast<float4 *>(orow + 64 + 4 * jj) = make_float4(v[4], v[5], v[6], v[7]);
-        }
-    }
-    if (!p.oq) return;
-    // the token's last row: quantize the token's Hq * 128 values as one row for the output projection
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) {
-        unsigned *c = p.tok_ctr + b;
-        const unsigned old = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = old == (unsigned)(p.Hkv - 1);
-        if (last) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last[1] = last;
-    }
-    __syncthreads();
-    if (!s_last[1]) return;
-    const int n4 = p.Hq * (D / 4);               // float4 groups of the token's row, Hq <= 64: at most 8 per thread
-    const float *row = p.rows_out + (int64_t)b * p.Hq * D;
-    float4 val[8];
-    float a = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int g4 = tid + 64 * NW * i;
-        val[i] = g4 < n4 ? attn::ld4<true>(row + 4 * g4) : make_float4(0.f, 0.f, 0.f, 0.f);
-        a = fmaxf(fmaxf(a, fmaxf(fabsf(val[i].x), fabsf(val[i].y))), fmaxf(fabsf(val[i].z), fabsf(val[i].w)));
-    }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
-    if (lane == 0) s_amax[wave] = a;
-    __syncthreads();
-    a = s_amax[0];
-#pragma unroll
-    for (int w = 1; w < NW; ++w) a = fmaxf(a, s_amax[w]);
-    const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
-    const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
-    if (tid == 0) p.oscale[b] = sc;
-    int8_t *qrow = p.oq + (int64_t)b * p.Hq * D;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int g4 = tid + 64 * NW * i;
-        if (g4 < n4) *reinterpret_cast<uint32_t *>(qrow + 4 * g4) = quant4(val[i].x, val[i].y, val[i].z, val[i].w, inv);
-    }
-}
-
 // NW: waves per workgroup; NT: blocks per wave; RING: 1 KB loads a wave keeps in flight (8 or 16).
 // DIRECT: the workgroup covers the whole sequence (one split): it normalizes and writes the output rows itself and
 // no partial result leaves the chip.
-// FUSED: one-dimensional grid; workgroup id i runs on XCD i % 8 (the hardware deals workgroups to the XCDs in turn;
-// checked once per device before this mode is used), and all workgroups of a row - of a token's rows, when the
-// output is quantized per token - get ids that agree modulo 8.  They therefore share one L2, and the last of them
-// can read what the others wrote without any cache being written back or invalidated (fused_tail).
-template <int NW, int NT, int RING, bool DIRECT, bool FUSED>
+template <int NW, int NT, int RING, bool DIRECT>
 __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
 {
     constexpr int SPAN = NW * NT * 64;                    // tokens a workgroup can cover
@@ -181,20 +88,10 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    int split, bkv;
-    if constexpr (FUSED) {
-        const int x = blockIdx.x & 7, k = blockIdx.x >> 3;
-        const int rl = k / p.splits;                      // row slot on this XCD
-        split = k - rl * p.splits;
-        bkv = ((rl / p.group) * 8 + x) * p.group + rl % p.group;
-        if (bkv >= p.rows) return;
-    } else {
-        split = blockIdx.x;
-        bkv = blockIdx.y;
-    }
+    const int split = blockIdx.x, bkv = blockIdx.y;
     const int b = bkv / p.Hkv, kvh = bkv % p.Hkv;
     const int G = p.G;
-    const int64_t pbase = (int64_t)bkv * p.splits + split;
+    const int64_t pbase = (int64_t)bkv * gridDim.x + split;
 
     int T = p.T;
     if (p.seq_len) T = min(max(__builtin_amdgcn_readfirstlane(p.seq_len[b]), 0), p.T);
@@ -211,7 +108,6 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
                 p.part_ml[pbase * 8 + tid] = -INFINITY;
                 p.part_ml[pbase * 8 + 4 + tid] = 0.0f;
             }
-            if constexpr (FUSED) fused_tail<NW>(p, bkv, b, kvh);
         }
         return;
     }
@@ -451,7 +347,6 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
             }
         }
     }
-    if constexpr (FUSED) fused_tail<NW>(p, bkv, b, kvh);
     if constexpr (DIRECT) {
         __syncthreads();
         if (tid < 64 && hr < G) {   // 16 lanes per head row, as the merge kernel has them
@@ -646,74 +541,6 @@ using namespace mi;
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
-// ---- what the FUSED kernels need from the host: arrival counters that are zero between calls, and the knowledge
-// that workgroup i of a one-dimensional grid runs on XCD i % 8.
-// The counters are slices of a static device array (zero when the code object is loaded; every device holds its
-// own copy); a call takes the next slice of the ring, so two calls that are in flight at once (other streams,
-// other threads) never share a counter unless 65536 counters' worth of calls were started in between.
-static constexpr int SYNC_POOL = 1 << 16;
-static __device__ __align__(256) unsigned sync_pool[SYNC_POOL];
-static constexpr int MAX_DEVICES = 64;
-static std::atomic<unsigned *> g_sync_ptr[MAX_DEVICES];
-static std::atomic<int> g_xcd_round_robin[MAX_DEVICES];   // 0: not probed, 1: workgroup i runs on XCD i % 8, -1: it does not
-static std::atomic<uint32_t> g_sync_ticket;
-
-namespace mi {
-namespace avt {
-__global__ void k_xcc_probe(int *out)
-{
-    // hardware register 20 (XCC_ID), bits 3:0: the XCD this wave runs on; a short sleep keeps earlier workgroups
-    // resident while later ones are placed
-    const int xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;
-    __builtin_amdgcn_s_sleep(16);
-    __builtin_amdgcn_s_sleep(16);
-    if (threadIdx.x == 0) out[blockIdx.x] = xcc;
-}
-}  // namespace avt
-
-// Called by mi_ctx_create with `device` current: address of the device's counter array, and one probe launch that
-// establishes how the hardware deals workgroups to the XCDs.  Allocates and synchronizes: not for capture.
-int32_t attn_sync_bind(int device)
-{
-    if (device < 0 || device >= MAX_DEVICES) return MI_OK;   // such a device simply never takes the fused path
-    if (!g_sync_ptr[device].load(std::memory_order_acquire)) {
-        void *sym = nullptr;
-        MI_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(sync_pool)));
-        if (!sym) return MI_EIO;
-        g_sync_ptr[device].store(static_cast<unsigned *>(sym), std::memory_order_release);
-    }
-    if (g_xcd_round_robin[device].load(std::memory_order_acquire) == 0) {
-        constexpr int N = 4096;
-        int *dev_out = nullptr;
-        MI_HIP(hipMalloc(reinterpret_cast<void **>(&dev_out), N * sizeof(int)));
-        static int host_out[N];
-        hipLaunchKernelGGL(avt::k_xcc_probe, dim3(N), dim3(64), 0, nullptr, dev_out);
-        hipError_t e = hipMemcpy(host_out, dev_out, N * sizeof(int), hipMemcpyDeviceToHost);
-        (void)hipFree(dev_out);
-        if (e != hipSuccess) return hip_fail(e);
-        bool ok = true;
-        for (int i = 0; i < N && ok; ++i) ok = host_out[i] == host_out[i & 7];
-        for (int i = 0; i < 8 && ok; ++i)
-            for (int j = 0; j < i; ++j) ok = ok && host_out[i] != host_out[j];
-        g_xcd_round_robin[device].store(ok ? 1 : -1, std::memory_order_release);
-    }
-    return MI_OK;
-}
-}  // namespace mi
-
-// counters for one call, or null when this device was never bound / the ring cannot hold them
-static unsigned *take_counters(int n)
-{
-    int device = -1;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MAX_DEVICES) return nullptr;
-    unsigned *base = g_sync_ptr[device].load(std::memory_order_acquire);
-    if (!base || n > SYNC_POOL || g_xcd_round_robin[device].load(std::memory_order_acquire) != 1) return nullptr;
-    for (;;) {
-        const uint32_t t = g_sync_ticket.fetch_add((uint32_t)n, std::memory_order_relaxed) % SYNC_POOL;
-        if (t + (uint32_t)n <= SYNC_POOL) return base + t;   // a slice that does not wrap
-    }
-}
-
 static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, const int8_t *vt, const float *vs, float *o,
                       int8_t *oq, float *oscale, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                       const int32_t *seq_len, int64_t T_max, int32_t out_rotated, void *workspace,
@@ -729,13 +556,6 @@ static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, cons
     if (workspace_bytes < mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max)) return MI_ENOSPC;
     const avt::Plan plan = avt::pick(B, Hkv, T_max);
     const bool direct = plan.splits == 1 && !oq;   // one workgroup sees the whole sequence: it writes the output rows
-    // Fused merge: rows (tokens' rows, when the token is quantized) are dealt to the 8 XCDs in turn, so it pays only
-    // when they come in multiples of 8, or nearly
-    const int64_t rows = B * Hkv, group = oq ? Hkv : 1, ngroups = rows / group, padded = (ngroups + 7) / 8 * 8;
-    unsigned *ctr = nullptr;
-    static const bool fused_allowed = [] { const char *e = getenv("MI_ATTN_FUSED_MERGE"); return !(e && e[0] == '0'); }();
-    if (!direct && fused_allowed && padded * 8 <= ngroups * 9 && padded * group * plan.splits < (1LL << 31))
-        ctr = take_counters((int)(rows + B));
     avt::Params p;
     p.q = q; p.kq = kq; p.ks = ks; p.vt = vt; p.vs = vs;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.G = (int)(Hq / Hkv); p.T = (int)T_max;
@@ -747,24 +567,9 @@ static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, cons
     p.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                           align_up(B * Hkv * plan.splits * 4 * avt::D * 4, 256));
     p.blocks_per_split = plan.per;
-    p.rows = (int)rows; p.splits = plan.splits;
-    p.row_ctr = ctr; p.tok_ctr = ctr ? ctr + rows : nullptr;
-    p.group = (int)group;
-    p.oq = oq; p.oscale = oscale;
-    // merged fp32 rows: the caller's buffer, or (quantized output without o_rot) the third area of the workspace
-    p.rows_out = o ? o : reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                                   align_up(B * Hkv * plan.splits * 4 * avt::D * 4, 256) +
-                                                   align_up(B * Hkv * plan.splits * 8 * 4, 256));
-    const int nt = (plan.per + 3) / 4;
-    if (ctr) {
-        const dim3 grid((unsigned)(padded * group * plan.splits));
-#define MI_FUSED(NT_) hipLaunchKernelGGL((avt::k_gqa_tiled_split<4, NT_, 8, false, true>), grid, dim3(256), 0, s, p)
-        if (nt <= 1) MI_FUSED(1); else if (nt <= 2) MI_FUSED(2); else MI_FUSED(4);
-#undef MI_FUSED
-        return launch_status();
-    }
     const dim3 grid((unsigned)plan.splits, (unsigned)(B * Hkv));
-#define MI_TILED(NT_, DIR_) hipLaunchKernelGGL((avt::k_gqa_tiled_split<4, NT_, 8, DIR_, false>), grid, dim3(256), 0, s, p)
+    const int nt = (plan.per + 3) / 4;
+#define MI_TILED(NT_, DIR_) hipLaunchKernelGGL((avt::k_gqa_tiled_split<4, NT_, 8, DIR_>), grid, dim3(256), 0, s, p)
     if (direct) { if (nt <= 1) MI_TILED(1, true); else if (nt <= 2) MI_TILED(2, true); else MI_TILED(4, true); }
     else { if (nt <= 1) MI_TILED(1, false); else if (nt <= 2) MI_TILED(2, false); else MI_TILED(4, false); }
 #undef MI_TILED

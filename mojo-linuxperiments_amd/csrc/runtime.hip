@@ -29,7 +29,6 @@ int32_t compute_units()
 }
 
 int32_t linear_scratch_bind(int device, unsigned char **out);   // gemm.hip: address of the static scratch array
-int32_t attn_sync_bind(int device);                             // attention_tiled.hip
 
 __global__ void k_fill_u32(uint32_t *dst, uint32_t value, int64_t count)
 {
@@ -117,8 +116,6 @@ int32_t mi_ctx_create(int32_t device, mi_ctx **out)
     // the library's set-up call: look up this device's copy of the static scratch array now, so that
     // mi_w8a8_linear_f32_noalloc never has to on a caller's critical path
     int32_t rc = linear_scratch_bind(device, nullptr);
-    if (rc) return rc;
-    rc = attn_sync_bind(device);   // counters of the attention kernels that merge their own splits, and the XCD probe
     if (rc) return rc;
     mi_ctx *c = new (std::nothrow) mi_ctx;
     if (!c) return MI_ENOMEM;

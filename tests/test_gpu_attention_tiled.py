@@ -236,43 +236,3 @@ def test_vt_append_matches_row_major_append(mi, dev, orc):
         assert np.array_equal(vt, want_v)
         assert np.array_equal(kt, want_k)
     dev.reset_to(mark)
-
-
-@pytest.mark.parametrize("B,Hq,Hkv,T", [(16, 32, 8, 4096), (8, 8, 2, 2048), (16, 16, 4, 1500)])
-def test_tiled_merge_inside_the_split_kernel_sees_fresh_partials(mi, dev, orc, B, Hq, Hkv, T):
-    """Row counts that are multiples of 8 take the kernel whose last workgroup per row merges the splits itself
-    (no second launch).  The workspace is poisoned with NaN before every call: a merge that read a stale line
-    instead of what the other workgroups just wrote would show it.  Both outputs - fp32 rows, and rows quantized
-    per token for the output projection - over several calls in a row."""
-    mark = dev.mark()
-    T_cap = (T + 63) // 64 * 64
-    q, kq, ks, vq, vs, ks_c, vs_c = make_cache(mi, dev, 900 + T, B, Hq, Hkv, T, T_cap)
-    dkt, dvt = convert(mi, dev, kq, vq, T, T_cap)
-    dq, dks, dvs = dev.upload(q), dev.upload(ks_c), dev.upload(vs_c)
-    nws = mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, 128, T_cap)
-    ws = dev.empty(nws, np.uint8)
-    do, dor = dev.empty((B, Hq, 128), np.float32), dev.empty((B, Hq, 128), np.float32)
-    doq, dos = dev.empty((B, Hq * 128), np.int8), dev.empty(B, np.float32)
-    dlen = dev.upload(np.full(B, T, np.int32))
-    want = orc.gqa_decode(q, kq, ks, vq, vs, out_rotated=True)
-    for it in range(6):
-        mi.check(mi.lib.mi_fill_u32(ws.ptr, 0x7fc00000, nws // 4, None))
-        mi.check(mi.lib.mi_fill_u32(do.ptr, 0x7fc00000, B * Hq * 128, None))
-        mi.check(mi.lib.mi_gqa_decode_attn_tiled(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, do.ptr, B, Hq, Hkv, 128, T_cap,
-                                                 dlen.ptr, T, 1, ws.ptr, ws.nbytes, None))
-        o = dev.download(do)
-        assert np.all(np.isfinite(o)), "call %d read a stale partial" % it
-        assert np.max(np.abs(o - want)) <= 2e-5
-        mi.check(mi.lib.mi_fill_u32(ws.ptr, 0x7fc00000, nws // 4, None))
-        mi.check(mi.lib.mi_fill_u32(dor.ptr, 0x7fc00000, B * Hq * 128, None))
-        with_rows = it % 2 == 0      # the fp32 row is optional: without it the kernel parks it in the workspace
-        mi.check(mi.lib.mi_gqa_decode_attn_tiled_quant_i8(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr,
-                                                          dor.ptr if with_rows else None, doq.ptr, dos.ptr, B, Hq, Hkv,
-                                                          128, T_cap, dlen.ptr, T, ws.ptr, ws.nbytes, None))
-        if with_rows:
-            assert np.array_equal(dev.download(dor), o)
-        codes, scales = dev.download(doq), dev.download(dos)
-        for b in range(B):
-            cq, cs = orc.quant_row(o[b].reshape(-1))
-            assert np.array_equal(codes[b], cq) and scales[b] == cs, (it, b)
-    dev.reset_to(mark)
