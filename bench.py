@@ -340,12 +340,17 @@ def graph_time(mi, dev, s, timer, calls, reps):
     for c in calls:
         c()
     dev.sync(s)
+    # a graph launch itself costs a pause of several microseconds on the stream (8.8 us between two launches in the
+    # kernel trace): the list is recorded as many times over as it takes to put 60 calls or more into one graph, so
+    # that the pause is spread over them instead of over three or six
+    rounds = max(1, -(-60 // len(calls)))
     with mi.Graph.capture(s) as g:
-        for c in calls:
-            c()
+        for _ in range(rounds):
+            for c in calls:
+                c()
     g.launch()
     dev.sync(s)
-    ms = timer.run(lambda: g.launch(), reps) / len(calls)
+    ms = timer.run(lambda: g.launch(), max(2, reps // rounds + 1)) / (len(calls) * rounds)
     g.destroy()
     return ms
 
