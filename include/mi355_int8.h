@@ -318,7 +318,9 @@ MI_API int32_t mi_moe_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_o
 /* ---- a11: grouped expert SwiGLU FFN over expert-sorted segments.
  * x fp32 [T,H]; idx,w [T,topk]; wg,wu int8 [E,I,H] + sg,su fp32 [E,I];
  * wd int8 [E,H,I] + sd fp32 [E,H]; y fp32 [T,H].
- * H % 128 == 0 (input block 128), I % 256 == 0 (inner block 256). */
+ * H % 128 == 0 (input block 128), I % 256 == 0 (inner block 256).
+ * idx as mi_moe_route writes it: a token lists an expert at most once (a repeated expert would be dispatched once:
+ * the kernels cannot check it).  A slot whose index lies outside [0, E) is skipped: it contributes 0 to y. */
 MI_API int64_t mi_moe_ffn_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk);
 MI_API int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w,
                           const int8_t *wg, const float *sg, const int8_t *wu, const float *su,

@@ -732,15 +732,19 @@ __global__ __launch_bounds__(256) void k_moe_expert_rx(const int8_t *__restrict_
         moe_expert_rx_body<DOWN, NSMAX, 3>(act, act_scale, perm, seg_off, w0, sc0, w1, sc1, out, Kdim, Nrows, Hout, topk, nchl, e, bx);
 }
 
-// y[t, n] = sum over slots in order of w[t, slot] * out[t*topk + slot, n]
+// y[t, n] = sum over slots in order of w[t, slot] * out[t*topk + slot, n].  A slot whose expert index lies outside
+// [0, E) was never dispatched, so its row of `out` was never written: it contributes nothing.
 __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ out, const float *__restrict__ w,
-                                                     float *__restrict__ y, int T, int H, int topk)
+                                                     const int32_t *__restrict__ idx, float *__restrict__ y, int T,
+                                                     int H, int topk, int E)
 {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (int64_t)T * H) return;
     const int t = (int)(i / H), n = (int)(i - (int64_t)t * H);
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s = 0; s < topk; ++s) {
+        const int e = idx[(int64_t)t * topk + s];
+        if (e < 0 || e >= E) continue;
         const float ws = w[(int64_t)t * topk + s];
         const float4 v = *reinterpret_cast<const float4 *>(out + ((int64_t)t * topk + s) * H + n);
         a.x = a.x + ws * v.x; a.y = a.y + ws * v.y; a.z = a.z + ws * v.z; a.w = a.w + ws * v.w;
@@ -953,8 +957,8 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     }
     rc = launch_status();
     if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_combine, dim3((unsigned)((T * H / 4 + 255) / 256)), dim3(256), 0, s, out, w, y,
-                       (int)T, (int)H, (int)topk);
+    hipLaunchKernelGGL(moe::k_moe_combine, dim3((unsigned)((T * H / 4 + 255) / 256)), dim3(256), 0, s, out, w, idx, y,
+                       (int)T, (int)H, (int)topk, (int)E);
     return launch_status();
 }
 

@@ -164,6 +164,36 @@ def test_ffn_skewed_routing_many_rows_per_expert(mi, dev, orc):
     dev.reset_to(mark)
 
 
+def test_ffn_slot_with_an_expert_out_of_range_contributes_nothing(mi, dev, orc):
+    """A caller-made idx with an index outside [0, E): that pair is never dispatched, its row of the workspace is
+    never written, and the combine leaves it out: y equals the FFN over the remaining slots."""
+    mark = dev.mark()
+    T, H, I, E, topk = 12, 256, 256, 16, 2
+    x = workload.activations(56, T, H)
+    g = np.random.default_rng(56)
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    w = g.random((T, topk)).astype(np.float32)
+    experts = make_experts(orc, 57, E, H, I)
+    bad = idx.copy()
+    bad[3, 1], bad[7, 0] = E + 5, -1
+    # poison the workspace so that a stale row would show
+    ws_bytes = mi.lib.mi_moe_ffn_workspace_bytes(T, H, I, E, topk)
+    junk = dev.empty(ws_bytes, np.uint8)
+    mi.check(mi.lib.mi_fill_u32(junk.ptr, 0x7fc00000, ws_bytes // 4, None))
+    dev.sync()
+    dev.reset_to(mark)
+    r = run_ffn(mi, dev, x, bad, w, experts)
+    # the same with weight 0 on those slots and a valid (unused) expert in their place
+    ok_idx, w0 = idx.copy(), w.copy()
+    w0[3, 1] = w0[7, 0] = 0.0
+    for t, s_ in ((3, 1), (7, 0)):
+        ok_idx[t, s_] = next(e for e in range(E) if e not in ok_idx[t])
+    yo = orc.moe_ffn(x, ok_idx, w0, *experts, 128, 256)
+    assert np.all(np.isfinite(r["y"]))
+    assert np.linalg.norm(r["y"] - yo) <= 1e-3 * np.linalg.norm(yo)
+    dev.reset_to(mark)
+
+
 def test_full_layer_cfg4(mi, dev, orc):
     """512 tokens, hidden 2048, 128 experts, top-8, inner 768."""
     mark = dev.mark()
