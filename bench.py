@@ -281,6 +281,7 @@ def main():
         sub.update(cfg0_linear(mi, wl, dev, s, timer, shapes))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer))
         sub.update(decode_layer_chain(mi, wl, dev, s, timer, batch=1))
+        sub.update(moe_decode_layer_chain(mi, wl, dev, s, timer))
         if not args.skip_stack:
             # the whole stack as one graph: 32 layers, each with its own weights and cache (11.4 GB), in an arena
             # of its own that lives only for this measurement
@@ -579,6 +580,59 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None, nlayers=3):
     res["us_per_step"] = round(ms * 1e3 * nlayers, 1)                           # measured: the stack is one graph
     res["tokens_per_s"] = round(B / (nlayers * ms * 1e-3), 1)
     return {"decode_stack_%d_layers_b%d_t4096" % (nlayers, B): res}
+
+
+def moe_decode_layer_chain(mi, wl, dev, s, timer, reps=10, nlayers=3):
+    """A decode step through decoder layers whose FFN is the cfg4 MoE (hidden 2048, 16/4 heads of 128, 128 experts
+    top-8, inner 768), 16 sequences with 4095 cached tokens each: three layers with their own weights (1.8 GB of
+    experts) and caches, one graph.  With 16 tokens x 8 picks about two thirds of the experts are hit per layer."""
+    c, m = wl.ATTN, wl.MOE
+    B, D, T = c["B"], c["D"], c["T"]
+    H, E, topk, I = m["H"], m["E"], m["topk"], m["I"]
+    Hq, Hkv = H // D, max(1, H // D // 4)
+    mark = dev.mark()
+    inv = 10000.0 ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
+    ang = np.arange(T, dtype=np.float64)[:, None] * inv[None, :]
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    g1 = np.ones(H, np.float32)
+    lib = mi.lib
+    layers = []
+    for li in range(nlayers):
+        wq = wl.weights(800 + li, (Hq + 2 * Hkv) * D, H, 0)
+        wo = wl.weights(800 + li, H, Hq * D, 1)
+        moe = {"wr": wl.weights(800 + li, E, H, 2), "topk": topk}
+        for name, n, k, b, st in (("g", I, H, wl.HADAMARD_BLOCK, 3), ("u", I, H, wl.HADAMARD_BLOCK, 4),
+                                  ("d", H, I, wl.MOE_INNER_BLOCK, 5)):
+            m2 = dev.mark()
+            q, sc = dev.empty((E, n, k), np.int8), dev.empty((E, n), np.float32)
+            keep = dev.mark()
+            w = dev.upload(wl.weights(800 + li, E * n, k, st))
+            mi.check(lib.mi_fwht_quant_f32_i8(w.ptr, q.ptr, sc.ptr, E * n, k, b, s))
+            dev.sync(s)
+            dev.reset_to(keep)
+            moe["w" + name], moe["s" + name] = q, sc
+        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, wq, wo, None, None, g1, g1, cos, sin, moe=moe)
+        m2 = dev.mark()
+        src = dev.upload(wl.normal(900 + li, (B * Hkv * T, D), 0))
+        L.fill_cache_from_rows(src, T, s)
+        dev.sync(s)
+        dev.reset_to(m2)
+        layers.append(L)
+    x = dev.upload(wl.activations(701, B, H))
+    out = dev.empty((B, H), np.float32)
+    dpos, dlen = dev.upload(np.full(B, T - 1, np.int32)), dev.upload(np.full(B, T, np.int32))
+
+    def step():
+        layers[0].step(x, dpos, dlen, T, None, s)
+        for li in range(1, nlayers):
+            layers[li].step(layers[li - 1].dn, dpos, dlen, T, out if li == nlayers - 1 else None, s,
+                            residual=layers[li - 1].h1)
+    ms = graph_time(mi, dev, s, timer, [step], reps) / nlayers
+    dev.reset_to(mark)
+    return {"decode_layer_moe_b%d_t4096" % B: {
+        "us_per_layer": round(ms * 1e3, 2), "layers_in_graph": nlayers, "tokens_per_s_per_layer": round(B / (ms * 1e-3), 1),
+        "shape": "hidden %d, %d/%d heads, %d experts top-%d, inner %d" % (H, Hq, Hkv, E, topk, I),
+        "expert_weight_bytes_per_layer": wl.moe_weight_bytes(E, H, I)}}
 
 
 def host_staging(mi, wl, dev, s, timer):

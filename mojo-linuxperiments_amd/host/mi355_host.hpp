@@ -315,6 +315,31 @@ struct PagedKvCache {
     }
 };
 
+// Router + top-k dispatch + grouped expert SwiGLU FFN.
+struct MoeFfn {
+    int64_t T = 0, H = 0, I = 0, E = 0;
+    int32_t topk = 0;
+    const float *wr = nullptr;
+    const int8_t *wg = nullptr, *wu = nullptr, *wd = nullptr;
+    const float *sg = nullptr, *su = nullptr, *sd = nullptr;
+    void *workspace = nullptr;
+    int64_t workspace_bytes = 0;
+
+    template <typename Arena>
+    bool prepare(Arena &arena, int64_t t, int64_t h, int64_t i, int64_t e, int32_t k)
+    {
+        T = t; H = h; I = i; E = e; topk = k;
+        workspace_bytes = mi_moe_layer_workspace_bytes(T, H, I, E, topk);
+        if (workspace_bytes <= 0) return false;
+        workspace = arena.template alloc<uint8_t>(workspace_bytes);
+        return workspace != nullptr;
+    }
+    int32_t forward(const float *x, float *y, void *stream) const
+    {
+        return mi_moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream);
+    }
+};
+
 // One decoder layer of a decode step (one new token per sequence), chained on one stream, ten launches (eight for a single sequence):
 // (residual +) RMSNorm + quantize -> QKV GEMV -> rotary + cache append -> attention over the cache (split, merge +
 // quantize: the output projection takes the rows in the rotated basis of V) -> O GEMV -> residual + RMSNorm +
@@ -325,6 +350,8 @@ struct DecoderLayer {
     float eps = 1e-5f;
     QuantLinear<128> qkv, o, gate_up, down;
     KvCache cache;
+    // the MoE FFN in place of the dense one (gate_up / down stay unprepared): set by use_moe()
+    const MoeFfn *moe = nullptr;
     const float *g1 = nullptr, *g2 = nullptr, *rope_cos = nullptr, *rope_sin = nullptr;
     // fp32 rows: layer input when it is a sum (h0), projections, attention output, residual stream after
     // attention (h1), down output (dn); xn / att (rotated basis) / hn / act only when prepare() was asked to trace
@@ -346,9 +373,10 @@ struct DecoderLayer {
         B = b; H = h; Hq = hq; Hkv = hkv; I = i; T_cap = t_cap; eps = epsilon;
         g1 = norm1; g2 = norm2; rope_cos = cos_table; rope_sin = sin_table;
         const int64_t nqkv = (Hq + 2 * Hkv) * 128;
+        // wgu == wd == nullptr: the FFN half will be an MoE (use_moe)
         bool ok = qkv.prepare(arena, wqkv, nqkv, H, B, stream) && o.prepare(arena, wo, H, Hq * 128, B, stream) &&
-                  gate_up.prepare(arena, wgu, 2 * I, H, B, stream) && down.prepare(arena, wd, H, I, B, stream) &&
-                  cache.prepare(arena, B, Hq, Hkv, T_cap);
+                  (!wgu || gate_up.prepare(arena, wgu, 2 * I, H, B, stream)) &&
+                  (!wd || down.prepare(arena, wd, H, I, B, stream)) && cache.prepare(arena, B, Hq, Hkv, T_cap);
         h0 = arena.template alloc<float>(B * H);
         qkv_out = arena.template alloc<float>(B * nqkv);
         q = arena.template alloc<float>(B * Hq * 128);
@@ -369,6 +397,17 @@ struct DecoderLayer {
         }
         return ok && h0 && qkv_out && q && ao && h1 && gu && dn && ca && ci && sa && si;
     }
+    // The FFN half becomes residual + RMSNorm -> router, dispatch, grouped expert FFN (ffn prepared for T = B tokens,
+    // hidden H; it must outlive the layer).  false if the arena is exhausted or the shapes disagree.
+    template <typename Arena>
+    bool use_moe(Arena &arena, const MoeFfn &ffn)
+    {
+        if (ffn.T != B || ffn.H != H || !ffn.workspace) return false;
+        if (!hn) hn = arena.template alloc<float>(B * H);
+        if (!hn) return false;
+        moe = &ffn;
+        return true;
+    }
     // x fp32 [B,H], plus residual fp32 [B,H] or nullptr: the layer input is their sum (left in h0).  pos, seq_len
     // int32 [B] in device memory (seq_len = pos + 1 in a plain decode step); t_max bounds seq_len.  out fp32 [B,H],
     // or nullptr: the closing residual add is left to the next layer (give it x = dn, residual = h1).
@@ -383,11 +422,16 @@ struct DecoderLayer {
         if (rc == MI_OK) rc = cache.rope_append(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, pos, stream);
         if (rc == MI_OK) rc = cache.attend_quant(q, att, ca, sa, seq_len, t_max, stream);
         if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
-        if (rc == MI_OK)
-            rc = mi_rmsnorm_linear_f32(ao, xin, g2, eps, h1, hn, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, 128,
-                                       gate_up.workspace, gate_up.workspace_bytes, stream);
-        if (rc == MI_OK) rc = mi_swiglu_quant_f32_i8(gu, act, ci, si, B, I, 128, stream);
-        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ci, si, down.qw, down.sw, dn, B, H, I, stream);
+        if (moe) {
+            if (rc == MI_OK) rc = mi_rmsnorm_f32(ao, xin, g2, eps, h1, hn, B, H, stream);
+            if (rc == MI_OK) rc = moe->forward(hn, dn, stream);
+        } else {
+            if (rc == MI_OK)
+                rc = mi_rmsnorm_linear_f32(ao, xin, g2, eps, h1, hn, gate_up.qw, gate_up.sw, gu, B, 2 * I, H, 128,
+                                           gate_up.workspace, gate_up.workspace_bytes, stream);
+            if (rc == MI_OK) rc = mi_swiglu_quant_f32_i8(gu, act, ci, si, B, I, 128, stream);
+            if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ci, si, down.qw, down.sw, dn, B, H, I, stream);
+        }
         if (rc == MI_OK && out) rc = mi_add_f32(h1, dn, out, B * H, stream);
         return rc;
     }
@@ -445,31 +489,6 @@ struct DecoderStack {
             res = layers[l].h1;
         }
         return MI_OK;
-    }
-};
-
-// Router + top-k dispatch + grouped expert SwiGLU FFN.
-struct MoeFfn {
-    int64_t T = 0, H = 0, I = 0, E = 0;
-    int32_t topk = 0;
-    const float *wr = nullptr;
-    const int8_t *wg = nullptr, *wu = nullptr, *wd = nullptr;
-    const float *sg = nullptr, *su = nullptr, *sd = nullptr;
-    void *workspace = nullptr;
-    int64_t workspace_bytes = 0;
-
-    template <typename Arena>
-    bool prepare(Arena &arena, int64_t t, int64_t h, int64_t i, int64_t e, int32_t k)
-    {
-        T = t; H = h; I = i; E = e; topk = k;
-        workspace_bytes = mi_moe_layer_workspace_bytes(T, H, I, E, topk);
-        if (workspace_bytes <= 0) return false;
-        workspace = arena.template alloc<uint8_t>(workspace_bytes);
-        return workspace != nullptr;
-    }
-    int32_t forward(const float *x, float *y, void *stream) const
-    {
-        return mi_moe_layer(x, wr, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream);
     }
 };
 

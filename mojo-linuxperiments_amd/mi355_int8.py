@@ -420,8 +420,13 @@ class DecoderLayer:
     (xn, att, hn, act) so that a test can gate every stage."""
 
     def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
-                 block=128, trace=False, tiled=None):
+                 block=128, trace=False, tiled=None, moe=None):
+        """moe: None for the dense FFN (wgu, wd), or the experts of an MoE FFN in its place (wgu = wd = None):
+        dict(wr fp32 [E,H], wg/wu int8 [E,I,H], sg/su fp32 [E,I], wd int8 [E,H,I], sd fp32 [E,H], topk), prepared codes.
+        The second half of the layer is then residual + RMSNorm -> router, dispatch and grouped expert FFN ->
+        residual."""
         D = 128
+        self.moe = None
         # the cache lives in the matrix-pipe layouts whenever its capacity allows (a multiple of 64 tokens)
         self.tiled = (T_cap % 64 == 0) if tiled is None else bool(tiled)
         self.dev, self.B, self.H, self.Hq, self.Hkv, self.I, self.T_cap, self.eps, self.block = \
@@ -437,7 +442,14 @@ class DecoderLayer:
             dev.sync()
             dev.reset_to(keep)
             return q, s
-        self.wqkv, self.wo, self.wgu, self.wd = prep(wqkv), prep(wo), prep(wgu), prep(wd)
+        self.wqkv, self.wo = prep(wqkv), prep(wo)
+        if moe is None:
+            self.wgu, self.wd = prep(wgu), prep(wd)
+        else:
+            self.wgu = self.wd = None
+            self.moe = {k: (dev.upload(v) if isinstance(v, np.ndarray) else v) for k, v in moe.items()}
+            E = moe["wg"].shape[0]
+            self.moe_ws = dev.empty(lib.mi_moe_layer_workspace_bytes(B, H, I, E, moe["topk"]), np.uint8)
         self.g1, self.g2 = dev.upload(g1), dev.upload(g2)
         self.cos, self.sin = dev.upload(rope_cos), dev.upload(rope_sin)
         self.kq, self.ks = dev.empty((B, Hkv, T_cap, D), np.int8), dev.empty((B, Hkv, T_cap), np.float32)
@@ -448,11 +460,11 @@ class DecoderLayer:
         self.att = dev.empty((B, Hq * D), f) if trace else None
         self.ca, self.sa = dev.empty((B, Hq * D), np.int8), dev.empty(B, f)   # codes of the attention rows
         self.ao, self.h1 = dev.empty((B, H), f), dev.empty((B, H), f)
-        self.gu, self.dn = dev.empty((B, 2 * I), f), dev.empty((B, H), f)
+        self.gu, self.dn = (dev.empty((B, 2 * I), f) if moe is None else None), dev.empty((B, H), f)
         self.xn = dev.empty((B, H), f) if trace else None
-        self.hn = dev.empty((B, H), f) if trace else None
+        self.hn = dev.empty((B, H), f) if (trace or moe is not None) else None   # the MoE FFN reads the normalized row
         self.act = dev.empty((B, I), f) if trace else None
-        self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, 2 * I, H), np.uint8)   # codes of the normalized rows
+        self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, max(2 * I, self.NQKV), H), np.uint8)   # codes of the normalized rows
         self.ci, self.si = dev.empty((B, I), np.int8), dev.empty(B, f)        # codes of the activated rows
         self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
 
@@ -478,12 +490,19 @@ class DecoderLayer:
                      self.sa.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
               "mi_gqa_decode_attn_quant_i8")
         gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
-        check(lib.mi_rmsnorm_linear_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
-                                        self.wgu[0].ptr, self.wgu[1].ptr, self.gu.ptr, B, 2 * I, H, self.block,
-                                        self.lin_ws.ptr, self.lin_ws.nbytes, s), "mi_rmsnorm_linear_f32")
-        check(lib.mi_swiglu_quant_f32_i8(self.gu.ptr, p(self.act), self.ci.ptr, self.si.ptr, B, I, self.block, s),
-              "mi_swiglu_quant_f32_i8")
-        gemm_dequant(self.ci, self.si, self.wd[0], self.wd[1], self.dn, s)
+        if self.moe is None:
+            check(lib.mi_rmsnorm_linear_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
+                                            self.wgu[0].ptr, self.wgu[1].ptr, self.gu.ptr, B, 2 * I, H, self.block,
+                                            self.lin_ws.ptr, self.lin_ws.nbytes, s), "mi_rmsnorm_linear_f32")
+            check(lib.mi_swiglu_quant_f32_i8(self.gu.ptr, p(self.act), self.ci.ptr, self.si.ptr, B, I, self.block, s),
+                  "mi_swiglu_quant_f32_i8")
+            gemm_dequant(self.ci, self.si, self.wd[0], self.wd[1], self.dn, s)
+        else:
+            m = self.moe
+            check(lib.mi_rmsnorm_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, self.hn.ptr, B, H, s),
+                  "mi_rmsnorm_f32")
+            moe_layer(self.hn, m["wr"], m["wg"], m["sg"], m["wu"], m["su"], m["wd"], m["sd"], self.dn, m["topk"],
+                      self.moe_ws, stream=s)
         if out is not None:
             check(lib.mi_add_f32(self.h1.ptr, self.dn.ptr, out.ptr, B * H, s), "mi_add_f32")
 

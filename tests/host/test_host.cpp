@@ -474,6 +474,54 @@ static void test_decoder_stack(const Context &ctx)
     report("decoder_stack", good);
 }
 
+// The decoder layer with an MoE FFN (use_moe): its FFN half is residual + RMSNorm followed by MoeFfn::forward on the
+// normalized row, so the down output must equal a separate forward on that row, bit for bit, and the layer output
+// the residual sum; the routing and the expert arithmetic themselves are gated against the oracle in the Python suite.
+static void test_moe_decoder_layer(const Context &ctx)
+{
+    const int64_t B = 3, H = 512, Hq = 4, Hkv = 2, I = 256, E = 16, T_cap = 64, D = 128, NQ = (Hq + 2 * Hkv) * D;
+    const int32_t topk = 2;
+    DeviceArena<256> arena(ctx, 256 << 20);
+    Rng rng{5};
+    auto gauss = [&](int64_t n, float s) { std::vector<float> v((size_t)n); for (auto &e : v) e = s * rng.normal(); return v; };
+    std::vector<float> wqkv = gauss(NQ * H, 0.02f), wo = gauss(H * Hq * D, 0.02f), g1((size_t)H, 1.0f), g2((size_t)H, 1.0f),
+                       x = gauss(B * H, 1.0f), wr = gauss(E * H, 0.02f);
+    std::vector<float> cs((size_t)(T_cap * 64), 1.0f), sn((size_t)(T_cap * 64), 0.0f);
+    // expert weights: rotate + quantize fp32 matrices on the device
+    auto prep = [&](int64_t n, int64_t k, int32_t block, int8_t *&q, float *&sc) {
+        std::vector<float> w = gauss(E * n * k, 0.02f);
+        float *dw = upload(arena, w);
+        q = arena.alloc<int8_t>(E * n * k);
+        sc = arena.alloc<float>(E * n);
+        return dw && q && sc && mi_fwht_quant_f32_i8(dw, q, sc, E * n, k, block, nullptr) == MI_OK;
+    };
+    int8_t *wg = nullptr, *wu = nullptr, *wd = nullptr;
+    float *sg = nullptr, *su = nullptr, *sd = nullptr;
+    bool ok = prep(I, H, 128, wg, sg) && prep(I, H, 128, wu, su) && prep(H, I, 256, wd, sd);
+    MoeFfn ffn;
+    ok = ok && ffn.prepare(arena, B, H, I, E, topk);
+    ffn.wr = upload(arena, wr); ffn.wg = wg; ffn.sg = sg; ffn.wu = wu; ffn.su = su; ffn.wd = wd; ffn.sd = sd;
+    DecoderLayer layer;
+    ok = ok && layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, upload(arena, wqkv), upload(arena, wo), (const float *)nullptr,
+                             (const float *)nullptr, upload(arena, g1), upload(arena, g2), upload(arena, cs),
+                             upload(arena, sn), 1e-5f, nullptr);
+    ok = ok && layer.use_moe(arena, ffn) && layer.cache.tiled;
+    const std::vector<int32_t> pos = {0, 30, 63}, len = {1, 31, 64};
+    int32_t *dpos = upload(arena, pos), *dlen = upload(arena, len);
+    float *dx = upload(arena, x), *dout = arena.alloc<float>(B * H), *dy = arena.alloc<float>(B * H);
+    ok = ok && dpos && dlen && dx && dout && dy && layer.step(dx, nullptr, dpos, dlen, 64, dout, nullptr) == MI_OK;
+    if (!ok) { report("moe_decoder_layer", false, "set-up or launch failed"); return; }
+    std::vector<float> out = download(dout, (size_t)(B * H)), h1 = download(layer.h1, (size_t)(B * H)),
+                       dn = download(layer.dn, (size_t)(B * H));
+    bool good = ffn.forward(layer.hn, dy, nullptr) == MI_OK && download(dy, (size_t)(B * H)) == dn;
+    bool finite = true;
+    for (size_t i = 0; i < out.size(); ++i) {
+        good = good && out[i] == h1[i] + dn[i];
+        finite = finite && std::isfinite(out[i]);
+    }
+    report("moe_decoder_layer", good && finite);
+}
+
 int main()
 {
     Context ctx(0);
@@ -488,6 +536,7 @@ int main()
     test_kv_cache(ctx, 64, "kv_cache_tiled_layouts_append_attend_vs_oracle");
     test_decoder_layer(ctx);
     test_decoder_stack(ctx);
+    test_moe_decoder_layer(ctx);
     std::printf("%s\n", g_failed ? "SOME TESTS FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;
 }

@@ -107,7 +107,7 @@ def rel(a, b):
     return float(np.linalg.norm(a.astype(np.float64) - b) / max(float(np.linalg.norm(b)), 1e-30))
 
 
-def oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=None):
+def oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=None, moe=None):
     """The same chain on the CPU oracle; `cache` = [kq, ks, vq, vs] numpy arrays, updated in place.
 
     With `gpu` (the GPU's own intermediates by name) every stage is fed what the GPU fed its next kernel and is
@@ -158,6 +158,18 @@ def oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=None):
     if gpu is not None:
         assert np.array_equal(gpu["h1"], h1)
         assert np.max(np.abs(gpu["hn"] - hn)) <= 2e-6 * np.max(np.abs(hn))
+    if moe is not None:
+        # the FFN half is router + dispatch + grouped experts on the normalized row (a9-a11)
+        xin = take("hn", hn)
+        idx, w = orc.moe_route(xin, moe["wr"], moe["topk"])
+        if gpu is not None:
+            assert np.array_equal(gpu["moe_idx"], idx)
+            assert np.max(np.abs(gpu["moe_w"] - w)) <= 2e-6
+            idx, w = gpu["moe_idx"], gpu["moe_w"]
+        dn = orc.moe_ffn(xin, idx, w, moe["wg"], moe["sg"], moe["wu"], moe["su"], moe["wd"], moe["sd"], 128, 256)
+        if gpu is not None:
+            assert rel(gpu["dn"], dn) <= 1e-3          # SwiGLU goes through expf: the stated gate of the FFN output
+        return take("h1", h1) + take("dn", dn)
     gu = orc.w8a8_linear(take("hn", hn), W["gu"][0], W["gu"][1], 128)[0]
     if gpu is not None:
         assert np.array_equal(gpu["gu"], gu)
@@ -393,4 +405,56 @@ def test_one_token_gets_the_same_codes_alone_and_in_a_batch(mi, dev, K):
         alone = run([m])
         for a, b in zip(alone, batch):
             assert np.array_equal(a[0], b[m])
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("B,H,Hq,Hkv,I,E,topk,T_cap,start", [
+    (3, 512, 4, 2, 256, 16, 2, 40, [0, 17, 38]),
+    (16, 2048, 16, 4, 768, 128, 8, 128, list(range(90, 106))),      # the cfg4 experts behind a 16-sequence decode step
+])
+def test_moe_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, Hq, Hkv, I, E, topk, T_cap, start):
+    """The decoder layer with the MoE FFN in place of the dense one: attention half as above, then residual + RMSNorm,
+    router (indices exact, weights to 2e-6), dispatch and grouped expert FFN (rel-L2 1e-3 against the oracle fed the
+    GPU's routing), residual."""
+    mark = dev.mark()
+    eps = 1e-5
+    cos, sin = rope_tables(T_cap)
+    fw = {"qkv": workload.weights(43, (Hq + 2 * Hkv) * D, H, 1), "o": workload.weights(43, H, Hq * D, 2)}
+    g = np.random.default_rng(43)
+    g1 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
+    g2 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
+    moe = {"wr": workload.weights(44, E, H), "topk": topk}
+    for name, n, k, b in (("g", I, H, 128), ("u", I, H, 128), ("d", H, I, 256)):
+        q, sc = orc.rotate_quant_rows(workload.weights(45, E * n, k, len(name) + n), b)
+        moe["w" + name], moe["s" + name] = q.reshape(E, n, k), sc.reshape(E, n)
+    layer = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T_cap, fw["qkv"], fw["o"], None, None, g1, g2, cos, sin, eps,
+                            trace=True, moe=moe)
+    W = {k: orc.rotate_quant_rows(v, 128) for k, v in fw.items()}
+    W["g1"], W["g2"] = g1, g2
+    start = np.array(start, np.int32)
+    cache = [g.integers(-127, 128, (B, Hkv, T_cap, D)).astype(np.int8),
+             ((g.random((B, Hkv, T_cap)) + 0.5) * 0.03).astype(np.float32),
+             g.integers(-127, 128, (B, Hkv, T_cap, D)).astype(np.int8),
+             ((g.random((B, Hkv, T_cap)) + 0.5) * 0.03).astype(np.float32)]
+    layer.set_cache_rows(*cache)
+    dpos, dlen = dev.empty(B, np.int32), dev.empty(B, np.int32)
+    dx, dout = dev.empty((B, H), np.float32), dev.empty((B, H), np.float32)
+    names = ("xn", "qkv", "q", "att", "ca", "sa", "ao", "h1", "hn", "dn")
+    off = lambda i: mi.lib.mi_moe_ffn_workspace_offset(i, B, H, I, E, topk)
+    for step in range(2):
+        pos = (start + step).astype(np.int32)
+        lens = (pos + 1).astype(np.int32)
+        x = workload.activations(310 + step, B, H)
+        for d, a in ((dpos, pos), (dlen, lens), (dx, x)):
+            mi.check(mi.lib.mi_memcpy_h2d(d.ptr, a.ctypes.data, a.nbytes, None))
+        layer.step(dx, dpos, dlen, int(lens.max()), dout)
+        out = dev.download(dout)
+        gpu = {n: dev.download(getattr(layer, n)) for n in names}
+        gpu["kq"], gpu["ks"], gpu["vq"], gpu["vs"] = layer.get_cache_rows()
+        gpu["q"] = gpu["q"].reshape(B, Hq, D)
+        gpu["moe_idx"] = dev.download(layer.moe_ws.offset(off(8), (B, topk), np.int32))
+        gpu["moe_w"] = dev.download(layer.moe_ws.offset(off(9), (B, topk), np.float32))
+        staged = oracle_layer(orc, x, W, cache, pos, lens, cos, sin, eps, Hq, Hkv, gpu=gpu, moe=moe)
+        assert np.array_equal(out, staged)
+        assert np.all(np.isfinite(out))
     dev.reset_to(mark)
