@@ -17,6 +17,7 @@
 //
 // Bound: HBM on the int8 expert weights, E * 3 * H * I bytes per layer call.
 #include "common.h"
+#include "fwht_core.h"
 
 namespace mi {
 namespace moe {
@@ -52,8 +53,13 @@ __device__ __forceinline__ void fold(float (&p)[64], int lane)
 
 // grid = (T/16, E/16): a workgroup of 4 waves covers 16 tokens x 16 experts, so the router weights are read
 // T/16 times and the activations E/16 times in all (both from L2), and every compute unit gets work.
+// CQ > 0: the kernel also rotates (block 128) and quantizes the token rows for the expert FFN, a wave per row with CQ
+// chunks per lane (H = 512 * CQ at most), the arithmetic of the stand-alone quantizer: the 16 tokens of a group are
+// dealt to the waves of the group's workgroups, so that the layer launches one kernel less.
+template <int CQ>
 __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x, const float *__restrict__ wr,
-                                                    float *__restrict__ logits, int T, int H, int E)
+                                                    float *__restrict__ logits, int T, int H, int E,
+                                                    int8_t *__restrict__ qx, float *__restrict__ sx)
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = blockIdx.x * 16 + wave * 4;
@@ -94,6 +100,50 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
     // lane l now holds pair l: token l/16, expert e0 + l%16
     const int t = t0 + (lane >> 4);
     if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
+    if constexpr (CQ > 0) {
+        constexpr int LPB = 16;
+        const int j = lane % LPB, nchunk = H / 8;
+        for (int tt = (int)blockIdx.y * 4 + wave; tt < 16; tt += (int)gridDim.y * 4) {
+            const int row = blockIdx.x * 16 + tt;
+            if (row >= T) break;   // whole wave
+            const float *xrow = x + (int64_t)row * H;
+            float v[CQ][8];
+            int base[CQ];
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                const int c = lane + i * 64;
+                base[i] = (c / LPB) * 128 + 4 * j;
+                if (c < nchunk) {
+                    const float4 lo = *reinterpret_cast<const float4 *>(xrow + base[i]);
+                    const float4 hi = *reinterpret_cast<const float4 *>(xrow + base[i] + 64);
+                    v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+                    v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+                }
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                fwht_chunk<128>(v[i], j);
+                amax = fmaxf(amax, abs8(v[i]));
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            const float sc = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+            const float inv = (amax == 0.0f) ? 0.0f : 127.0f / amax;
+            if (lane == 0) sx[row] = sc;
+            int8_t *qrow = qx + (int64_t)row * H;
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                if (lane + i * 64 < nchunk) {
+                    *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                    *reinterpret_cast<uint32_t *>(qrow + base[i] + 64) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+                }
+            }
+        }
+    }
 }
 
 template <int CTRL>
@@ -734,20 +784,36 @@ __global__ __launch_bounds__(256) void k_moe_expert_rx(const int8_t *__restrict_
 
 // y[t, n] = sum over slots in order of w[t, slot] * out[t*topk + slot, n].  A slot whose expert index lies outside
 // [0, E) was never dispatched, so its row of `out` was never written: it contributes nothing.
+// TOPK > 0: the slot count is known at compile time (the loads of a token are then all in flight at once); 0: any.
+template <int TOPK>
 __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ out, const float *__restrict__ w,
                                                      const int32_t *__restrict__ idx, float *__restrict__ y, int T,
-                                                     int H, int topk, int E)
+                                                     int H, int topk_rt, int E)
 {
+    constexpr int NS = TOPK > 0 ? TOPK : MAX_TOPK;
+    const int topk = TOPK > 0 ? TOPK : topk_rt;
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (int64_t)T * H) return;
     const int t = (int)(i / H), n = (int)(i - (int64_t)t * H);
+    // every load of the token goes out before the first use; a slot that was never dispatched is read like the
+    // others (its row of the workspace exists, whatever it holds) and dropped by value
+    float ws[NS];
+    float4 v[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int sc = s < topk ? s : topk - 1;
+        const int e = idx[(int64_t)t * topk + sc];
+        const bool ok = s < topk && e >= 0 && e < E;
+        ws[s] = w[(int64_t)t * topk + sc];
+        v[s] = *reinterpret_cast<const float4 *>(out + ((int64_t)t * topk + sc) * H + n);
+        if (!ok) { ws[s] = 0.0f; v[s] = make_float4(0.f, 0.f, 0.f, 0.f); }
+    }
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < topk; ++s) {
-        const int e = idx[(int64_t)t * topk + s];
-        if (e < 0 || e >= E) continue;
-        const float ws = w[(int64_t)t * topk + s];
-        const float4 v = *reinterpret_cast<const float4 *>(out + ((int64_t)t * topk + s) * H + n);
-        a.x = a.x + ws * v.x; a.y = a.y + ws * v.y; a.z = a.z + ws * v.z; a.w = a.w + ws * v.w;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        if (s < topk) {
+            a.x = a.x + ws[s] * v[s].x; a.y = a.y + ws[s] * v[s].y; a.z = a.z + ws[s] * v[s].z; a.w = a.w + ws[s] * v[s].w;
+        }
     }
     *reinterpret_cast<float4 *>(y + i) = a;
 }
@@ -777,6 +843,31 @@ static int32_t check_shapes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t 
     return MI_OK;
 }
 
+// can the router's first kernel also produce the FFN's activation codes? (block 128, a wave per row)
+static bool route_can_quantize(int64_t H) { return H % 128 == 0 && H <= 2048; }
+
+// logits + top-k; qx / sx non-null (and route_can_quantize(H)): the logits kernel also rotates and quantizes x
+static int32_t launch_route(const float *x, const float *wr, int32_t *idx, float *w, int64_t T, int64_t H, int64_t E,
+                            int32_t topk, float *logits, int8_t *qx, float *sx, void *stream)
+{
+    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)(E / 16));
+    const int cq = qx ? (int)((H / 8 + 63) / 64) : 0;
+#define MI_LOGITS(CQ_) hipLaunchKernelGGL(k_moe_logits<CQ_>, grid, dim3(256), 0, as_stream(stream), x, wr, logits, (int)T, (int)H, (int)E, qx, sx)
+    switch (cq) {
+    case 0: MI_LOGITS(0); break;
+    case 1: MI_LOGITS(1); break;
+    case 2: MI_LOGITS(2); break;
+    case 3: MI_LOGITS(3); break;
+    default: MI_LOGITS(4); break;
+    }
+#undef MI_LOGITS
+    int32_t rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_moe_topk, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, as_stream(stream), logits, idx, w, (int)T,
+                       (int)E, (int)topk);
+    return launch_status();
+}
+
 }  // namespace moe
 }  // namespace mi
 
@@ -798,14 +889,7 @@ extern "C" int32_t mi_moe_route(const float *x, const float *wr, int32_t *idx, f
     if (!workspace || !aligned16(workspace)) return MI_EINVAL;
     if (workspace_bytes < mi_moe_route_workspace_bytes(T, E)) return MI_ENOSPC;
     if (T == 0) return MI_OK;
-    float *logits = static_cast<float *>(workspace);
-    hipLaunchKernelGGL(moe::k_moe_logits, dim3((unsigned)((T + 15) / 16), (unsigned)(E / 16)), dim3(256), 0,
-                       as_stream(stream), x, wr, logits, (int)T, (int)H, (int)E);
-    int32_t rc = launch_status();
-    if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_topk, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, as_stream(stream), logits, idx, w,
-                       (int)T, (int)E, (int)topk);
-    return launch_status();
+    return moe::launch_route(x, wr, idx, w, T, H, E, topk, static_cast<float *>(workspace), nullptr, nullptr, stream);
 }
 
 static int32_t launch_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_off, int32_t *order, int64_t T,
@@ -853,10 +937,11 @@ extern "C" int64_t mi_moe_ffn_workspace_offset(int32_t which, int64_t T, int64_t
     return moe::layout(T, H, I, E, topk).off[which];
 }
 
-extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w, const int8_t *wg, const float *sg,
-                              const int8_t *wu, const float *su, const int8_t *wd, const float *sd, float *y,
-                              int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk, void *workspace,
-                              int64_t workspace_bytes, void *stream)
+// codes_ready: the activation codes and scales already sit in the workspace (written by the router's first kernel)
+static int32_t run_ffn(const float *x, const int32_t *idx, const float *w, const int8_t *wg, const float *sg,
+                       const int8_t *wu, const float *su, const int8_t *wd, const float *sd, float *y, int64_t T,
+                       int64_t H, int64_t I, int64_t E, int32_t topk, void *workspace, int64_t workspace_bytes,
+                       void *stream, bool codes_ready)
 {
     int32_t rc = moe::check_shapes(T, H, I, E, topk);
     if (rc) return rc;
@@ -880,8 +965,10 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     int32_t *order = seg + E + 1;
     rc = launch_dispatch(idx, perm, seg, order, T, E, topk, stream);
     if (rc) return rc;
-    rc = mi_fwht_quant_f32_i8(x, qx, sx, T, H, 128, stream);
-    if (rc) return rc;
+    if (!codes_ready) {
+        rc = mi_fwht_quant_f32_i8(x, qx, sx, T, H, 128, stream);
+        if (rc) return rc;
+    }
     static bool attr_set = false;  // idempotent; a race only repeats the calls
     if (!attr_set) {
         MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_gemm<false>),
@@ -957,9 +1044,25 @@ extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w
     }
     rc = launch_status();
     if (rc) return rc;
-    hipLaunchKernelGGL(moe::k_moe_combine, dim3((unsigned)((T * H / 4 + 255) / 256)), dim3(256), 0, s, out, w, idx, y,
-                       (int)T, (int)H, (int)topk, (int)E);
+    const dim3 cgrid((unsigned)((T * H / 4 + 255) / 256));
+#define MI_COMBINE(K_) hipLaunchKernelGGL(moe::k_moe_combine<K_>, cgrid, dim3(256), 0, s, out, w, idx, y, (int)T, (int)H, (int)topk, (int)E)
+    switch (topk) {
+    case 1: MI_COMBINE(1); break;
+    case 2: MI_COMBINE(2); break;
+    case 4: MI_COMBINE(4); break;
+    case 8: MI_COMBINE(8); break;
+    default: MI_COMBINE(0); break;
+    }
+#undef MI_COMBINE
     return launch_status();
+}
+
+extern "C" int32_t mi_moe_ffn(const float *x, const int32_t *idx, const float *w, const int8_t *wg, const float *sg,
+                              const int8_t *wu, const float *su, const int8_t *wd, const float *sd, float *y,
+                              int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk, void *workspace,
+                              int64_t workspace_bytes, void *stream)
+{
+    return run_ffn(x, idx, w, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream, false);
 }
 
 extern "C" int32_t mi_moe_layer(const float *x, const float *wr, const int8_t *wg, const float *sg, const int8_t *wu,
@@ -975,7 +1078,12 @@ extern "C" int32_t mi_moe_layer(const float *x, const float *wr, const int8_t *w
     char *ws = static_cast<char *>(workspace);
     int32_t *idx = reinterpret_cast<int32_t *>(ws + L.off[8]);
     float *w = reinterpret_cast<float *>(ws + L.off[9]);
-    rc = mi_moe_route(x, wr, idx, w, T, H, E, topk, ws + L.off[10], mi_moe_route_workspace_bytes(T, E), stream);
+    // the checks of mi_moe_route, which this call stands in for
+    if (!x || !wr || H % 256 || E % 16 || E > 256 || !aligned16(x) || !aligned16(wr)) return MI_EINVAL;
+    const bool fuse = moe::route_can_quantize(H);
+    rc = moe::launch_route(x, wr, idx, w, T, H, E, topk, reinterpret_cast<float *>(ws + L.off[10]),
+                           fuse ? reinterpret_cast<int8_t *>(ws + L.off[0]) : nullptr,
+                           fuse ? reinterpret_cast<float *>(ws + L.off[1]) : nullptr, stream);
     if (rc) return rc;
-    return mi_moe_ffn(x, idx, w, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream);
+    return run_ffn(x, idx, w, wg, sg, wu, su, wd, sd, y, T, H, I, E, topk, workspace, workspace_bytes, stream, fuse);
 }
