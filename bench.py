@@ -33,6 +33,9 @@ PEAK_HBM_GBS = 8000.0
 MALL_BYTES = 256 << 20
 
 
+NO_GRAPH = False    # --no-graph: every timing loop launches eagerly
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -103,10 +106,15 @@ def main():
                          "caches), each with its own weights and KV cache, as one graph")
     ap.add_argument("--skip-stack", action="store_true", help="no 32-layer decode stack leg (it takes 15 GB more)")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch everything eagerly: for runs under rocprofv3's kernel trace, whose tool library "
+                         "ended in a segmentation fault inside hipGraphLaunch; the line then says method: eager")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
+    global NO_GRAPH
+    NO_GRAPH = args.no_graph
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
 
@@ -202,13 +210,17 @@ def main():
     # The declared method: the same K steps recorded once into a graph (the weight rotation is baked in) and
     # replayed as one launch, exactly K steps inside the timed region and no host work between kernels.  The eager
     # figure is reported beside it and never picked.
-    with mi.Graph.capture(s) as g:
-        for _ in range(args.steps):
-            prefill_step()
-    timer.settle(lambda: g.launch())
-    ms_graph = timer.run(lambda: g.launch(), 1) / args.steps
-    g.destroy()
-    ms_step = ms_graph
+    if NO_GRAPH:
+        ms_graph = None
+        ms_step = ms_eager
+    else:
+        with mi.Graph.capture(s) as g:
+            for _ in range(args.steps):
+                prefill_step()
+        timer.settle(lambda: g.launch())
+        ms_graph = timer.run(lambda: g.launch(), 1) / args.steps
+        g.destroy()
+        ms_step = ms_graph
     step_ops = sum(wl.gemm_ops(M, N, K) for _, K, N in wl.PROJECTIONS)
     value = step_ops / (ms_step * 1e-3) / 1e12
 
@@ -268,7 +280,8 @@ def main():
                                "run untimed before the W warm-up steps so that timing starts at the sustained clock",
                    "tokens": M, "ops_per_step": step_ops, "tokens_per_s": round(M / (ms_step * 1e-3), 1),
                    "wall_ms_per_step": round(wall_ms, 4),
-                   "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph": round(ms_graph, 4)},
+                   "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
+                   "method": "eager (--no-graph)" if NO_GRAPH else "graph replay"},
         "roofline": roofline,
         "host": host_topology(),
     }
@@ -338,6 +351,8 @@ def graph_time(mi, dev, s, timer, calls, reps):
     """Per-call ms of a list of closures recorded once into a graph and replayed
     (decode kernels are a few microseconds: eager launches from Python would
     measure the interpreter)."""
+    if NO_GRAPH:
+        return eager_time(dev, s, timer, calls, max(1, reps // 2))
     for c in calls:
         c()
     dev.sync(s)
@@ -461,11 +476,11 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
                                       "row_major_paged_16_token_pages_us": round(ms_paged * 1e3, 2)}}
 
 
-def eager_time(dev, s, timer, calls):
+def eager_time(dev, s, timer, calls, reps=1):
     for c in calls:
         c()
     dev.sync(s)
-    return timer.run(lambda: [c() for c in calls], 1) / len(calls)
+    return timer.run(lambda: [c() for c in calls], reps) / len(calls)
 
 
 def moe_layer(mi, wl, dev, s, timer, reps=20, graph=True):

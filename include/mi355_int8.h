@@ -278,6 +278,24 @@ MI_API int32_t mi_gqa_decode_attn_tiled_quant_i8(const float *q, const int8_t *k
                                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                                                  const int32_t *seq_len, int64_t T_max,
                                                  void *workspace, int64_t workspace_bytes, void *stream);
+/* ... and with the output projection behind it, as one call: y fp32 [B, N] = the attention rows of a token (Hq*D
+ * values in the rotated basis of V, quantized as one row) contracted with prepared projection weights qw int8
+ * [N, Hq*D], sw fp32 [N] (rotated along K with block D), N % 16 == 0, Hq <= 64.  The values are those of
+ * mi_gqa_decode_attn_tiled_quant_i8 followed by mi_w8a8_gemm_dequant_f32, bit for bit; what differs is the division
+ * of the work for ONE token (B == 1, Hq*D in {2048, 4096}): the merge then runs over many workgroups and leaves the
+ * fp32 row, and the projection's GEMV quantizes that row in its own prologue (three launches, none of which reads
+ * every split's partials through one compute unit).  o_rot (optional, fp32 [B,Hq,D]) receives the merged row.
+ * Workspace: mi_gqa_decode_attn_linear_workspace_bytes(B, Hq, Hkv, D, T_max).  It starts with the merged rows
+ * (fp32, B*Hq*D*4 bytes), their codes (int8 [B, Hq*D]) and their scales (fp32 [B]), each area rounded up to 256
+ * bytes - a caller may read them there after the call - and the attention's own workspace follows.  No upstream
+ * counterpart. */
+MI_API int64_t mi_gqa_decode_attn_linear_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T);
+MI_API int32_t mi_gqa_decode_attn_tiled_linear_f32(const float *q, const int8_t *kt, const float *ks,
+                                                   const int8_t *vt, const float *vs, float *o_rot,
+                                                   const int8_t *qw, const float *sw, float *y,
+                                                   int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                                   const int32_t *seq_len, int64_t T_max, int64_t N,
+                                                   void *workspace, int64_t workspace_bytes, void *stream);
 /* Row-major codes [rows, src_stride tokens, 128] (rows = B*Hkv) -> the tiled layouts, first T tokens of every row
  * (the rest of the last 64-token block touched is zero-filled); either pair (kq, kt) / (vq, vt) may be NULL.  For
  * caches that were quantized in one go (prefill) with mi_fwht_quant_f32_i8. */

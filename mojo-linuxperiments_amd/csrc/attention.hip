@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256) void k_gqa_split(Params p)
 // Merge of the splits of one (b, h) row by the 16 lanes that own it (lane j: elements 4j..4j+3 and 64+4j..).
 // SP > 0: the split count is known at compile time and every load of the row goes out before the first use (one
 // memory round trip).  Returns the normalized row in the rotated basis of V.
-template <int SP>
+template <int SP, int BATCH = 8>
 __device__ __forceinline__ void merge_row(const float *__restrict__ part_o, const float *__restrict__ part_ml,
                                           int splits_rt, int64_t bkv, int hl, int j, float (&v)[8])
 {
@@ -428,21 +428,21 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ part_o, cons
             v[6] = __builtin_fmaf(hi[s].z, w, v[6]); v[7] = __builtin_fmaf(hi[s].w, w, v[7]);
         }
     } else {
-        // any split count: the maxima first (one round trip), then the partials in batches of eight whose loads all
+        // any split count: the maxima first (one round trip), then the partials in batches of BATCH whose loads all
         // go out before the first use
         float mx = -INFINITY;
-        for (int s0 = 0; s0 < splits; s0 += 8) {
-            float ms[8];
+        for (int s0 = 0; s0 < splits; s0 += BATCH) {
+            float ms[BATCH];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ms[i] = ml0[min(s0 + i, splits - 1) * 8 + hl];
+            for (int i = 0; i < BATCH; ++i) ms[i] = ml0[min(s0 + i, splits - 1) * 8 + hl];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) mx = fmaxf(mx, ms[i]);
+            for (int i = 0; i < BATCH; ++i) mx = fmaxf(mx, ms[i]);
         }
-        for (int s0 = 0; s0 < splits; s0 += 8) {
-            float ms[8], ls[8];
-            float4 lo[8], hi[8];
+        for (int s0 = 0; s0 < splits; s0 += BATCH) {
+            float ms[BATCH], ls[BATCH];
+            float4 lo[BATCH], hi[BATCH];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < BATCH; ++i) {
                 const int s = min(s0 + i, splits - 1);
                 ms[i] = ml0[s * 8 + hl];
                 ls[i] = ml0[s * 8 + 4 + hl];
@@ -450,7 +450,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ part_o, cons
                 hi[i] = *reinterpret_cast<const float4 *>(po0 + s * 4 * attn::D + 64 + 4 * j);
             }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < BATCH; ++i) {
                 const float w = (s0 + i >= splits || ms[i] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[i] - mx);
                 l = __builtin_fmaf(ls[i], w, l);
                 v[0] = __builtin_fmaf(lo[i].x, w, v[0]); v[1] = __builtin_fmaf(lo[i].y, w, v[1]);
@@ -465,23 +465,80 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ part_o, cons
     for (int e = 0; e < 8; ++e) v[e] *= rl;
 }
 
-// merge the splits of 16 (b, h) rows per workgroup; 16 lanes per row
+// merge the splits of blockDim.x / 16 (b, h) rows per workgroup; 16 lanes per row.  Few rows with many splits (one
+// token) take one row per workgroup, so that no compute unit reads more than one row's partials.
 template <int SP>
 __global__ __launch_bounds__(256) void k_gqa_merge(const float *__restrict__ part_o,
                                                    const float *__restrict__ part_ml, float *__restrict__ o,
                                                    int rows, int Hq, int Hkv, int G, int splits_rt, int out_rotated)
 {
     const int tid = threadIdx.x, j = tid & 15;
-    const int row = blockIdx.x * 16 + (tid >> 4);
+    const int row = blockIdx.x * (int)(blockDim.x >> 4) + (tid >> 4);
     const bool live = row < rows;
     const int rr = live ? row : rows - 1;
     const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
     const int64_t bkv = (int64_t)b * Hkv + kvh;
     float v[8];
-    merge_row<SP>(part_o, part_ml, splits_rt, bkv, hl, j, v);
+    merge_row<SP, 16>(part_o, part_ml, splits_rt, bkv, hl, j, v);
     if (!out_rotated) fwht128(v, j);  // whole workgroup takes the same branch
     if (live) {
         float *orow = o + (int64_t)row * attn::D;
+        *reinterpret_cast<float4 *>(orow + 4 * j) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(orow + 64 + 4 * j) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
+// Rows that were cut into 17 .. 32 splits (one or two tokens over a long cache): 32 lanes per row, one float4 per lane
+// and split, and every load of the row in flight at once.  The partials were written by workgroups all over the
+// chip, so every dependent batch of loads is a round trip to memory of 2-3 us: merge_row's batches of 8 or 16 cost
+// four of them here, this kernel one.  Per element the sum runs over the splits in index order with the same
+// operations as merge_row: the same bits.
+__global__ __launch_bounds__(64) void k_gqa_merge_wide(const float *__restrict__ part_o,
+                                                       const float *__restrict__ part_ml, float *__restrict__ o,
+                                                       int rows, int Hq, int Hkv, int G, int splits, int out_rotated)
+{
+    constexpr int SMAX = 32;
+    const int tid = threadIdx.x, j = tid & 15, half = (tid >> 4) & 1;
+    const int row = blockIdx.x * 2 + (tid >> 5);
+    const bool live = row < rows;
+    const int rr = live ? row : rows - 1;
+    const int b = rr / Hq, h = rr % Hq, kvh = h / G, hl = h % G;
+    const int64_t bkv = (int64_t)b * Hkv + kvh;
+    const float *ml0 = part_ml + bkv * splits * 8;
+    const float *po0 = part_o + (bkv * splits * 4 + hl) * attn::D + half * 64 + 4 * j;
+    float ms[SMAX], ls[SMAX];
+    float4 d[SMAX];
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+        const int sc = min(s, splits - 1);
+        ms[s] = ml0[sc * 8 + hl];
+        ls[s] = ml0[sc * 8 + 4 + hl];
+        d[s] = *reinterpret_cast<const float4 *>(po0 + sc * 4 * attn::D);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) mx = fmaxf(mx, ms[s]);
+    float l = 0.0f, v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+        const float w = (s >= splits || ms[s] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms[s] - mx);
+        l = __builtin_fmaf(ls[s], w, l);
+        v0 = __builtin_fmaf(d[s].x, w, v0); v1 = __builtin_fmaf(d[s].y, w, v1);
+        v2 = __builtin_fmaf(d[s].z, w, v2); v3 = __builtin_fmaf(d[s].w, w, v3);
+    }
+    const float rl = l > 0.0f ? 1.0f / l : 0.0f;
+    v0 *= rl; v1 *= rl; v2 *= rl; v3 *= rl;
+    float *orow = o + (int64_t)row * attn::D;
+    if (out_rotated) {
+        if (live) *reinterpret_cast<float4 *>(orow + half * 64 + 4 * j) = make_float4(v0, v1, v2, v3);
+        return;
+    }
+    // inverse rotation: the lower 16 lanes of a row collect the upper 16 lanes' elements 64 + 4j .. and run the
+    // 16-lane butterfly (the upper lanes run it too, on their own values twice, and store nothing)
+    const int src = (tid & ~31) | (16 + j);
+    float v[8] = {v0, v1, v2, v3, __shfl(v0, src, 64), __shfl(v1, src, 64), __shfl(v2, src, 64), __shfl(v3, src, 64)};
+    fwht128(v, j);
+    if (live && half == 0) {
         *reinterpret_cast<float4 *>(orow + 4 * j) = make_float4(v[0], v[1], v[2], v[3]);
         *reinterpret_cast<float4 *>(orow + 64 + 4 * j) = make_float4(v[4], v[5], v[6], v[7]);
     }
@@ -587,9 +644,16 @@ int32_t launch_merge(const float *part_o, const float *part_ml, float *o, int8_t
         return launch_status();
     }
     const int rows = (int)(B * Hq);
-    const dim3 mgrid((unsigned)((rows + 15) / 16));
+    if (splits > 16 && splits <= 32 && rows <= 2 * compute_units()) {
+        hipLaunchKernelGGL(k_gqa_merge_wide, dim3((unsigned)((rows + 1) / 2)), dim3(64), 0, s, part_o, part_ml, o, rows,
+                           (int)Hq, (int)Hkv, G, splits, out_rotated);
+        return launch_status();
+    }
+    int rpw = 16;   // rows per workgroup: fewer while that still adds workgroups below half a chip's worth
+    while (rpw > 1 && rows / rpw < compute_units() / 2) rpw >>= 1;
+    const dim3 mgrid((unsigned)((rows + rpw - 1) / rpw)), mblock((unsigned)(16 * rpw));
 #define MI_MERGE(SP)                                                                                              \
-    hipLaunchKernelGGL(k_gqa_merge<SP>, mgrid, dim3(256), 0, s, part_o, part_ml, o, rows, (int)Hq, (int)Hkv, G, \
+    hipLaunchKernelGGL(k_gqa_merge<SP>, mgrid, mblock, 0, s, part_o, part_ml, o, rows, (int)Hq, (int)Hkv, G, \
                        splits, out_rotated)
     switch (splits) {
     case 1: MI_MERGE(1); break;

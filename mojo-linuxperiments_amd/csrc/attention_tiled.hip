@@ -601,6 +601,58 @@ extern "C" int32_t mi_gqa_decode_attn_tiled_quant_i8(const float *q, const int8_
                   workspace_bytes, as_stream(stream));
 }
 
+namespace mi {
+int32_t launch_linear_fused(const float *, const int8_t *, const float *, float *, int8_t *, float *, int64_t, int64_t,
+                            int64_t, hipStream_t, bool);
+}
+
+// Attention and the output projection behind it as one call.  Workspace: the merged rows (fp32, rotated basis), their
+// codes and their scales (offsets that depend on B and Hq alone), then the attention's own.
+extern "C" int64_t mi_gqa_decode_attn_linear_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T)
+{
+    const int64_t a = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T);
+    if (a < 0) return a;
+    return a + align_up(B * Hq * D * 4, 256) + align_up(B * Hq * D, 256) + align_up(B * 4, 256);
+}
+
+extern "C" int32_t mi_gqa_decode_attn_tiled_linear_f32(const float *q, const int8_t *kq, const float *ks,
+                                                       const int8_t *vt, const float *vs, float *o_rot,
+                                                       const int8_t *qw, const float *sw, float *y, int64_t B,
+                                                       int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
+                                                       const int32_t *seq_len, int64_t T_max, int64_t N,
+                                                       void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!qw || !sw || !y || !workspace || N <= 0 || N % 16) return MI_EINVAL;
+    if (!aligned16(qw) || !aligned16(sw) || !aligned16(y) || !aligned16(workspace) || (o_rot && !aligned16(o_rot)))
+        return MI_EINVAL;
+    if (Hq > 64) return MI_ERANGE;
+    const int64_t attn_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max);
+    if (attn_bytes < 0) return (int32_t)attn_bytes;
+    if (workspace_bytes < mi_gqa_decode_attn_linear_workspace_bytes(B, Hq, Hkv, D, T_max)) return MI_ENOSPC;
+    const int64_t K = Hq * D;
+    char *base = static_cast<char *>(workspace);
+    float *row = reinterpret_cast<float *>(base);
+    int8_t *oq = reinterpret_cast<int8_t *>(base + align_up(B * K * 4, 256));
+    float *oscale = reinterpret_cast<float *>(reinterpret_cast<char *>(oq) + align_up(B * K, 256));
+    void *attn_ws = reinterpret_cast<char *>(oscale) + align_up(B * 4, 256);
+    hipStream_t s = as_stream(stream);
+    if (B == 1 && (K == 2048 || K == 4096)) {
+        // One token: merging its Hq rows AND quantizing them in one workgroup makes that workgroup read every split's
+        // partials (Hq x splits x 512 B, half a megabyte at 32 splits) through one compute unit.  Here the merge runs
+        // over many workgroups and leaves the fp32 row; the projection's GEMV quantizes it in its own prologue
+        // (the same row quantizer on the same values: identical codes, scale and y).
+        float *orow = o_rot ? o_rot : row;
+        int32_t rc = run_tiled(q, kq, ks, vt, vs, orow, nullptr, nullptr, B, Hq, Hkv, D, T_cap, seq_len, T_max, 1, attn_ws,
+                               attn_bytes, s);
+        if (rc) return rc;
+        return launch_linear_fused(orow, qw, sw, y, oq, oscale, 1, N, K, s, false);
+    }
+    int32_t rc = run_tiled(q, kq, ks, vt, vs, o_rot, oq, oscale, B, Hq, Hkv, D, T_cap, seq_len, T_max, 1, attn_ws,
+                           attn_bytes, s);
+    if (rc) return rc;
+    return mi_w8a8_gemm_dequant_f32(oq, oscale, qw, sw, y, B, N, K, stream);
+}
+
 extern "C" int32_t mi_kv_tiled_from_rows_i8(const int8_t *kq, const int8_t *vq, int8_t *kt, int8_t *vt, int64_t rows,
                                             int64_t T, int64_t src_stride, int64_t T_cap, void *stream)
 {

@@ -13,7 +13,7 @@ int32_t launch_tiled(const int8_t *, const float *, const int8_t *, const float 
                      int64_t, int64_t, hipStream_t);
 
 int32_t launch_linear_fused(const float *, const int8_t *, const float *, float *, int8_t *, float *, int64_t, int64_t,
-                            int64_t, hipStream_t);
+                            int64_t, hipStream_t, bool);
 int32_t launch_norm_linear_fused(const float *, const float *, const float *, float, float *, float *, const int8_t *,
                                  const float *, float *, int8_t *, float *, int64_t, int64_t, int64_t, hipStream_t);
 
@@ -135,7 +135,7 @@ static int32_t linear_with(const float *x, const int8_t *qw, const float *sw, fl
     if (!x || !sw || !aligned16(sw)) return MI_EINVAL;
     if (M == 1 && block == 128 && aligned16(x)) {
         // decode: one kernel that quantizes its own activations (MI_EINVAL = shape not covered)
-        rc = launch_linear_fused(x, qw, sw, y, qx, sx, M, N, K, as_stream(stream));
+        rc = launch_linear_fused(x, qw, sw, y, qx, sx, M, N, K, as_stream(stream), true);
         if (rc != MI_EINVAL) return rc;
     }
     rc = mi_fwht_quant_f32_i8(x, qx, sx, M, K, block, stream);

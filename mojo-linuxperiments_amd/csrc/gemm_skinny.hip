@@ -28,6 +28,7 @@
 //  the main loop, only vmcnt / lgkmcnt waits, and several stages stay in
 //  flight per wave.  Waves of a workgroup split K; their partial accumulators
 //  meet in LDS at the end.
+#include <algorithm>
 #include "common.h"
 #include "fwht_core.h"
 
@@ -151,10 +152,11 @@ __global__ __launch_bounds__(256) void k_gemv_reg(const int8_t *__restrict__ qx,
     }
 }
 
-// k_gemv_fused: k_gemv_reg with the rotate + quantize prologue inside.  The weight loads of every wave
-// go out first; while they are in flight the workgroup rotates and quantizes the M activation rows (the same
-// per-chunk code as the stand-alone quantizer, so the codes and scales are bit-identical), parks the codes in
-// LDS and every lane picks up its share.  One launch per linear instead of two.
+// k_gemv_fused: k_gemv_reg with the rotate + quantize prologue inside.  The row's own loads go out first and the
+// first group's weight loads right behind them; while the weights are in flight the workgroup rotates and quantizes
+// the M activation rows (the same per-chunk code as the stand-alone quantizer, so the codes and scales are
+// bit-identical), parks the codes in LDS and every lane picks up its share.  One launch per linear instead of two.
+// ROT = false: the row arrives in the rotated basis and is only quantized.
 // NORM: the row is first normalized, v = ((x (+ res)) * r) * g with r = 1 / sqrt(mean((x + res)^2) + eps), the
 // arithmetic of the stand-alone RMSNorm + quantize kernel; workgroup 0 also leaves the residual sum (h_out) and, on
 // request, the normalized row (xn_out) for the caller.
@@ -164,7 +166,7 @@ struct FusedNorm {
     float eps;
 };
 
-template <int MB, int CW, int CQ, bool NORM>
+template <int MB, int CW, int CQ, bool NORM, bool ROT>
 __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x, const int8_t *__restrict__ qw,
                                                     const float *__restrict__ sw, float *__restrict__ y,
                                                     int8_t *__restrict__ qx_out, float *__restrict__ sx_out, int M,
@@ -181,18 +183,29 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = wave % QW;                  // which CW-chunk slice of the row
     const int rows_per_wg = (4 / QW) * R;
-    const int row0 = blockIdx.x * rows_per_wg + (wave / QW) * R;
+    // the workgroup owns a run of consecutive groups of rows_per_wg weight rows (the groups dealt out evenly over
+    // the grid): one prologue serves them all
+    const int ngroups = (N + rows_per_wg - 1) / rows_per_wg;
+    const int g0 = (int)((int64_t)ngroups * blockIdx.x / gridDim.x);
+    const int g1 = (int)((int64_t)ngroups * (blockIdx.x + 1) / gridDim.x);
     const int kbase = q * CW * 1024 + lane * 16;
 
+    auto load_w = [&](v4i (&w)[R][CW], int g) {
+        const int row0 = g * rows_per_wg + (wave / QW) * R;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < CW; ++c) {
+                const int off = kbase + c * 1024;
+                w[r][c] = (row0 + r < N && off < K) ? *reinterpret_cast<const v4i *>(qw + (int64_t)(row0 + r) * K + off)
+                                                    : (v4i){0, 0, 0, 0};
+            }
+    };
+    // Loads return in the order they were issued: the first row's own loads (activations, residual, gain) go out
+    // BEFORE the first group's weights, so that the prologue's arithmetic runs while the weights are on their way
+    // (issued behind them, the row would arrive only after 64 KB of weights per workgroup, and nothing would be in
+    // flight while the prologue computes).
     v4i w[R][CW];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int c = 0; c < CW; ++c) {
-            const int off = kbase + c * 1024;
-            w[r][c] = (row0 + r < N && off < K) ? *reinterpret_cast<const v4i *>(qw + (int64_t)(row0 + r) * K + off)
-                                                : (v4i){0, 0, 0, 0};
-        }
 
     // rotate + quantize, one row at a time: thread t owns chunks t, t + 256, ... of the row
     const int j = tid % LPB;
@@ -216,18 +229,31 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
             }
         }
         const bool keeper = blockIdx.x == 0;   // one workgroup also leaves the codes and scales in the caller's workspace
+        if constexpr (!NORM) {
+            if (m == 0) load_w(w, g0);
+        }
         if constexpr (NORM) {
-            float4 gl[CQ], gh[CQ];
+            float4 gl[CQ], gh[CQ], rl_[CQ], rh_[CQ];
             float ss[CQ];   // per chunk, then per group of 64 chunks (group wave + 4 * i): the order of fwht_core.h
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
-                ss[i] = 0.0f;
                 if (tid + i * 256 < nchunk) {
                     gl[i] = *reinterpret_cast<const float4 *>(nm.g + base[i]);
                     gh[i] = *reinterpret_cast<const float4 *>(nm.g + base[i] + BLOCK / 2);
                     if (nm.res) {
                         const float *rr = nm.res + (int64_t)m * K + base[i];
-                        const float4 rl = *reinterpret_cast<const float4 *>(rr), rh = *reinterpret_cast<const float4 *>(rr + BLOCK / 2);
+                        rl_[i] = *reinterpret_cast<const float4 *>(rr);
+                        rh_[i] = *reinterpret_cast<const float4 *>(rr + BLOCK / 2);
+                    }
+                }
+            }
+            if (m == 0) load_w(w, g0);
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                ss[i] = 0.0f;
+                if (tid + i * 256 < nchunk) {
+                    if (nm.res) {
+                        const float4 rl = rl_[i], rh = rh_[i];
                         v[i][0] = v[i][0] + rl.x; v[i][1] = v[i][1] + rl.y; v[i][2] = v[i][2] + rl.z; v[i][3] = v[i][3] + rl.w;
                         v[i][4] = v[i][4] + rh.x; v[i][5] = v[i][5] + rh.y; v[i][6] = v[i][6] + rh.z; v[i][7] = v[i][7] + rh.w;
                         if (keeper) {
@@ -267,7 +293,7 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < CQ; ++i) {
-            fwht_chunk<BLOCK>(v[i], j);
+            if constexpr (ROT) fwht_chunk<BLOCK>(v[i], j);   // !ROT: the row arrives in the rotated basis
             amax = fmaxf(amax, abs8(v[i]));
         }
 #pragma unroll
@@ -306,42 +332,56 @@ __global__ __launch_bounds__(256) void k_gemv_fused(const float *__restrict__ x,
             const int ms = m < M ? m : M - 1;
             xr[m][c] = off < K ? *reinterpret_cast<const v4i *>(s_x + (size_t)ms * K + off) : (v4i){0, 0, 0, 0};
         }
-    int p[V];
-#pragma unroll
-    for (int i = 0; i < V; ++i) p[i] = 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int m = 0; m < MB; ++m) {
-            int a = 0;
-#pragma unroll
-            for (int c = 0; c < CW; ++c) {
-                a = __builtin_amdgcn_sdot4(w[r][c][0], xr[m][c][0], a, false);
-                a = __builtin_amdgcn_sdot4(w[r][c][1], xr[m][c][1], a, false);
-                a = __builtin_amdgcn_sdot4(w[r][c][2], xr[m][c][2], a, false);
-                a = __builtin_amdgcn_sdot4(w[r][c][3], xr[m][c][3], a, false);
-            }
-            p[r * MB + m] = a;
-        }
-    fold_sum<V, 32>(p, lane);
     constexpr int SH = 6 - __builtin_ctz(V);
     const int vi = lane >> SH;
     const bool speaker = (lane & ((1 << SH) - 1)) == 0;
-    int total = p[0];
-    if (QW > 1) {
-        if (speaker) s_red[wave * V + vi] = total;
-        __syncthreads();
-        if (q == 0 && speaker) {
-            for (int o = 1; o < QW; ++o) total += s_red[(wave + o) * V + vi];
+#pragma unroll 1
+    for (int g = g0; g < g1; ++g) {
+        // the next group's weight loads go out before this group's arithmetic
+        v4i wn[R][CW];
+        const bool more = g + 1 < g1;   // the same for every thread of the workgroup
+        if (more) load_w(wn, g + 1);
+        int p[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) p[i] = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                int a = 0;
+#pragma unroll
+                for (int c = 0; c < CW; ++c) {
+                    a = __builtin_amdgcn_sdot4(w[r][c][0], xr[m][c][0], a, false);
+                    a = __builtin_amdgcn_sdot4(w[r][c][1], xr[m][c][1], a, false);
+                    a = __builtin_amdgcn_sdot4(w[r][c][2], xr[m][c][2], a, false);
+                    a = __builtin_amdgcn_sdot4(w[r][c][3], xr[m][c][3], a, false);
+                }
+                p[r * MB + m] = a;
+            }
+        fold_sum<V, 32>(p, lane);
+        int total = p[0];
+        if (QW > 1) {
+            if (speaker) s_red[wave * V + vi] = total;
+            __syncthreads();
+            if (q == 0 && speaker) {
+                for (int o = 1; o < QW; ++o) total += s_red[(wave + o) * V + vi];
+            }
+            __syncthreads();   // s_red is free for the next group
         }
-    }
-    if (q == 0 && speaker && vi < R * MB) {
-        const int r = vi / MB, m = vi % MB, n = row0 + r;
-        if (n < N && m < M) y[(int64_t)m * N + n] = ((float)total * s_scale[m]) * sw[n];
+        if (q == 0 && speaker && vi < R * MB) {
+            const int r = vi / MB, m = vi % MB, n = g * rows_per_wg + (wave / QW) * R + r;
+            if (n < N && m < M) y[(int64_t)m * N + n] = ((float)total * s_scale[m]) * sw[n];
+        }
+        if (more) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int c = 0; c < CW; ++c) w[r][c] = wn[r][c];
+        }
     }
 }
 
-template <int MB, int CW, int CQ, bool NORM>
+template <int MB, int CW, int CQ, bool NORM, bool ROT = true>
 static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx, int M,
                             int N, int K, int QW, const FusedNorm &nm, hipStream_t s)
 {
@@ -350,30 +390,40 @@ static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, f
     const size_t lds = (size_t)MB * K + (MB + 4 + 4 * CQ) * sizeof(float) + 4 * V * sizeof(int);
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ, NORM>),
+        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ, NORM, ROT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
         attr_set = true;
     }
+    // Every workgroup reads the whole activation row (with the norm: the residual and the gain too, 48 KB at
+    // K = 4096) before its first dot product.  Beyond two workgroups per compute unit a workgroup therefore takes
+    // several groups of rows in turn, the next group's weights on their way while it works on the current one.
     const int rows_per_wg = (4 / QW) * R;
-    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
-    hipLaunchKernelGGL((k_gemv_fused<MB, CW, CQ, NORM>), dim3(grid), dim3(256), lds, s, x, qw, sw, y, qx, sx, M, N, K,
-                       QW, nm);
+    const int ngroups = (N + rows_per_wg - 1) / rows_per_wg;
+    const unsigned grid = (unsigned)std::min(ngroups, 2 * compute_units());   // three per unit measured the same
+    hipLaunchKernelGGL((k_gemv_fused<MB, CW, CQ, NORM, ROT>), dim3(grid), dim3(256), lds, s, x, qw, sw, y, qx, sx, M, N,
+                       K, QW, nm);
     return launch_status();
 }
 
 // The fused decode linear is taken for one token and K <= 4096 only (MI_EINVAL tells the caller to take the
 // two-kernel path).  Measured: 9.3 against 10.6 us for 4096 -> 6144 at M = 1, but every workgroup repeats the
 // quantization, which at M = 4 or K = 14336 costs more than the launch it saves (15.6 against 11.7 us, 20.8
-// against 18.8 us).
+// against 18.8 us).  rotate = false: x is already in the rotated basis (the attention output as the merge leaves
+// it) and is only quantized.
 int32_t launch_linear_fused(const float *x, const int8_t *qw, const float *sw, float *y, int8_t *qx, float *sx,
-                            int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
+                            int64_t M64, int64_t N64, int64_t K64, hipStream_t s, bool rotate)
 {
     const int M = (int)M64, N = (int)N64, K = (int)K64;
     if (M != 1 || K % 1024) return MI_EINVAL;
     const int nchunk = K >> 10;
     const FusedNorm none = {nullptr, nullptr, nullptr, nullptr, 0.0f};
-    if (nchunk == 4) return launch_fused<1, 4, 2, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 4096
-    if (nchunk == 2) return launch_fused<1, 2, 1, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 2048
+    if (rotate) {
+        if (nchunk == 4) return launch_fused<1, 4, 2, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 4096
+        if (nchunk == 2) return launch_fused<1, 2, 1, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);   // K = 2048
+    } else {
+        if (nchunk == 4) return launch_fused<1, 4, 2, false, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);
+        if (nchunk == 2) return launch_fused<1, 2, 1, false, false>(x, qw, sw, y, qx, sx, M, N, K, 1, none, s);
+    }
     return MI_EINVAL;
 }
 

@@ -220,7 +220,8 @@ struct KvCache {
     {
         B = b; Hq = hq; Hkv = hkv; T_cap = t_cap; tiled = use_tiled_layouts;
         if (tiled && T_cap % 64) return false;
-        workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap);
+        // sized for attend_project: the largest of the attend calls' workspaces
+        workspace_bytes = mi_gqa_decode_attn_linear_workspace_bytes(B, Hq, Hkv, D, T_cap);
         if (workspace_bytes <= 0) return false;
         kq = arena.template alloc<int8_t>(B * Hkv * T_cap * D);
         vq = arena.template alloc<int8_t>(B * Hkv * T_cap * D);
@@ -266,6 +267,15 @@ struct KvCache {
                                                          t_max, workspace, workspace_bytes, stream)
                      : mi_gqa_decode_attn_cache_quant_i8(q, kq, ks, vq, vs, o_rot, oq, oscale, B, Hq, Hkv, D, T_cap, seq_len,
                                                          t_max, workspace, workspace_bytes, stream);
+    }
+    // attention and the output projection behind it (prepared weights qw [N, Hq*128], sw [N]) as one call: y fp32 [B, N].
+    // Tiled layouts only; o_rot (optional) receives the merged rows.
+    int32_t attend_project(const float *q, float *o_rot, const int8_t *qw, const float *sw, float *y, int64_t N,
+                           const int32_t *seq_len, int64_t t_max, void *stream) const
+    {
+        if (!tiled) return MI_EINVAL;
+        return mi_gqa_decode_attn_tiled_linear_f32(q, kq, ks, vq, vs, o_rot, qw, sw, y, B, Hq, Hkv, D, T_cap, seq_len, t_max,
+                                                   N, workspace, workspace_bytes, stream);
     }
     // a cache quantized in one go (prefill): row-major codes [B*Hkv, T, 128] (rows src_stride tokens apart) into this
     // cache's layout, first T tokens of every row; the scales are the caller's to copy into ks / vs
@@ -420,8 +430,12 @@ struct DecoderLayer {
                                            qkv.N, H, 128, qkv.workspace, qkv.workspace_bytes, stream);
         const float *xin = residual ? h0 : x;
         if (rc == MI_OK) rc = cache.rope_append(qkv_out, (Hq + 2 * Hkv) * 128, rope_cos, rope_sin, q, pos, stream);
-        if (rc == MI_OK) rc = cache.attend_quant(q, att, ca, sa, seq_len, t_max, stream);
-        if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
+        if (cache.tiled) {
+            if (rc == MI_OK) rc = cache.attend_project(q, att, o.qw, o.sw, ao, H, seq_len, t_max, stream);
+        } else {
+            if (rc == MI_OK) rc = cache.attend_quant(q, att, ca, sa, seq_len, t_max, stream);
+            if (rc == MI_OK) rc = mi_w8a8_gemm_dequant_f32(ca, sa, o.qw, o.sw, ao, B, H, Hq * 128, stream);
+        }
         if (moe) {
             if (rc == MI_OK) rc = mi_rmsnorm_f32(ao, xin, g2, eps, h1, hn, B, H, stream);
             if (rc == MI_OK) rc = moe->forward(hn, dn, stream);

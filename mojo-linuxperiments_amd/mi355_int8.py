@@ -106,6 +106,9 @@ SIGNATURES = {
     "mi_kv_append_paged_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, vp]),
     "mi_kv_append_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_gqa_decode_attn_tiled": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64, vp]),
+    "mi_gqa_decode_attn_linear_workspace_bytes": (i64, [i64, i64, i64, i64, i64]),
+    "mi_gqa_decode_attn_tiled_linear_f32": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i64,
+                                                  vp, i64, vp]),
     "mi_gqa_decode_attn_tiled_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, vp, i64,
                                              vp]),
     "mi_kv_tiled_from_rows_i8": (i32, [vp, vp, vp, vp, i64, i64, i64, i64, vp]),
@@ -466,7 +469,13 @@ class DecoderLayer:
         self.act = dev.empty((B, I), f) if trace else None
         self.lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(B, max(2 * I, self.NQKV), H), np.uint8)   # codes of the normalized rows
         self.ci, self.si = dev.empty((B, I), np.int8), dev.empty(B, f)        # codes of the activated rows
-        self.att_ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
+        self.att_ws = dev.empty(lib.mi_gqa_decode_attn_linear_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
+        if self.tiled:
+            # the one-call attention + projection leaves the codes and scales of the attention rows in its workspace
+            up = lambda v: (v + 255) // 256 * 256
+            off = up(B * Hq * D * 4)
+            self.ca = DevBuf(self.att_ws.ptr + off, (B, Hq * D), np.int8)
+            self.sa = DevBuf(self.att_ws.ptr + off + up(B * Hq * D), (B,), f)
 
     def step(self, x, pos, seq_len, t_max, out, stream=None, residual=None):
         """x fp32 [B,H] (+ residual fp32 [B,H]: the layer input is their sum, left in self.h0); pos, seq_len int32
@@ -485,11 +494,18 @@ class DecoderLayer:
                      self.vq.ptr, self.vs.ptr, pos.ptr, B, Hq, Hkv, D, self.T_cap, s), "mi_rope_kv_append")
         # attention output stays in the rotated basis of V and is quantized by the merge itself: the O weights were
         # rotated with block 128 = head_dim along K, so their GEMV takes these codes as they are
-        attend = lib.mi_gqa_decode_attn_tiled_quant_i8 if self.tiled else lib.mi_gqa_decode_attn_cache_quant_i8
-        check(attend(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr, p(self.att), self.ca.ptr,
-                     self.sa.ptr, B, Hq, Hkv, D, self.T_cap, seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
-              "mi_gqa_decode_attn_quant_i8")
-        gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
+        if self.tiled:
+            # attention and the O projection as one call (for one token the projection's GEMV quantizes the merged row)
+            check(lib.mi_gqa_decode_attn_tiled_linear_f32(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
+                                                          p(self.att), self.wo[0].ptr, self.wo[1].ptr, self.ao.ptr, B, Hq,
+                                                          Hkv, D, self.T_cap, seq_len.ptr, t_max, H, self.att_ws.ptr,
+                                                          self.att_ws.nbytes, s), "mi_gqa_decode_attn_tiled_linear_f32")
+        else:
+            check(lib.mi_gqa_decode_attn_cache_quant_i8(self.q.ptr, self.kq.ptr, self.ks.ptr, self.vq.ptr, self.vs.ptr,
+                                                        p(self.att), self.ca.ptr, self.sa.ptr, B, Hq, Hkv, D, self.T_cap,
+                                                        seq_len.ptr, t_max, self.att_ws.ptr, self.att_ws.nbytes, s),
+                  "mi_gqa_decode_attn_cache_quant_i8")
+            gemm_dequant(self.ca, self.sa, self.wo[0], self.wo[1], self.ao, s)
         if self.moe is None:
             check(lib.mi_rmsnorm_linear_f32(self.ao.ptr, xin.ptr, self.g2.ptr, self.eps, self.h1.ptr, p(self.hn),
                                             self.wgu[0].ptr, self.wgu[1].ptr, self.gu.ptr, B, 2 * I, H, self.block,

@@ -76,6 +76,7 @@ def make_cache(mi, dev, seed, B, Hq, Hkv, T, T_cap):
 @pytest.mark.parametrize("B,Hq,Hkv,T,T_cap", [
     (2, 8, 2, 256, 256), (1, 4, 1, 16, 64), (1, 32, 8, 1000, 1024), (3, 6, 3, 77, 128), (2, 4, 4, 130, 192),
     (1, 8, 2, 1, 64), (1, 8, 2, 4096, 4096), (16, 32, 8, 700, 1024), (2, 8, 8, 64, 64),
+    (1, 32, 8, 2000, 2048), (2, 16, 4, 1500, 1536),     # 32 and 24 splits: the merge with 32 lanes per row
 ])
 def test_vt_attention_matches_oracle(mi, dev, orc, B, Hq, Hkv, T, T_cap):
     mark = dev.mark()
@@ -236,3 +237,45 @@ def test_vt_append_matches_row_major_append(mi, dev, orc):
         assert np.array_equal(vt, want_v)
         assert np.array_equal(kt, want_k)
     dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T_cap,N", [(1, 32, 8, 4096, 4096), (1, 16, 4, 1024, 2048), (1, 32, 8, 64, 6144),
+                                               (1, 8, 2, 256, 1024), (3, 32, 8, 512, 4096), (16, 32, 8, 256, 4096)])
+def test_vt_attention_with_projection_is_the_two_calls(mi, dev, B, Hq, Hkv, T_cap, N):
+    """mi_gqa_decode_attn_tiled_linear_f32 = mi_gqa_decode_attn_tiled_quant_i8 + mi_w8a8_gemm_dequant_f32, bit for bit,
+    also where it divides the work differently (one token with 2048 or 4096 attention values: merge over many
+    workgroups, quantizer inside the projection's GEMV); ragged lengths; the merged row comes back on request."""
+    lib = mi.lib
+    mark = dev.mark()
+    D, K = 128, Hq * 128
+    lens = np.array([T_cap, 1, 77, T_cap - 3] * 4, np.int32)[:B]
+    q, kq, ks, vq, vs, _, _ = make_cache(mi, dev, 23 + B, B, Hq, Hkv, T_cap, T_cap)
+    dkt, dvt = convert(mi, dev, kq, vq, T_cap, T_cap)
+    dq, dks, dvs, dl = dev.upload(q), dev.upload(ks), dev.upload(vs), dev.upload(lens)
+    w = workload.normal(5, (N, K), 3)
+    dqw, dsw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+    mi.fwht_quant(dev.upload(w), dqw, dsw, 128)
+    # the two calls
+    ws = dev.empty(lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_cap), np.uint8)
+    orot, oq, osc = dev.empty((B, Hq, D), np.float32), dev.empty((B, K), np.int8), dev.empty(B, np.float32)
+    y0 = dev.empty((B, N), np.float32)
+    mi.check(lib.mi_gqa_decode_attn_tiled_quant_i8(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, orot.ptr, oq.ptr, osc.ptr, B,
+                                                   Hq, Hkv, D, T_cap, dl.ptr, T_cap, ws.ptr, ws.nbytes, None))
+    mi.check(lib.mi_w8a8_gemm_dequant_f32(oq.ptr, osc.ptr, dqw.ptr, dsw.ptr, y0.ptr, B, N, K, None))
+    # the one call, with and without the merged row
+    need = lib.mi_gqa_decode_attn_linear_workspace_bytes(B, Hq, Hkv, D, T_cap)
+    assert need > ws.nbytes
+    ws2 = dev.upload(np.full(need, 0xA5, np.uint8))
+    orot2, y1, y2 = dev.empty((B, Hq, D), np.float32), dev.empty((B, N), np.float32), dev.empty((B, N), np.float32)
+    args = (dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr)
+    tail = (B, Hq, Hkv, D, T_cap, dl.ptr, T_cap, N, ws2.ptr, ws2.nbytes, None)
+    mi.check(lib.mi_gqa_decode_attn_tiled_linear_f32(*args, orot2.ptr, dqw.ptr, dsw.ptr, y1.ptr, *tail))
+    mi.check(lib.mi_gqa_decode_attn_tiled_linear_f32(*args, None, dqw.ptr, dsw.ptr, y2.ptr, *tail))
+    a, b, c = dev.download(y0), dev.download(y1), dev.download(y2)
+    r0, r1 = dev.download(orot), dev.download(orot2)
+    assert lib.mi_gqa_decode_attn_tiled_linear_f32(*args, None, dqw.ptr, dsw.ptr, y2.ptr, B, Hq, Hkv, D, T_cap, dl.ptr, T_cap,
+                                                   N, ws2.ptr, need - 256, None) == mi.ENOSPC
+    dev.reset_to(mark)
+    assert np.isfinite(a).all() and np.abs(a).max() > 0
+    assert np.array_equal(r0, r1)
+    assert np.array_equal(a, b) and np.array_equal(a, c)
