@@ -109,6 +109,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true",
                     help="launch everything eagerly: for runs under rocprofv3's kernel trace, whose tool library "
                          "ended in a segmentation fault inside hipGraphLaunch; the line then says method: eager")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="context only: the vendor library's int8 GEMM (torch._int_mm, int32 out) beside this "
+                         "library's on the cfg3 shapes, same codes, same sustained clock state; one JSON line")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -123,6 +126,8 @@ def main():
 
     if args.pmc_probe:
         return pmc_probe(mi, wl)
+    if args.vendor_gemm:
+        return vendor_gemm(mi, wl)
     if args.decode_stack:
         dev = mi.Device(arena_bytes=(2 << 30) + args.decode_stack * (400 << 20))
         pool = mi.StreamPool(dev, 1)
@@ -511,6 +516,95 @@ def moe_layer(mi, wl, dev, s, timer, reps=20, graph=True):
                                "hbm_frac": round(wbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                "TOPS": round(ops / (ms * 1e-3) / 1e12, 2),
                                "tokens_per_s": round(T / (ms * 1e-3), 1), "weight_bytes": wbytes}}
+
+
+VENDOR_CHILD = r"""
+import json, os, sys
+import numpy as np, torch
+tmp, ncopy, warm = sys.argv[1], int(sys.argv[2]), int(sys.argv[3])
+a = torch.from_numpy(np.load(os.path.join(tmp, "x.npy"))).cuda()
+wh = np.load(os.path.join(tmp, "w.npy"))
+ws = [torch.from_numpy(wh).cuda().t() for _ in range(ncopy)]   # [K, N] views of row-major [N, K]: A . B^T
+for i in range(warm):
+    torch._int_mm(a, ws[i % ncopy])
+torch.cuda.synchronize()
+e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+e0.record()
+for i in range(40):
+    torch._int_mm(a, ws[i % ncopy])
+e1.record()
+torch.cuda.synchronize()
+np.save(os.path.join(tmp, "acc.npy"), torch._int_mm(a, ws[0]).cpu().numpy())
+print(json.dumps({"us": round(e0.elapsed_time(e1) / 40 * 1e3, 2)}))
+"""
+
+
+def vendor_gemm(mi, wl):
+    """Context, not a target: torch._int_mm (hipBLASLt underneath) on the cfg3 shapes with the codes this library's
+    own quantizer produces from the benchmark's activations and weights, timed like the headline (HIP events on the
+    launch stream, about 60 ms of the same launches first, weights rotated through more than 256 MB)."""
+    import subprocess
+    import tempfile
+    lib = mi.lib
+    dev = mi.Device(arena_bytes=6 << 30)
+    pool = mi.StreamPool(dev, 1)
+    s = pool.stream(0)
+    timer = Timer(mi, s)
+    M = wl.PREFILL_M
+    out = {}
+    for name, K, N in (("qkv", 4096, 6144), ("gate_up", 4096, 14336), ("down", 14336, 4096)):
+        mark = dev.mark()
+        a = dev.upload(wl.activations(2025, M, K, stream=K))
+        qx, sx = dev.empty((M, K), np.int8), dev.empty(M, np.float32)
+        mi.fwht_quant(a, qx, sx, wl.HADAMARD_BLOCK)
+        w = dev.upload(wl.weights(2025, N, K, stream=K + N))
+        qw, sw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+        mi.fwht_quant(w, qw, sw, wl.HADAMARD_BLOCK)
+        dev.sync()
+        xh, wh = dev.download(qx), dev.download(qw)
+        ncopy = MALL_BYTES // (N * K) + 2
+        qws = [dev.upload(wh) for _ in range(ncopy)]
+        acc = dev.empty((M, N), np.int32)
+        y = dev.empty((M, N), np.float32)
+        state = {"i": 0}
+
+        def ours_i32():
+            state["i"] = (state["i"] + 1) % ncopy
+            mi.check(lib.mi_w8a8_gemm_i32(qx.ptr, qws[state["i"]].ptr, acc.ptr, M, N, K, s))
+
+        def ours_f32():
+            state["i"] = (state["i"] + 1) % ncopy
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qws[state["i"]].ptr, sw.ptr, y.ptr, M, N, K, s))
+        res = {}
+        for tag, fn in (("this_library_dequant_f32_us", ours_f32), ("this_library_i32_us", ours_i32)):
+            timer.settle(fn, 150.0)
+            res[tag] = round(timer.run(fn, 40) * 1e3, 2)
+        # torch brings its own HIP runtime, which finds no device once this library's runtime holds it: a child
+        # process times the vendor GEMM on the same codes and hands back its accumulators' checksum
+        mi.check(lib.mi_w8a8_gemm_i32(qx.ptr, qws[0].ptr, acc.ptr, M, N, K, s))
+        dev.sync(s)
+        ours = dev.download(acc)
+        with tempfile.TemporaryDirectory() as tmp:
+            np.save(os.path.join(tmp, "x.npy"), xh)
+            np.save(os.path.join(tmp, "w.npy"), wh)
+            warm = max(3, int(150e3 / max(res["this_library_i32_us"], 1.0)))
+            child = subprocess.run([sys.executable, "-c", VENDOR_CHILD, tmp, str(ncopy), str(warm)],
+                                   capture_output=True, text=True, timeout=600)
+            if child.returncode != 0:
+                raise SystemExit("vendor GEMM child failed:\n" + child.stderr[-2000:])
+            got = json.loads(child.stdout.strip().splitlines()[-1])
+            ref = np.load(os.path.join(tmp, "acc.npy"))
+        res["torch_int_mm_i32_us"] = got["us"]
+        res["accumulators_equal"] = bool(np.array_equal(ref, ours))
+        ops = 2.0 * M * N * K
+        res["this_library_i32_frac_of_peak"] = round(ops / res["this_library_i32_us"] / 1e6 / PEAK_INT8_TOPS, 4)
+        res["torch_int_mm_frac_of_peak"] = round(ops / res["torch_int_mm_i32_us"] / 1e6 / PEAK_INT8_TOPS, 4)
+        out[name] = res
+        dev.reset_to(mark)
+    pool.destroy()
+    dev.close()
+    print(json.dumps({"vendor_gemm_context": out, "M": M, "note": "torch._int_mm writes int32; this library's "
+                      "dequantizing form writes fp32 (the same number of bytes)"}), flush=True)
 
 
 def cfg0_linear(mi, wl, dev, s, timer, shapes):
