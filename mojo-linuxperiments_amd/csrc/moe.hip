@@ -65,6 +65,34 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
     const int t0 = blockIdx.x * 16 + wave * 4;
     const int e0 = blockIdx.y * 16;
 
+    // the token row this wave quantizes (if any) is requested first: its loads then fly under the logits' rounds
+    // instead of costing a memory round trip after them
+    constexpr int LPB = 16;
+    constexpr int CQR = CQ > 0 ? CQ : 1;
+    const int jq = lane % LPB, nchunk = H / 8;
+    const int qtt = (int)blockIdx.y * 4 + wave;                 // the workgroups of a token group deal its 16 rows
+    const int qrow = blockIdx.x * 16 + qtt;
+    const bool has_row = CQ > 0 && qtt < 16 && qrow < T;        // whole wave
+    float v[CQR][8];
+    int base[CQR];
+    if constexpr (CQ > 0) {
+        const float *xrow = x + (int64_t)min(qrow, T - 1) * H;
+#pragma unroll
+        for (int i = 0; i < CQ; ++i) {
+            const int c = lane + i * 64;
+            base[i] = (c / LPB) * 128 + 4 * jq;
+            if (has_row && c < nchunk) {
+                const float4 lo = *reinterpret_cast<const float4 *>(xrow + base[i]);
+                const float4 hi = *reinterpret_cast<const float4 *>(xrow + base[i] + 64);
+                v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
+                v[i][4] = hi.x; v[i][5] = hi.y; v[i][6] = hi.z; v[i][7] = hi.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+            }
+        }
+    }
+
     float p[64];
 #pragma unroll
     for (int i = 0; i < 64; ++i) p[i] = 0.0f;
@@ -101,19 +129,35 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
     const int t = t0 + (lane >> 4);
     if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
     if constexpr (CQ > 0) {
-        constexpr int LPB = 16;
-        const int j = lane % LPB, nchunk = H / 8;
-        for (int tt = (int)blockIdx.y * 4 + wave; tt < 16; tt += (int)gridDim.y * 4) {
+        if (has_row) {
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                fwht_chunk<128>(v[i], jq);
+                amax = fmaxf(amax, abs8(v[i]));
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            const float sc = (amax == 0.0f) ? 1.0f : amax / 127.0f;
+            const float inv = (amax == 0.0f) ? 0.0f : 127.0f / amax;
+            if (lane == 0) sx[qrow] = sc;
+            int8_t *qr = qx + (int64_t)qrow * H;
+#pragma unroll
+            for (int i = 0; i < CQ; ++i) {
+                if (lane + i * 64 < nchunk) {
+                    *reinterpret_cast<uint32_t *>(qr + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                    *reinterpret_cast<uint32_t *>(qr + base[i] + 64) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+                }
+            }
+        }
+        // fewer than four expert groups: a wave has further rows of the token group to do
+        for (int tt = qtt + (int)gridDim.y * 4; tt < 16; tt += (int)gridDim.y * 4) {
             const int row = blockIdx.x * 16 + tt;
             if (row >= T) break;   // whole wave
             const float *xrow = x + (int64_t)row * H;
-            float v[CQ][8];
-            int base[CQ];
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
-                const int c = lane + i * 64;
-                base[i] = (c / LPB) * 128 + 4 * j;
-                if (c < nchunk) {
+                if (lane + i * 64 < nchunk) {
                     const float4 lo = *reinterpret_cast<const float4 *>(xrow + base[i]);
                     const float4 hi = *reinterpret_cast<const float4 *>(xrow + base[i] + 64);
                     v[i][0] = lo.x; v[i][1] = lo.y; v[i][2] = lo.z; v[i][3] = lo.w;
@@ -126,7 +170,7 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
             float amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
-                fwht_chunk<128>(v[i], j);
+                fwht_chunk<128>(v[i], jq);
                 amax = fmaxf(amax, abs8(v[i]));
             }
 #pragma unroll
@@ -134,12 +178,12 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
             const float sc = (amax == 0.0f) ? 1.0f : amax / 127.0f;
             const float inv = (amax == 0.0f) ? 0.0f : 127.0f / amax;
             if (lane == 0) sx[row] = sc;
-            int8_t *qrow = qx + (int64_t)row * H;
+            int8_t *qr = qx + (int64_t)row * H;
 #pragma unroll
             for (int i = 0; i < CQ; ++i) {
                 if (lane + i * 64 < nchunk) {
-                    *reinterpret_cast<uint32_t *>(qrow + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
-                    *reinterpret_cast<uint32_t *>(qrow + base[i] + 64) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
+                    *reinterpret_cast<uint32_t *>(qr + base[i]) = quant4(v[i][0], v[i][1], v[i][2], v[i][3], inv);
+                    *reinterpret_cast<uint32_t *>(qr + base[i] + 64) = quant4(v[i][4], v[i][5], v[i][6], v[i][7], inv);
                 }
             }
         }
