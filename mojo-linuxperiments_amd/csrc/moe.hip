@@ -880,7 +880,7 @@ static Layout layout(int64_t T, int64_t H, int64_t I, int64_t E, int64_t topk)
 
 static int32_t check_shapes(int64_t T, int64_t H, int64_t I, int64_t E, int32_t topk)
 {
-    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return MI_EINVAL;
+    if (T < 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return MI_EINVAL;   // T == 0: an empty batch, a call that does nothing
     if (H % 128 || I % 256 || topk > MAX_TOPK || topk > E) return MI_EINVAL;
     if (H > 32768 || I > 32768 || T * topk > (1LL << 24) || E > 65535) return MI_ERANGE;
     if (2 * E * ((T + 31) / 32) + E + 1 > DISPATCH_MAX_WORDS) return MI_ERANGE;  // dispatch bitmap in LDS
@@ -994,6 +994,7 @@ static int32_t run_ffn(const float *x, const int32_t *idx, const float *w, const
         return MI_EINVAL;
     const moe::Layout L = moe::layout(T, H, I, E, topk);
     if (workspace_bytes < L.total) return MI_ENOSPC;
+    if (T == 0) return MI_OK;
     char *ws = static_cast<char *>(workspace);
     int8_t *qx = reinterpret_cast<int8_t *>(ws + L.off[0]);
     float *sx = reinterpret_cast<float *>(ws + L.off[1]);
@@ -1119,6 +1120,7 @@ extern "C" int32_t mi_moe_layer(const float *x, const float *wr, const int8_t *w
     if (!workspace || !aligned16(workspace)) return MI_EINVAL;
     const moe::Layout L = moe::layout(T, H, I, E, topk);
     if (workspace_bytes < L.total) return MI_ENOSPC;
+    if (T == 0) return MI_OK;
     char *ws = static_cast<char *>(workspace);
     int32_t *idx = reinterpret_cast<int32_t *>(ws + L.off[8]);
     float *w = reinterpret_cast<float *>(ws + L.off[9]);
