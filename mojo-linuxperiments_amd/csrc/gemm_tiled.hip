@@ -417,6 +417,11 @@ static int32_t launch_shape(const int8_t *qx, const float *sx, const int8_t *qw,
     return launch_status();
 }
 
+// gemm_pair.hip
+template <bool DEQ>
+int32_t launch_pair(int tm, int tn, const int8_t *, const float *, const int8_t *, const float *, int32_t *, float *, int,
+                    int, int, hipStream_t);
+
 template <bool DEQ>
 int32_t launch_tiled(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc, float *y,
                      int64_t M64, int64_t N64, int64_t K64, hipStream_t s)
@@ -439,6 +444,9 @@ int32_t launch_tiled(const int8_t *qx, const float *sx, const int8_t *qw, const 
         const double cost = (double)rounds * per_cu * bm * bn * eff;
         if (i == 0 || cost < best) { best = cost; pick = i; }
     }
+    // one tile per compute unit of a shape that divides evenly: two waves per SIMD on the same wave tile
+    if ((pick == 2 || pick == 3) && M % (32 * shapes[pick].tm) == 0 && N % (32 * shapes[pick].tn) == 0)
+        return launch_pair<DEQ>(shapes[pick].tm, shapes[pick].tn, qx, sx, qw, sw, acc, y, M, N, K, s);
     switch (pick) {
     case 0: return launch_shape<8, 8, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);
     case 1: return launch_shape<8, 7, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, s);

@@ -43,6 +43,30 @@ def test_tiled_accumulators_bit_exact(mi, dev, orc, M, N, K):
     assert np.array_equal(gpu_gemm_i32(mi, dev, qx, qw), orc.gemm_i8_i32(qx, qw))
 
 
+@pytest.mark.parametrize("M,N,K", [
+    # whole 256 x 192 and 128 x 256 tiles, one per compute unit: the kernel with two waves per SIMD.  K of 1 to 5
+    # stages walks every branch of its prologue and of its last stages.
+    (2048, 6144, 128), (2048, 6144, 256), (2048, 6144, 384), (2048, 6144, 512), (2048, 6144, 640),
+    (2048, 4096, 128), (2048, 4096, 256), (2048, 4096, 384), (2048, 4096, 896),
+])
+def test_paired_wave_kernel_bit_exact(mi, dev, orc, M, N, K):
+    """Every accumulator, then the dequantized form of the same product (fp32, scale by scale as the oracle does)."""
+    qx, qw = rand_codes(M + N + K, (M, K)), rand_codes(K + 9, (N, K))
+    want = orc.gemm_i8_i32(qx, qw)
+    assert np.array_equal(gpu_gemm_i32(mi, dev, qx, qw), want)
+    g = np.random.default_rng(K)
+    sx = g.uniform(0.01, 1, M).astype(np.float32)
+    sw = g.uniform(0.001, 0.1, N).astype(np.float32)
+    mark = dev.mark()
+    dy = dev.empty((M, N), np.float32)
+    mi.check(mi.lib.mi_w8a8_gemm_dequant_f32(dev.upload(qx).ptr, dev.upload(sx).ptr, dev.upload(qw).ptr,
+                                             dev.upload(sw).ptr, dy.ptr, M, N, K, None))
+    dev.sync()
+    y = dev.download(dy)
+    dev.reset_to(mark)
+    assert np.array_equal(y, orc.dequant(want, sx, sw))
+
+
 def test_extreme_codes_do_not_overflow(mi, dev):
     K = 14336
     qx = np.full((80, K), 127, np.int8)
