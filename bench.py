@@ -112,6 +112,10 @@ def main():
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="context only: the vendor library's int8 GEMM (torch._int_mm, int32 out) beside this "
                          "library's on the cfg3 shapes, same codes, same sustained clock state; one JSON line")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="context only: what a loop of v_mfma_i32_16x16x64_i8 alone sustains on this machine "
+                         "(operands in registers, with and without the GEMM's LDS fragment reads, zeros and "
+                         "activation-like codes); one JSON line")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -124,6 +128,9 @@ def main():
     import mi355_int8 as mi     # fails loudly when the HIP library is not built
     import workload as wl
 
+    if args.mfma_probe:
+        print(json.dumps(mfma_probe()), flush=True)
+        return
     if args.pmc_probe:
         return pmc_probe(mi, wl)
     if args.vendor_gemm:
@@ -147,6 +154,9 @@ def main():
         pool.destroy()
         dev.close()
         return
+
+    log("matrix-pipe probe ...")
+    probe = mfma_probe()   # a child process, finished before this process takes the device
 
     dev = mi.Device(arena_bytes=12 << 30)
     pool = mi.StreamPool(dev, 1)
@@ -255,7 +265,7 @@ def main():
         traffic = {k: v["fetch"] + v["write"] for k, v in per.items()}
         traffic_total = sum(traffic.values())
     roofline = {
-        "kernel": "k_w8a8_tiled (v_mfma_i32_16x16x64_i8), four cfg3 shapes, ops-weighted",
+        "kernel": "k_w8a8_pair (qkv, down) / k_w8a8_tiled (gate, up), v_mfma_i32_16x16x64_i8, four cfg3 shapes, ops-weighted",
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_total,
         "traffic_unit": "bytes over the four launches (fetched + written), rocprofv3 PMC, calibrated",
@@ -270,6 +280,20 @@ def main():
         "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
                            for name, K, N in wl.PROJECTIONS},
     }
+    # what the matrix pipe sustains here with nothing else in the way (power-limited clock): context for `frac`,
+    # which stays against the published peak
+    runs = (probe.get("mfma_power_limited_peak") or {}).get("runs") if probe else None
+    if runs:
+        like = [r for r in runs if r["operands"] != "zeros" and r["lds_fragment_reads"]]
+        best = max(r["tops"] for r in like)
+        roofline["sustained_mfma_measured"] = {
+            "tops": best, "frac_of_it": round(gemm_tops / best, 4),
+            "what": "a loop of the same MFMA alone with the 8 x 6 wave tile's LDS fragment reads, activation-like "
+                    "codes, best of one and two waves per SIMD, ~3 ms per run (mojo-linuxperiments_amd/mfma_peak_probe)",
+            "zeros_no_reads_tops": max(r["tops"] for r in runs if r["operands"] == "zeros" and not r["lds_fragment_reads"]),
+        }
+    else:
+        roofline["sustained_mfma_measured"] = None
 
     out = {
         "metric": "W8A8 GEMM int8 TOPS & decode GB/s (% roofline) @1 GPU; vs CPU host cores",
@@ -516,6 +540,19 @@ def moe_layer(mi, wl, dev, s, timer, reps=20, graph=True):
                                "hbm_frac": round(wbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                "TOPS": round(ops / (ms * 1e-3) / 1e12, 2),
                                "tokens_per_s": round(T / (ms * 1e-3), 1), "weight_bytes": wbytes}}
+
+
+def mfma_probe():
+    """Runs the matrix-pipe probe (its own process, csrc/probe_mfma_peak.hip) and returns its JSON, or None with
+    the reason when the executable is not built.  Context for the roofline, never part of `value`."""
+    import subprocess
+    exe = os.path.join(ROOT, "mojo-linuxperiments_amd", "mfma_peak_probe")
+    if not os.path.exists(exe):
+        return {"mfma_power_limited_peak": None, "reason": "mfma_peak_probe is not built (make -C mojo-linuxperiments_amd/csrc)"}
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    if r.returncode != 0:
+        return {"mfma_power_limited_peak": None, "reason": "probe failed: " + r.stderr.strip()[-200:]}
+    return json.loads(r.stdout.strip().splitlines()[-1])
 
 
 VENDOR_CHILD = r"""
