@@ -1,8 +1,9 @@
 // What the int8 matrix pipe of this machine sustains when nothing else limits it: a loop of
 // v_mfma_i32_16x16x64_i8 alone, operands in registers, no memory traffic inside the loop, on every SIMD of the chip,
-// for about 3 ms.  The published peak (5.0 POP/s dense) is the instruction's rate at the top clock; under a sustained
-// matrix load the clock is set by the power limit, and how far it falls depends on how many bits the operands
-// toggle.  This probe measures that ceiling, which a GEMM's roofline fraction has to be read against:
+// for about 3 ms a run, twelve runs in a row of which the last counts.  The published peak (5.0 POP/s dense) is the
+// instruction's rate at the top clock; under a sustained matrix load the clock is set by the power limit, and how
+// far it falls depends on how many bits the operands toggle.  This probe measures that ceiling, which a GEMM's
+// roofline fraction has to be read against:
 //   - one and two waves per SIMD (one wave cannot issue the instruction back to back at the pipe's full rate);
 //   - operands all zero, and int8 codes drawn like rotated, quantized activations (normal, sigma 30, clipped to 127);
 //   - with and without the LDS fragment reads of the 8 x 6 wave tile (14 ds_read_b128 to 48 matrix instructions).
@@ -94,7 +95,7 @@ static Result run(const unsigned *codes, long long *ticks, int waves_per_simd, i
     CK(hipEventCreate(&e0));
     CK(hipEventCreate(&e1));
     float ms = 0;
-    for (int rep = 0; rep < 4; ++rep) {   // the last repetition counts: the clock has settled by then
+    for (int rep = 0; rep < 12; ++rep) {   // the last repetition counts: 35 ms of the same load lie before it
         CK(hipEventRecord(e0, 0));
         hipLaunchKernelGGL(k_mfma_loop<READS>, dim3(cus), dim3(threads), 64 * 1024, 0, codes, ticks, iters);
         CK(hipEventRecord(e1, 0));
