@@ -10,7 +10,8 @@
 // kernel (16*TM x 16*TN outputs, TM*TN accumulators of four registers) and split every 128-byte K stage between
 // them: wave p (0..3) takes the first 64 bytes of each stage, wave p + 4 the second.  LDS layout, swizzle, load
 // shapes and bytes read from LDS per matrix instruction are those of the four-wave kernel; each wave issues half
-// of the stage's matrix instructions, and the two partial sums of a tile meet in LDS after the last stage.
+// of the stage's matrix instructions, and the two partial sums of a tile meet in LDS after the last stage (each wave
+// then finishes half of the row tiles).
 // The matrix pipe serves the lower-numbered wave of a SIMD first, so waves 0..3 run ahead of their partners and
 // would spend the difference at the barriers: they issue ALL loads of a stage, their partners none.
 //
@@ -326,90 +327,71 @@ __global__ __launch_bounds__(512) void k_w8a8_pair(const int8_t *__restrict__ qx
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
     __syncthreads();   // every wave is done with the stage buffers: they carry the exchange below
 
-    // ---- the two partial sums of a wave tile meet.  Wave `half` finishes column tiles j in [half*TN/2, +TN/2); it
-    // hands the other half of its accumulators to its partner through LDS, in two rounds of TM/2 row tiles so that
-    // the eight waves' parcels fit (TN/2 * TM/2 * 1 KB each), and adds the partner's parcel to its own.
-    constexpr int JH = TN / 2, IH = TM / 2;
-    constexpr int PARCEL = JH * IH * 1024;
-    static_assert(8 * PARCEL <= C::STAGES, "parcels fit the stage buffers");
-    char *const mine = smem + wave * PARCEL;
-    const char *const theirs = smem + (wave ^ 4) * PARCEL;
+    // ---- the two partial sums of a wave tile meet.  Wave `half` finishes row tiles i in [half*TM/2, +TM/2) of every
+    // column tile; it hands the other row tiles of its accumulators to its partner through LDS, one pair of column
+    // tiles a round (2 * TM/2 KB a wave; two parcel areas in turn, so one barrier a round), adds the partner's
+    // parcel to its own and stores the pair: 8 rows x 128 B per store instruction.
+    constexpr int IH = TM / 2;
+    constexpr int PARCEL = 2 * IH * 1024;
+    static_assert(2 * 8 * PARCEL <= C::STAGES, "two parcel areas fit the stage buffers");
     const bool lo = r < 8;
 
     // `half` is uniform over the wave: both forms of the exchange are compiled and a scalar branch picks one, so
     // that every accumulator register is named by a constant
-    auto finish = [&](auto HALF, auto CHECKED) {
+    auto finish = [&](auto HALF) {
         constexpr int hf = decltype(HALF)::value;
-        constexpr bool checked = decltype(CHECKED)::value;
-        float4 swP[(JH + 1) / 2];
-        if constexpr (DEQ) {
+        float sxA[IH], sxB[IH];
 #pragma unroll
-            for (int jj = 0; jj < JH; jj += 2)
-                swP[jj / 2] = *reinterpret_cast<const float4 *>(s_sw + (wn * TN + hf * JH + jj) * 16 +
-                                                                ((!lo && jj + 1 < JH) ? 16 : 0) + 4 * g_);
+        for (int ii = 0; ii < IH; ++ii) {
+            sxA[ii] = sxB[ii] = 1.0f;
+            if constexpr (DEQ) {
+                const float *tsx = s_sx + (wm * TM + hf * IH + ii) * 16;
+                sxA[ii] = tsx[r & 7];
+                sxB[ii] = tsx[8 + (r & 7)];
+            }
         }
-        static_for<2>([&](auto RD) {
+        static_for<TN / 2>([&](auto RD) {
             constexpr int rd = decltype(RD)::value;
-            if constexpr (rd > 0) __syncthreads();   // the parcels of the round before have been read
-            // hand over the accumulators of the partner's column tiles, row tiles of this round
-            static_for<JH>([&](auto JJ) {
+            char *const mine = smem + ((rd & 1) * 8 + wave) * PARCEL;
+            const char *const theirs = smem + ((rd & 1) * 8 + (wave ^ 4)) * PARCEL;
+            // hand over: column tiles 2rd, 2rd+1, the partner's row tiles
+            static_for<2>([&](auto JJ) {
                 static_for<IH>([&](auto II) {
                     constexpr int jj = decltype(JJ)::value, ii = decltype(II)::value;
-                    constexpr int i = rd * IH + ii, j = (1 - hf) * JH + jj;
+                    constexpr int i = (1 - hf) * IH + ii, j = 2 * rd + jj;
                     *reinterpret_cast<v4i *>(mine + (jj * IH + ii) * 1024 + lane * 16) = acc_read4<4 * (j * TM + i)>();
                 });
             });
             __syncthreads();
+            float4 sw4 = {1.0f, 1.0f, 1.0f, 1.0f};
+            if constexpr (DEQ) sw4 = *reinterpret_cast<const float4 *>(s_sw + (wn * TN + 2 * rd) * 16 + (lo ? 0 : 16) + 4 * g_);
+            const int n = n0 + (wn * TN + 2 * rd) * 16 + (lo ? 0 : 16) + 4 * g_;
             // take over, add, store
             static_for<IH>([&](auto II) {
                 constexpr int ii = decltype(II)::value;
-                constexpr int i = rd * IH + ii;
+                constexpr int i = hf * IH + ii;
                 const int mrow = m0 + (wm * TM + i) * 16;
                 const int mA = mrow + (r & 7), mB = mrow + 8 + (r & 7);
-                float sxA = 1.0f, sxB = 1.0f, sxO = 1.0f;
-                if constexpr (DEQ) {
-                    const float *tsx = s_sx + (wm * TM + i) * 16;
-                    sxA = tsx[r & 7];
-                    sxB = tsx[8 + (r & 7)];
-                    if constexpr (JH & 1) sxO = tsx[r];
-                }
-                auto total = [&](auto JJ) {
-                    constexpr int jj = decltype(JJ)::value;
-                    const v4i own = acc_read4<4 * ((hf * JH + jj) * TM + i)>();
-                    const v4i got = *reinterpret_cast<const v4i *>(theirs + (jj * IH + ii) * 1024 + lane * 16);
-                    return own + got;
-                };
-                static_for<JH / 2>([&](auto PP) {
-                    constexpr int jj = 2 * decltype(PP)::value;
-                    const int nb0 = n0 + (wn * TN + hf * JH + jj) * 16;
-                    const v4i a0 = total(std::integral_constant<int, jj>{}), a1 = total(std::integral_constant<int, jj + 1>{});
-                    v4i t0, t1;
+                const v4i a0 = acc_read4<4 * ((2 * rd) * TM + i)>() +
+                               *reinterpret_cast<const v4i *>(theirs + (0 * IH + ii) * 1024 + lane * 16);
+                const v4i a1 = acc_read4<4 * ((2 * rd + 1) * TM + i)>() +
+                               *reinterpret_cast<const v4i *>(theirs + (1 * IH + ii) * 1024 + lane * 16);
+                v4i t0, t1;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        t0[e] = ror8(a0[e]);
-                        t1[e] = ror8(a1[e]);
-                    }
-                    const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
-                    const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
-                    const int n = nb0 + (lo ? 0 : 16) + 4 * g_;
-                    if (!checked || n < N) {
-                        if (!checked || mA < M) store4<DEQ>(y, acc_out, (int64_t)mA * N + n, vA, sxA, swP[jj / 2]);
-                        if (!checked || mB < M) store4<DEQ>(y, acc_out, (int64_t)mB * N + n, vB, sxB, swP[jj / 2]);
-                    }
-                });
-                if constexpr (JH & 1) {
-                    constexpr int jj = JH - 1;
-                    const int m = mrow + r;
-                    const int n = n0 + (wn * TN + hf * JH + jj) * 16 + 4 * g_;
-                    const v4i a = total(std::integral_constant<int, jj>{});
-                    if (!checked || (m < M && n < N)) store4<DEQ>(y, acc_out, (int64_t)m * N + n, a, sxO, swP[jj / 2]);
+                for (int e = 0; e < 4; ++e) {
+                    t0[e] = ror8(a0[e]);
+                    t1[e] = ror8(a1[e]);
                 }
+                const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile 2rd (own), lanes r>=8 tile 2rd+1 (from lane r-8)
+                const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile 2rd+1 (own), lanes r<8 tile 2rd (from lane r+8)
+                store4<DEQ>(y, acc_out, (int64_t)mA * N + n, vA, sxA[ii], sw4);
+                store4<DEQ>(y, acc_out, (int64_t)mB * N + n, vB, sxB[ii], sw4);
             });
         });
     };
     // whole tiles only (the launcher sends ragged shapes to the four-wave kernel)
-    if (half == 0) finish(std::integral_constant<int, 0>{}, std::false_type{});
-    else finish(std::integral_constant<int, 1>{}, std::false_type{});
+    if (half == 0) finish(std::integral_constant<int, 0>{});
+    else finish(std::integral_constant<int, 1>{});
 }
 
 template <int TM, int TN, bool DEQ>
