@@ -116,6 +116,10 @@ def main():
                     help="context only: what a loop of v_mfma_i32_16x16x64_i8 alone sustains on this machine "
                          "(operands in registers, with and without the GEMM's LDS fragment reads, zeros and "
                          "activation-like codes); one JSON line")
+    ap.add_argument("--gemm-timeline", action="store_true",
+                    help="context only: where the eight-wave GEMM's time goes (prologue / stage loop / stores, in "
+                         "clock ticks read inside the kernel), from the instrumented build of the library; one JSON line")
+    ap.add_argument("--gemm-timeline-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--pmc-probe", action="store_true",
                     help="a few launches of the dominant kernels plus a copy-like kernel of known size, "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -125,12 +129,24 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
 
+    if args.gemm_timeline:
+        # the instrumented library is another build of the same sources: a child process loads it in place of the
+        # product library (nothing has touched the GPU in this process yet)
+        import subprocess
+        tl = os.path.join(ROOT, "mojo-linuxperiments_amd", "libmi355_int8_timeline.so")
+        if not os.path.exists(tl):
+            sys.exit("bench.py: %s is not built (make -C mojo-linuxperiments_amd/csrc)" % tl)
+        env = dict(os.environ, MI355_INT8_LIB=tl)
+        sys.exit(subprocess.run([sys.executable, os.path.abspath(__file__), "--gemm-timeline-child"], env=env).returncode)
+
     import mi355_int8 as mi     # fails loudly when the HIP library is not built
     import workload as wl
 
     if args.mfma_probe:
         print(json.dumps(mfma_probe()), flush=True)
         return
+    if args.gemm_timeline_child:
+        return gemm_timeline(mi, wl)
     if args.pmc_probe:
         return pmc_probe(mi, wl)
     if args.vendor_gemm:
@@ -540,6 +556,71 @@ def moe_layer(mi, wl, dev, s, timer, reps=20, graph=True):
                                "hbm_frac": round(wbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                "TOPS": round(ops / (ms * 1e-3) / 1e12, 2),
                                "tokens_per_s": round(T / (ms * 1e-3), 1), "weight_bytes": wbytes}}
+
+
+def gemm_timeline(mi, wl):
+    """The eight-wave GEMM on its two cfg3 shapes, 400 launches each on the benchmark's codes (sustained clock), then
+    the ticks the last launch left: per workgroup and K half, first instruction -> first stage ready, the stage
+    loop, exchange + stores until the last store is issued, until the stores are acknowledged."""
+    import ctypes as C
+    lib = mi.lib
+    if not hasattr(lib, "mi_debug_gemm_timeline"):
+        sys.exit("bench.py --gemm-timeline-child needs the instrumented library (run bench.py --gemm-timeline)")
+    dev = mi.Device(arena_bytes=4 << 30)
+    pool = mi.StreamPool(dev, 1)
+    s = pool.stream(0)
+    M = wl.PREFILL_M
+    out = {}
+    for name, K, N, tile in (("qkv", 4096, 6144, (256, 192)), ("down", 14336, 4096, (128, 256))):
+        mark = dev.mark()
+        m2 = dev.mark()
+        qx, sx = dev.empty((M, K), np.int8), dev.empty(M, np.float32)
+        mi.fwht_quant(dev.upload(wl.activations(2025, M, K, stream=K)), qx, sx, wl.HADAMARD_BLOCK)
+        qw0, sw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+        mi.fwht_quant(dev.upload(wl.weights(2025, N, K, stream=K + N)), qw0, sw, wl.HADAMARD_BLOCK)
+        dev.sync()
+        xh, sxh, wh, swh = dev.download(qx), dev.download(sx), dev.download(qw0), dev.download(sw)
+        dev.reset_to(m2)
+        qx, sx, sw = dev.upload(xh), dev.upload(sxh), dev.upload(swh)
+        copies = MALL_BYTES // (N * K) + 2
+        qws = [dev.upload(wh) for _ in range(copies)]
+        y = dev.empty((M, N), np.float32)
+        e0, e1 = mi.Event(), mi.Event()
+        reps = 400
+        for it in range(reps + 40):
+            if it == reps:
+                e0.record(s)
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qws[it % copies].ptr, sw.ptr, y.ptr, M, N, K, s))
+        e1.record(s)
+        e1.synchronize()
+        us = e0.elapsed_ms(e1) / 40 * 1e3
+        ntile = (M // tile[0]) * (N // tile[1])
+        buf = np.zeros(ntile * 2 * 8, np.uint64)
+        lib.mi_debug_gemm_timeline.restype = C.c_int32
+        mi.check(lib.mi_debug_gemm_timeline(buf.ctypes.data_as(C.c_void_p), C.c_int32(buf.size)))
+        t = buf.reshape(ntile, 2, 8).astype(np.float64)
+        nk = K // 128
+        mhz = float((t[:, :, 4] / t[:, :, 5]).mean() * 100.0)
+        out[name] = {
+            "kernel_us_event": round(us, 2), "workgroups": ntile, "stages": nk, "clock_mhz": round(mhz),
+            "ticks": {"prologue": round(float(t[:, :, 0].mean())), "stage_loop": round(float(t[:, :, 1].mean())),
+                      "exchange_and_stores_issued": [round(float(t[:, h, 2].mean())) for h in (0, 1)],
+                      "stores_acknowledged": round(float(t[:, :, 3].mean())), "whole_kernel": round(float(t[:, :, 4].mean()))},
+            "ticks_per_stage": round(float(t[:, :, 1].mean()) / nk),
+            "mfma_per_simd_and_stage": (tile[0] // 32) * (tile[1] // 32) * 2,
+            "us": {"prologue": round(float(t[:, :, 0].mean()) / mhz, 2), "stage_loop": round(float(t[:, :, 1].mean()) / mhz, 2),
+                   "exchange_and_stores": round(float((t[:, :, 2] + t[:, :, 3]).mean()) / mhz, 2)},
+            "first_entry_to_last_end_us": round(float(t[:, :, 7].max() - t[:, :, 6].min()) / 100.0, 2),
+            "entry_skew_us": round(float(t[:, :, 6].max() - t[:, :, 6].min()) / 100.0, 2),
+            "end_skew_us": round(float(t[:, :, 7].max() - t[:, :, 7].min()) / 100.0, 2),
+        }
+        dev.reset_to(mark)
+    print(json.dumps({"gemm_timeline": out, "M": M,
+                      "note": "k_w8a8_pair, clock ticks = s_memtime read by waves 0 and 4 of every workgroup in the "
+                              "last of 440 launches; real time = s_memrealtime (100 MHz); instrumented build "
+                              "(libmi355_int8_timeline.so), five clock reads a wave outside the stage loop"}), flush=True)
+    pool.destroy()
+    dev.close()
 
 
 def mfma_probe():

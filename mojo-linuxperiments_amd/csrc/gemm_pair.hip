@@ -41,7 +41,6 @@
 
 namespace mi {
 
-struct GemmGrid;   // gemm_tiled.hip
 namespace pair {
 
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -51,6 +50,14 @@ struct Grid {
     int pm, pn;  // XCD partition; pm == 0 -> plain row-major tile order
 };
 
+
+#ifdef MI_GEMM_TIMELINE
+// Built only into libmi355_int8_timeline.so (bench.py --gemm-timeline): waves 0 and 4 of every workgroup leave the
+// clock ticks (s_memtime) of the kernel's three phases and the 100 MHz real time of entry and end.  Five clock reads
+// a wave; the stage loop itself is untouched.
+constexpr int TIMELINE_WGS = 4096;
+__device__ unsigned long long g_timeline[TIMELINE_WGS * 2 * 8];
+#endif
 
 template <int N>
 __device__ __forceinline__ void wait_lgkm()
@@ -146,6 +153,9 @@ __global__ __launch_bounds__(512) void k_w8a8_pair(const int8_t *__restrict__ qx
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int pw = wave & 3, half = wave >> 2;   // wave tile of the pair, K half of every stage
+#ifdef MI_GEMM_TIMELINE
+    const unsigned long long tl_entry = __builtin_amdgcn_s_memtime(), tl_rentry = __builtin_amdgcn_s_memrealtime();
+#endif
 
     int tile_m, tile_n;
     {
@@ -258,6 +268,9 @@ __global__ __launch_bounds__(512) void k_w8a8_pair(const int8_t *__restrict__ qx
         static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb[decltype(I)::value], xo); });
     }
     int kt = 0;
+#ifdef MI_GEMM_TIMELINE
+    const unsigned long long tl_loop0 = __builtin_amdgcn_s_memtime();
+#endif
     // one stage; LAST: no stage follows, nothing is requested
     auto stage = [&](auto LAST_) {
         constexpr bool LAST = decltype(LAST_)::value;
@@ -323,6 +336,9 @@ __global__ __launch_bounds__(512) void k_w8a8_pair(const int8_t *__restrict__ qx
                   "the last group must not use wa[0] or wa[1], nor the one before it wa[0]");
     for (; kt + 1 < nk; ++kt) stage(std::false_type{});
     stage(std::true_type{});
+#ifdef MI_GEMM_TIMELINE
+    const unsigned long long tl_loop1 = __builtin_amdgcn_s_memtime();
+#endif
     // everything of this wave is home; 2 x 16 wait states cover the longest MFMA-result -> read hazard
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
     __syncthreads();   // every wave is done with the stage buffers: they carry the exchange below
@@ -392,6 +408,24 @@ __global__ __launch_bounds__(512) void k_w8a8_pair(const int8_t *__restrict__ qx
     // whole tiles only (the launcher sends ragged shapes to the four-wave kernel)
     if (half == 0) finish(std::integral_constant<int, 0>{});
     else finish(std::integral_constant<int, 1>{});
+#ifdef MI_GEMM_TIMELINE
+    {
+        const unsigned long long tl_issued = __builtin_amdgcn_s_memtime();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned long long tl_done = __builtin_amdgcn_s_memtime(), tl_rdone = __builtin_amdgcn_s_memrealtime();
+        if (lane == 0 && pw == 0 && blockIdx.x < TIMELINE_WGS) {
+            unsigned long long *o = g_timeline + (blockIdx.x * 2 + half) * 8;
+            o[0] = tl_loop0 - tl_entry;    // first instruction -> first stage in LDS, first fragments requested
+            o[1] = tl_loop1 - tl_loop0;    // the stage loop
+            o[2] = tl_issued - tl_loop1;   // exchange of the K halves and the stores, to the last store issued
+            o[3] = tl_done - tl_issued;    // this wave's stores acknowledged
+            o[4] = tl_done - tl_entry;
+            o[5] = tl_rdone - tl_rentry;
+            o[6] = tl_rentry;
+            o[7] = tl_rdone;
+        }
+    }
+#endif
 }
 
 template <int TM, int TN, bool DEQ>
@@ -437,6 +471,14 @@ int32_t launch_pair(int tm, int tn, const int8_t *qx, const float *sx, const int
     return MI_EINVAL;
 }
 
+
+#ifdef MI_GEMM_TIMELINE
+extern "C" __attribute__((visibility("default"))) int32_t mi_debug_gemm_timeline(unsigned long long *out, int32_t n)
+{
+    if (!out || n < 0 || n > pair::TIMELINE_WGS * 2 * 8) return MI_EINVAL;
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(pair::g_timeline), (size_t)n * 8) == hipSuccess ? MI_OK : MI_EIO;
+}
+#endif
 
 template int32_t launch_pair<true>(int, int, const int8_t *, const float *, const int8_t *, const float *, int32_t *,
                                    float *, int, int, int, hipStream_t);

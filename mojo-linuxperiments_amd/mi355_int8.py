@@ -14,7 +14,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmi355_int8.so")
+# MI355_INT8_LIB names another build of the same library (bench.py --gemm-timeline loads the instrumented one)
+LIB_PATH = os.environ.get("MI355_INT8_LIB") or os.path.join(_HERE, "libmi355_int8.so")
 
 OK, EIO, ENOMEM, EBUSY, ENODEV, EINVAL, ENOSPC, ERANGE = 0, -5, -12, -16, -19, -22, -28, -34
 
