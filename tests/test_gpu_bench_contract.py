@@ -33,6 +33,32 @@ def test_bench_line_fields():
     assert b["ms_per_step"] == b["config"]["ms_per_step_graph"] and "ms_per_step_eager" in b["config"]
     # the HBM traffic figure says where it comes from: a separate counter run, not this one
     assert r["traffic"] is None or "profiles/" in r["traffic_source"]
+    # the matrix-pipe probe's figure rides along as context: below the published peak, above what the GEMMs reach
+    m = r["sustained_mfma_measured"]
+    assert m is not None and r["achieved"] < m["tops"] < r["peak"] and m["tops"] <= m["zeros_no_reads_tops"] <= r["peak"]
+    assert abs(m["frac_of_it"] - r["achieved"] / m["tops"]) < 1e-3
+
+
+@pytest.mark.gpu
+def test_probe_and_timeline_modes_print_one_json_line_each():
+    """The two measurement modes behind profiles/mfma_power_limited_peak.md and profiles/gemm_pair_timeline.md."""
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--mfma-probe"], capture_output=True, text=True,
+                         timeout=300, cwd=ROOT)
+    assert out.returncode == 0, out.stderr[-2000:]
+    runs = json.loads(out.stdout.strip().splitlines()[-1])["mfma_power_limited_peak"]["runs"]
+    assert len(runs) == 8 and all(1000 < r["tops"] < 5000 and 10 < r["clock_ticks_per_mfma"] < 20 for r in runs)
+    # two waves of a SIMD issue the instruction faster than one wave can
+    for a, b in zip(runs[0::2], runs[1::2]):
+        assert (a["waves_per_simd"], b["waves_per_simd"]) == (1, 2) and b["clock_ticks_per_mfma"] < a["clock_ticks_per_mfma"]
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gemm-timeline"], capture_output=True,
+                         text=True, timeout=300, cwd=ROOT)
+    assert out.returncode == 0, out.stderr[-2000:]
+    tl = json.loads(out.stdout.strip().splitlines()[-1])["gemm_timeline"]
+    for name in ("qkv", "down"):
+        t = tl[name]["ticks"]
+        parts = t["prologue"] + t["stage_loop"] + min(t["exchange_and_stores_issued"]) + t["stores_acknowledged"]
+        assert 0.9 * parts <= t["whole_kernel"] <= 1.1 * (parts + 3000)
+        assert tl[name]["ticks_per_stage"] > 12 * tl[name]["mfma_per_simd_and_stage"]   # the pipe's own floor
 
 
 def test_cpu_baseline_leg_pins_its_threads_per_numa_node():
