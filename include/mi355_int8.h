@@ -176,6 +176,36 @@ MI_API int32_t mi_w8a8_gemm_i32(const int8_t *qx, const int8_t *qw, int32_t *acc
 MI_API int32_t mi_w8a8_gemm_dequant_f32(const int8_t *qx, const float *sx,
                                         const int8_t *qw, const float *sw, float *y,
                                         int64_t M, int64_t N, int64_t K, void *stream);
+/* a4 for several contractions at once: ONE launch whose workgroups (one per compute unit) walk a list of 256 x 192
+ * output tiles drawn from every problem of the batch, so that no problem's tile count has to divide by the number
+ * of compute units, no launch gap or first memory round trip lies between the problems, and one unit's stores fall
+ * under the other units' stage loops.  No upstream counterpart.  A batch is made once for a list of shapes
+ * (mnk int64 [n][3] = M, N, K per problem; n <= 8; M >= 256, N >= 192, N % 16 == 0, K % 128 == 0): the tile lists
+ * are computed on the host and copied (synchronously) into `plan`, device memory of the caller of at least
+ * mi_gemm_batch_plan_bytes(mnk, n) bytes that must stay untouched while the batch lives.  A run takes the operands
+ * of this call (shapes must equal the batch's) and is an ordinary asynchronous launch: it may be captured into a
+ * graph.  Outputs of different problems must not overlap.  Results equal those of mi_w8a8_gemm_dequant_f32 /
+ * mi_w8a8_gemm_i32 on each problem, bit for bit. */
+typedef struct mi_gemm_problem {
+    const int8_t *qx;   /* int8 [M,K] */
+    const float *sx;    /* fp32 [M]   (unused by the int32 form) */
+    const int8_t *qw;   /* int8 [N,K] */
+    const float *sw;    /* fp32 [N]   (unused by the int32 form) */
+    void *out;          /* fp32 [M,N] (run_f32) or int32 [M,N] (run_i32), 16-byte aligned */
+    int64_t M, N, K;
+} mi_gemm_problem;
+typedef struct mi_gemm_batch mi_gemm_batch;
+MI_API int64_t mi_gemm_batch_plan_bytes(const int64_t *mnk, int32_t n);
+/* The tile lists a batch would hold on a device of `compute_units` units, written to host memory (int32
+ * [compute_units][per_wg][4] = problem or -1 for the end of a workgroup's list, first row, first column, cost in K
+ * stages; workgroup w runs on XCD w % 8): for tests and for callers that want to look at the balance.  Returns the
+ * bytes written.  Makes no device call. */
+MI_API int64_t mi_gemm_batch_plan_host(const int64_t *mnk, int32_t n, int32_t compute_units, int32_t *lists_out,
+                                       int64_t capacity_bytes, int32_t *per_wg_out);
+MI_API int32_t mi_gemm_batch_create(const int64_t *mnk, int32_t n, void *plan, int64_t plan_bytes, mi_gemm_batch **out);
+MI_API int32_t mi_gemm_batch_destroy(mi_gemm_batch *b);
+MI_API int32_t mi_gemm_batch_run_f32(mi_gemm_batch *b, const mi_gemm_problem *problems, void *stream);
+MI_API int32_t mi_gemm_batch_run_i32(mi_gemm_batch *b, const mi_gemm_problem *problems, void *stream);
 /* a6 alone. */
 MI_API int32_t mi_dequant_i32_f32(const int32_t *acc, const float *sx, const float *sw,
                                   float *y, int64_t M, int64_t N, void *stream);

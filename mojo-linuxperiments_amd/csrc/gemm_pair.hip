@@ -38,12 +38,11 @@
 #include <utility>
 
 #include "common.h"
+#include "gemm_pair_ops.h"
 
 namespace mi {
 
 namespace pair {
-
-typedef __attribute__((address_space(3))) void *lptr_t;
 
 struct Grid {
     int tiles_m, tiles_n;
@@ -58,69 +57,6 @@ struct Grid {
 constexpr int TIMELINE_WGS = 4096;
 __device__ unsigned long long g_timeline[TIMELINE_WGS * 2 * 8];
 #endif
-
-template <int N>
-__device__ __forceinline__ void wait_lgkm()
-{
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-}
-template <int OFF>
-__device__ __forceinline__ void ds_read128(v4i &dst, unsigned addr)
-{
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
-}
-// direct-to-LDS load of 16 bytes per lane: global address = sbase + voff, LDS address = ldsaddr + 16 * lane
-__device__ __forceinline__ void dma16(const int8_t *sbase, unsigned voff, unsigned ldsaddr)
-{
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(voff), "s"(sbase), "s"(ldsaddr)
-                 : "memory", "m0");
-}
-// accumulator (j, i) lives in a[4*(j*TM+i) .. +3]
-template <int LO>
-__device__ __forceinline__ void mfma_acc(const v4i &a, const v4i &b)
-{
-    asm volatile("v_mfma_i32_16x16x64_i8 a[%c2:%c3], %0, %1, a[%c2:%c3]" ::"v"(a), "v"(b), "n"(LO), "n"(LO + 3));
-}
-template <int R>
-__device__ __forceinline__ int acc_read()
-{
-    int v;
-    asm volatile("v_accvgpr_read_b32 %0, a%c1" : "=v"(v) : "n"(R));
-    return v;
-}
-template <int LO>
-__device__ __forceinline__ v4i acc_read4()
-{
-    v4i v;
-    v[0] = acc_read<LO>();
-    v[1] = acc_read<LO + 1>();
-    v[2] = acc_read<LO + 2>();
-    v[3] = acc_read<LO + 3>();
-    return v;
-}
-template <int R>
-__device__ __forceinline__ void acc_zero()
-{
-    asm volatile("v_accvgpr_write_b32 a%c0, 0" ::"n"(R));
-}
-__device__ __forceinline__ int ror8(int v) { return __builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false); }
-
-template <bool DEQ>
-__device__ __forceinline__ void store4(float *y, int32_t *acc_out, int64_t idx, const v4i &v, float sxm, const float4 &s4)
-{
-    if constexpr (DEQ) {
-        float4 o;
-        o.x = ((float)v[0] * sxm) * s4.x;
-        o.y = ((float)v[1] * sxm) * s4.y;
-        o.z = ((float)v[2] * sxm) * s4.z;
-        o.w = ((float)v[3] * sxm) * s4.w;
-        *reinterpret_cast<float4 *>(y + idx) = o;
-    } else {
-        *reinterpret_cast<v4i *>(acc_out + idx) = v;
-    }
-}
 
 template <int TM, int TN>
 struct Cfg {

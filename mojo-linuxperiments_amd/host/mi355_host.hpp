@@ -173,6 +173,35 @@ struct QuantLinear {
     }
 };
 
+// Several W8A8 contractions in one launch (mi_gemm_batch_*): made once for a list of shapes, run with the operands of
+// each call.  Move-only; the tile lists live in arena memory.
+struct GemmBatch {
+    mi_gemm_batch *h = nullptr;
+    void *plan = nullptr;
+    int32_t n = 0;
+
+    GemmBatch() = default;
+    GemmBatch(const GemmBatch &) = delete;
+    GemmBatch &operator=(const GemmBatch &) = delete;
+    GemmBatch(GemmBatch &&o) noexcept : h(o.h), plan(o.plan), n(o.n) { o.h = nullptr; }
+    ~GemmBatch() { if (h) mi_gemm_batch_destroy(h); }
+    explicit operator bool() const { return h != nullptr; }
+
+    // mnk: [count][3] = M, N, K per problem.  Status as in the C ABI (MI_ENOMEM: the arena is exhausted).
+    template <typename Arena>
+    int32_t prepare(Arena &arena, const int64_t *mnk, int32_t count)
+    {
+        const int64_t bytes = mi_gemm_batch_plan_bytes(mnk, count);
+        if (bytes < 0) return (int32_t)bytes;
+        plan = arena.template alloc<uint8_t>(bytes);
+        if (!plan) return MI_ENOMEM;
+        n = count;
+        return mi_gemm_batch_create(mnk, count, plan, bytes, &h);
+    }
+    int32_t run(const mi_gemm_problem *problems, void *stream) const { return mi_gemm_batch_run_f32(h, problems, stream); }
+    int32_t run_i32(const mi_gemm_problem *problems, void *stream) const { return mi_gemm_batch_run_i32(h, problems, stream); }
+};
+
 // Decode attention over an int8 KV cache held by the caller.
 struct DecodeAttention {
     int64_t B = 0, Hq = 0, Hkv = 0, D = 128, T = 0;

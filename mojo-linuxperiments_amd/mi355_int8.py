@@ -85,6 +85,12 @@ SIGNATURES = {
     "mi_w8a8_gemm_i32": (i32, [vp, vp, vp, i64, i64, i64, vp]),
     "mi_w8a8_gemm_dequant_f32": (i32, [vp, vp, vp, vp, vp, i64, i64, i64, vp]),
     "mi_dequant_i32_f32": (i32, [vp, vp, vp, vp, i64, i64, vp]),
+    "mi_gemm_batch_plan_bytes": (i64, [vp, i32]),
+    "mi_gemm_batch_plan_host": (i64, [vp, i32, i32, vp, i64, C.POINTER(i32)]),
+    "mi_gemm_batch_create": (i32, [vp, i32, vp, i64, C.POINTER(vp)]),
+    "mi_gemm_batch_destroy": (i32, [vp]),
+    "mi_gemm_batch_run_f32": (i32, [vp, vp, vp]),
+    "mi_gemm_batch_run_i32": (i32, [vp, vp, vp]),
     "mi_w8a8_linear_workspace_bytes": (i64, [i64, i64, i64]),
     "mi_w8a8_linear_f32": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
     "mi_w8a8_linear_f32_noalloc": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp]),
@@ -324,6 +330,49 @@ def fwht_quant(x, q, scale, block, stream=None):
 def fwht(x, out, block, stream=None):
     M, K = x.shape
     check(lib.mi_fwht_f32(x.ptr, out.ptr, M, K, block, stream), "mi_fwht_f32")
+
+
+class GemmProblem(C.Structure):
+    """mi_gemm_problem of the header: one contraction of a batch."""
+    _fields_ = [("qx", vp), ("sx", vp), ("qw", vp), ("sw", vp), ("out", vp), ("M", i64), ("N", i64), ("K", i64)]
+
+
+class GemmBatch:
+    """Several W8A8 contractions in one launch (mi_gemm_batch_*): made once for a list of (M, N, K) shapes, run
+    with the operands of each call.  The tile lists live in arena memory of `dev`."""
+
+    def __init__(self, dev, shapes):
+        self.shapes = [tuple(int(v) for v in s) for s in shapes]
+        n = len(self.shapes)
+        mnk = (i64 * (3 * n))(*[v for s in self.shapes for v in s])
+        nbytes = lib.mi_gemm_batch_plan_bytes(mnk, n)
+        if nbytes < 0:
+            raise MiError(int(nbytes), "mi_gemm_batch_plan_bytes")
+        self.plan = dev.empty(nbytes, np.uint8)
+        self.h = vp()
+        check(lib.mi_gemm_batch_create(mnk, n, self.plan.ptr, nbytes, C.byref(self.h)), "mi_gemm_batch_create")
+
+    def _problems(self, ops):
+        arr = (GemmProblem * len(ops))()
+        for g, (qx, sx, qw, sw, out) in zip(arr, ops):
+            g.qx, g.qw, g.out = qx.ptr, qw.ptr, out.ptr
+            g.sx = sx.ptr if sx is not None else None
+            g.sw = sw.ptr if sw is not None else None
+            (g.M, g.K), g.N = qx.shape, qw.shape[0]
+        return arr
+
+    def run_f32(self, ops, stream=None):
+        """ops: [(qx, sx, qw, sw, y)] DevBufs per problem."""
+        check(lib.mi_gemm_batch_run_f32(self.h, self._problems(ops), stream), "mi_gemm_batch_run_f32")
+
+    def run_i32(self, ops, stream=None):
+        """ops: [(qx, None, qw, None, acc)] DevBufs per problem."""
+        check(lib.mi_gemm_batch_run_i32(self.h, self._problems(ops), stream), "mi_gemm_batch_run_i32")
+
+    def destroy(self):
+        if self.h:
+            lib.mi_gemm_batch_destroy(self.h)
+            self.h = None
 
 
 def gemm_i32(qx, qw, acc, stream=None):

@@ -1,0 +1,104 @@
+"""The work list of the batched GEMM, checked on the host (no device call): every output element of every problem
+is covered by a tile that lies inside its matrix, every address the kernel forms from a tile stays inside the
+operands and inside the kernel's LDS areas, and the list is balanced."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+BM, BN = 256, 192
+CFG3 = [(2048, 6144, 4096), (2048, 14336, 4096), (2048, 14336, 4096), (2048, 4096, 14336)]
+
+
+def plan(mi, shapes, cus=256):
+    n = len(shapes)
+    mnk = (C.c_int64 * (3 * n))(*[v for s in shapes for v in s])
+    cap = 64 << 20
+    buf = np.empty(cap // 4, np.int32)
+    per_wg = C.c_int32()
+    nbytes = mi.lib.mi_gemm_batch_plan_host(mnk, n, cus, buf.ctypes.data, cap, C.byref(per_wg))
+    assert nbytes > 0, nbytes
+    assert nbytes == cus * per_wg.value * 16
+    return buf[:nbytes // 4].reshape(cus, per_wg.value, 4)
+
+
+@pytest.mark.parametrize("shapes,cus", [
+    (CFG3, 256), ([(300, 272, 512)], 256), ([(256, 192, 128)], 256), ([(2048, 6144, 256)] * 8, 256),
+    ([(1000, 1008, 384), (4096, 208, 128)], 64), (CFG3, 304), ([(777, 4096, 1024)], 7),
+])
+def test_every_output_is_covered_once_or_with_equal_tiles(mi, shapes, cus):
+    lists = plan(mi, shapes, cus)
+    cover = [np.zeros((M, N), np.uint8) for M, N, K in shapes]
+    for w in range(cus):
+        ended = False
+        for p, m0, n0, cost in lists[w]:
+            if p < 0:
+                ended = True
+                continue
+            assert not ended, "an entry behind the end mark"
+            M, N, K = shapes[p]
+            assert 0 <= m0 <= M - BM and 0 <= n0 <= N - BN and n0 % 16 == 0
+            assert cost == K // 128 + 4
+            cover[p][m0:m0 + BM, n0:n0 + BN] += 1
+        assert ended, "every list ends with a mark"
+    for c, (M, N, K) in zip(cover, shapes):
+        assert c.min() >= 1
+        # only the last row / column of tiles is moved inwards: at most four tiles meet in a corner
+        assert c.max() <= 4
+        tiles = -(-M // BM) * -(-N // BN)
+        assert int(c.sum()) == tiles * BM * BN
+
+
+def test_addresses_formed_from_a_tile_stay_inside(mi):
+    """Replays the kernel's address arithmetic for the first and last tile rows/columns of a problem: global byte
+    offsets of the direct-to-LDS loads (row (pw + 4q) * 8 + rho of the tile, chunk c ^ sigma of a 128-byte K stage),
+    their LDS targets, the exchange parcels and the scale areas."""
+    TM, TN = 8, 6
+    NBX, NBW = 4 * TM, 4 * TN
+    XSTAGE, WSTAGE = NBX * 1024, NBW * 1024
+    XAREA, STAGES = 2 * XSTAGE, 2 * XSTAGE + 3 * WSTAGE
+    PARCELS_AT, PARCELS = XAREA + 2 * WSTAGE, 2 * 8 * 2048
+    SCALES_AT = max(STAGES, PARCELS_AT + PARCELS)
+    LDS = SCALES_AT + 2 * (BM + BN) * 4
+    assert LDS <= 160 * 1024
+    for M, N, K in [(2048, 14336, 4096), (300, 272, 512), (256, 192, 128)]:
+        lists = plan(mi, [(M, N, K)])
+        tiles = lists[lists[:, :, 0] >= 0]
+        for _, m0, n0, _ in tiles[[0, -1]]:
+            for pw in range(4):
+                for lane in range(64):
+                    rho, c = lane >> 3, lane & 7
+                    sigma = ((pw & 1) << 2) | (rho >> 1)
+                    voff = (pw * 8 + rho) * K + ((c ^ sigma) << 4)
+                    for kt in (0, K // 128 - 1):
+                        for rows, base, nblk, lds0, stage, nbuf in ((M, m0, NBX // 4, pw * 1024, XSTAGE, 2),
+                                                                    (N, n0, NBW // 4, XAREA + pw * 1024, WSTAGE, 3)):
+                            for q in range(nblk):
+                                off = base * K + kt * 128 + q * 32 * K + voff
+                                assert 0 <= off and off + 16 <= rows * K
+                                for buf in range(nbuf):
+                                    lds = lds0 + buf * stage + q * 4096 + 16 * lane
+                                    lo, hi = (0, XAREA) if rows is M and stage == XSTAGE and lds0 < XAREA else (XAREA, STAGES)
+                                    assert lo <= lds and lds + 16 <= hi
+        # parcels and scales
+        for wave in range(8):
+            for area in range(2):
+                end = PARCELS_AT + (area * 8 + wave) * 2048 + 1024 + 63 * 16 + 16
+                assert PARCELS_AT <= end <= SCALES_AT
+            for par in range(2):
+                if wave * 64 < BM + BN:
+                    end = SCALES_AT + par * (BM + BN) * 4 + wave * 256 + 63 * 4 + 4
+                    assert end <= LDS
+
+
+def test_cfg3_list_is_balanced(mi):
+    lists = plan(mi, CFG3)
+    load = np.where(lists[:, :, 0] >= 0, lists[:, :, 3], 0).sum(axis=1)
+    assert load.min() > 0
+    # one tile of the K = 14336 problem is 116 of the 270 units a workgroup gets: the longest list may exceed the
+    # mean by less than a short tile
+    assert load.max() <= load.mean() * 1.10, (load.max(), load.mean())
+    # workgroup id mod 8 is the XCD: each XCD gets an eighth of every problem
+    for p in range(4):
+        per_xcd = [(lists[x::8, :, 0] == p).sum() for x in range(8)]
+        assert max(per_xcd) - min(per_xcd) <= 1, per_xcd
