@@ -1,28 +1,39 @@
-// Several W8A8 contractions in ONE launch: a workgroup per compute unit walks a list of output tiles.
+// Several W8A8 contractions in ONE launch: a workgroup per compute unit walks a list of output tiles, and the K
+// stages of all its tiles form one uninterrupted stream.
 //   acc[m,n] = sum_k qx[m,k] * qw[n,k],   y = ((float)acc * sx[m]) * sw[n]      (per problem of the batch)
 //
 // Why.  A prefill GEMM launched on its own spends a third of its time outside the stage loop: the gap to the
-// previous kernel, the first memory round trip of 256 workgroups asking at once, and a store phase in which every
-// tile of the chip writes at the same moment with the matrix pipe idle.  Its tile shape is also dictated by how
-// the tile count divides by the number of compute units.  Here the tiles of all problems form one work list:
-//   - one tile shape for everything (32*TM x 32*TN = 256 x 192, eight waves, two per SIMD: the stage loop of
-//     gemm_pair.hip, which is the fastest one), because the list is balanced as a whole and not per problem;
-//   - the first two K stages of a workgroup's next tile are requested BEFORE the current tile's sums are exchanged
-//     and stored, so the next stage loop starts on data that is already in LDS;
-//   - workgroups drift apart (tiles differ in K), so stores of one unit fall under the stage loops of the others.
+// previous kernel, the first memory round trip of 256 workgroups asking at once, and an epilogue in which the matrix
+// pipe idles while 196 KB per compute unit are converted and stored.  Its tile shape is also dictated by how the
+// tile count divides by the number of compute units.  Here
+//   - the tiles of all problems form one work list of 256 x 192 tiles, balanced as a whole on the host;
+//   - the direct-to-LDS loads run two stages ahead of the matrix instructions ACROSS tile boundaries (the stage
+//     buffers rotate for the whole life of the workgroup and never drain between tiles);
+//   - a wave owns 64 x 96 outputs over the WHOLE of K (96 accumulation registers), so no partial sums are exchanged
+//     between waves: when a tile's last stage has been issued the wave converts, scales, stores and clears its 24
+//     accumulators in one straight run of vector instructions, while the loads of the next tile (requested two
+//     stages ago) are already landing.
+//     (Measured and not kept: a second accumulator set, drained one accumulator per stage under the next tile's
+//     matrix instructions.  Both waves of a SIMD reach the drain at the same point of a stage, so the matrix pipe
+//     idles all the same, and the store queues behind the stage's direct-to-LDS loads on the unit's one memory path:
+//     it cost 1,000 ticks per stage, more than the straight run at the end of the tile.)
 // A tile that would cross the edge of its matrix is moved inwards until it fits: the overlap with its neighbour
 // is computed twice, both times to the same values (exact integers, the same fp32 operations), so every problem
 // needs only M >= 256, N >= 192; no ragged code path exists.
 //
-// Per wave, stage loop, LDS layout and swizzle: see gemm_pair.hip (this file repeats its stage, with the first
-// stage of a tile writing the accumulators instead of adding to them).  What differs:
-//   - the K halves of a wave pair meet in rounds of two accumulators (one row tile, two column tiles) through
-//     2 x 8 parcels of 2 KB that lie in the third weight buffer, the only stage buffer the prefetched stages 0 and
-//     1 of the next tile do not use;
-//   - the epilogue's scales sit in one of two LDS areas, by tile parity (the next tile's are requested with its
-//     first stages, while the current tile's are still being read).
+// Waves: 8 = 4 (rows) x 2 (columns), two per SIMD; wave tile 4 x 6 matrix-instruction tiles.  A 128-byte K stage
+// is two halves of 64 bytes; a half is six groups (one weight fragment against the four activation fragments).
+// LDS layout, swizzle and load shapes are those of gemm_pair.hip.  Per wave and half: 6 weight fragment reads
+// (through four register slots, two groups ahead) and 4 activation fragment reads (each right behind the last
+// matrix instruction that reads the old fragment; the last two groups of a half are interleaved so that the first
+// reload is 6 instructions ahead of its use).
+//
+// Registers: v[64..159] are the accumulators, named by hand; the kernel is limited to v0..v63 for everything the
+// compiler places (see gemm_pair_ops.h).
+//
 // Memory operations complete in issue order (one counter for loads and stores), and every wait below is written
-// against that order: at most 1 + 4*(LX+LW) + IH*TN = 53 are ever in flight per wave (the counter holds 63).
+// against that order.  Only waves 0..3 (the ones the matrix pipe serves first) issue loads; every wave stores its
+// own results.
 //
 // The list itself is made on the host when the batch is created (longest tiles first, each to the least loaded
 // workgroup of its XCD; tiles that run at the same time on one XCD are neighbours in column-major order, so they
@@ -38,6 +49,10 @@
 
 #include "common.h"
 #include "gemm_pair_ops.h"
+
+#ifndef MI_STORE_MOD
+#define MI_STORE_MOD " nt"   // the results are not read again by this kernel: stores that do not displace the operands in L2 (measured: 385 -> 363 us for the four prefill projections as one batch)
+#endif
 
 namespace mi {
 namespace list {
@@ -57,41 +72,44 @@ struct Batch {
     Problem p[MAX_PROBLEMS];
 };
 
-template <int TM, int TN>
 struct Cfg {
-    static constexpr int BM = 32 * TM, BN = 32 * TN;
-    static constexpr int NBX = 4 * TM, NBW = 4 * TN;   // 1 KB blocks (8 rows x 128 B) per stage
+    static constexpr int TM = 4, TN = 6;                // matrix-instruction tiles of a wave
+    static constexpr int BM = 256, BN = 192;            // 4 x 2 waves
+    static constexpr int NBX = BM / 8, NBW = BN / 8;    // 1 KB blocks (8 rows x 128 B) per stage
     static constexpr int XSTAGE = NBX * 1024, WSTAGE = NBW * 1024, XAREA = 2 * XSTAGE;
-    static constexpr int STAGES = XAREA + 3 * WSTAGE;
-    static constexpr int IH = TM / 2;
-    static constexpr int PARCEL = 2048;                         // two accumulators of a wave
-    static constexpr int PARCELS_AT = XAREA + 2 * WSTAGE;       // the third weight buffer and what follows it
-    static constexpr int PARCELS = 2 * 8 * PARCEL;
-    static constexpr int SCALES = (BM + BN) * 4;
-    static constexpr int SCALES_AT = (STAGES > PARCELS_AT + PARCELS) ? STAGES : PARCELS_AT + PARCELS;
-    static constexpr int LDS = SCALES_AT + 2 * SCALES;
-    static constexpr int LX = NBX / 8, LW = NBW / 8;            // parts (pairs of loads) per loading wave and stage
-    static constexpr int NS = IH * TN;                          // stores per wave and tile
-    static_assert(NBX % 8 == 0 && NBW % 8 == 0, "blocks are dealt to eight waves");
-    static_assert(TN % 2 == 0 && TM % 2 == 0, "the two waves of a pair finish half of the tile each");
-    static_assert(TM * TN * 4 <= 192, "64 ordinary registers must remain");
+    static constexpr int STAGES = XAREA + 3 * WSTAGE;   // two activation buffers, three weight buffers
+    static constexpr int SCALES = (BM + BN) * 4;        // of one tile: BM row scales, then BN column scales
+    static constexpr int SCALES_AT = STAGES;
+    static constexpr int LDS = SCALES_AT + 2 * SCALES;  // two scale areas, by tile parity
+    static constexpr int LX = NBX / 8, LW = NBW / 8;    // parts (pairs of loads) per loading wave and stage
+    static constexpr int NACC = TM * TN;                // accumulators of a set
+    static constexpr int MIN_STAGES = 3;                // the loads run up to three stages ahead, into the next tile at most
+    static_assert(LX == 4 && LW == 3, "the stage's load slots are written out for four and three parts");
+    static_assert(vacc::ACC0 + 4 * NACC <= 256, "the accumulators lie above the compiler's registers");
     static_assert(LDS <= 160 * 1024, "LDS of a compute unit");
-    static_assert(1 + 4 * (LX + LW) + NS <= 63, "the memory counter has six bits");
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && BM + BN <= 512, "a wave brings 64 scales of one kind");
 };
 
 // direct-to-LDS load of 4 bytes per lane: global address = sbase + voff, LDS address = ldsaddr + 4 * lane
 __device__ __forceinline__ void dma4(const float *sbase, unsigned voff, unsigned ldsaddr)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 4\n\tglobal_load_lds_dword %0, %1"
                  :
                  : "v"(voff), "s"(sbase), "s"(ldsaddr)
                  : "memory", "m0");
 }
 #ifdef MI_GEMM_TIMELINE
+// The measurement build keeps a few more scalars alive and may spill some: a base the compiler brings back with a
+// vector instruction needs five wait states before a memory instruction reads it (see the build check of the
+// product library, which allows no such spill); here every load pays them.
+__device__ __forceinline__ void dma16(const int8_t *sbase, unsigned voff, unsigned ldsaddr)
+{
+    asm volatile("s_nop 4" ::: "memory");
+    pair::dma16(sbase, voff, ldsaddr);
+}
+#endif
+#ifdef MI_GEMM_TIMELINE
 // Built only into libmi355_int8_timeline.so (bench.py --gemm-timeline): wave 0 of every workgroup leaves, per tile,
-// the clock ticks (s_memtime) at which the tile's first stage was in LDS, its stage loop ended and its last store
-// was issued, and the 100 MHz real time at the first and the last of them.
+// the clock ticks (s_memtime) and the 100 MHz real time at which the tile's first and last stage began and ended.
 constexpr int TL_WGS = 512, TL_TILES = 16;
 __device__ unsigned long long g_list_timeline[TL_WGS * TL_TILES * 8];
 #endif
@@ -102,15 +120,9 @@ __device__ __forceinline__ v4i sload4(const v4i *p)
     asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(p) : "memory");
     return v;
 }
-
-struct Epi {   // what the epilogue of a tile needs once the load side has moved on to the next tile
-    void *out;
-    int N, K, m0, n0;
-};
-
-// lane-derived values are recomputed in every phase of a tile from a copy of the lane number that the compiler
-// cannot see through: otherwise it computes all of them once, before the tile loop, and 64 registers cannot hold them
-// beside the fragments
+// lane-derived values are recomputed where they are needed from a copy of the lane number that the compiler
+// cannot see through: otherwise it computes all of them once, before the tile loop, and 64 registers cannot hold
+// them beside the fragments
 __device__ __forceinline__ int opaque(int v)
 {
     asm volatile("" : "+v"(v));
@@ -123,350 +135,365 @@ __device__ __forceinline__ unsigned add_vs(unsigned a, unsigned s)
     asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(s), "v"(a));
     return r;
 }
+__device__ __forceinline__ void lds_read32(float &dst, unsigned addr)
+{
+    asm volatile("ds_read_b32 %0, %1" : "=v"(dst) : "v"(addr));
+}
+__device__ __forceinline__ void lds_read128f(v4f &dst, unsigned addr)
+{
+    asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(addr));
+}
 
-template <int TM, int TN, bool DEQ>
+template <bool DEQ>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2))) void k_w8a8_list(
     const Batch bt, const v4i *__restrict__ lists, int per_wg)
 {
-    using C = Cfg<TM, TN>;
-    constexpr int BM = C::BM, BN = C::BN;
+    using C = Cfg;
+    constexpr int TM = C::TM, TN = C::TN, BM = C::BM;
     constexpr int XSTAGE = C::XSTAGE, WSTAGE = C::WSTAGE, XAREA = C::XAREA;
-    constexpr int LX = C::LX, LW = C::LW, NS = C::NS, IH = C::IH;
-    constexpr int R = (TN % 3 == 0) ? 3 : 4;    // weight fragment registers in rotation
+    constexpr int NACC = C::NACC;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     // v[64 .. 255] are this kernel's accumulators, named by hand: the attribute above keeps everything the compiler
     // places below v64, and this clobber makes the wave's register count cover them
-    static_assert(vacc::ACC0 + 4 * TM * TN <= 256);
     asm volatile("" ::: "v64", "v255");
 
     const int tid = threadIdx.x, lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int pw = wave & 3, half = wave >> 2;   // wave tile of the pair, K half of every stage
-    const int wm = pw >> 1, wn = pw & 1;
-    const bool loader = half == 0;               // the waves the matrix pipe serves first issue every load
+    const int pw = wave & 3;
+    const int wm = wave >> 1, wn = wave & 1;   // wave tile: rows wm*64.., columns wn*96..
+    const bool loader = wave < 4;              // the waves the matrix pipe serves first issue every load
     const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
     const unsigned lds_x = lds_base + pw * 1024, lds_w = lds_base + XAREA + pw * 1024;
 
     const v4i *const my = lists + (int64_t)blockIdx.x * per_wg;
-    v4i ent = sload4(my);   // {problem or -1, first row, first column, -}
-    if (ent[0] < 0) return;
-    static_for<TM * TN>([&](auto I) { vacc::acc_zero4<4 * decltype(I)::value>(); });
+    // {problem or -1, first row, first column, -}: the tile the matrix pipe works on (three scalars, not the entry's four)
+    int e_p, e_m0, e_n0;
+    {
+        const v4i e = sload4(my);
+        e_p = e[0];
+        e_m0 = e[1];
+        e_n0 = e[2];
+    }
+    if (e_p < 0) return;
+    static_for<NACC>([&](auto I) { vacc::acc_zero4<4 * decltype(I)::value>(); });
 
-    // ---- the tile whose stages are being loaded
-    const int8_t *xtile = nullptr, *wtile = nullptr;
-    unsigned voff = 0;
-    int64_t bstep = 0;
-    int nk = 0;
-
-    // load side: lane l = 8*rho + c fetches the 16-byte chunk c ^ sigma of row rho of a block; wave pw fills
-    // blocks pw + 4q, so one lane offset serves every block on a uniform base that moves with q
-    auto lane_offset = [&](int K) {
+    // ---- load side.  The load cursor (a tile and a stage of it) runs two stages ahead of the matrix instructions.
+    // lane l = 8*rho + c fetches the 16-byte chunk c ^ sigma of row rho of a block; wave pw fills blocks pw + 4q,
+    // so one lane offset serves every block on a uniform base that moves with q
+    const int8_t *lx = nullptr, *lw = nullptr;
+    int64_t lbstep = 0;
+    unsigned lvoff = 0;
+    int lkt = 0, lnk = 0;
+    bool ldv = false;   // the cursor stands on a stage that exists
+    auto cursor_to = [&](const v4i &e) {
+        const Problem &P = bt.p[e[0]];
+        const int K = P.K;
+        lnk = K >> 7;
+        lkt = 0;
+        lx = P.qx + (int64_t)e[1] * K;
+        lw = P.qw + (int64_t)e[2] * K;
+        lbstep = (int64_t)32 * K;   // four blocks of eight rows
         const int l = opaque(lane0);
         const int lrow = pw * 8 + (l >> 3);
         const unsigned lchunk = (unsigned)(((l & 7) ^ (((pw & 1) << 2) | (l >> 4))) << 4);
-        return (unsigned)lrow * (unsigned)K + lchunk;
+        lvoff = (unsigned)lrow * (unsigned)K + lchunk;
+        ldv = true;
     };
-    auto issue_x1 = [&](auto I, unsigned buf, int kt) {
+    auto issue_x = [&](auto I, unsigned buf) {   // part p of the cursor's stage
         constexpr int p_ = decltype(I)::value;
-        if constexpr (p_ < LX) {
-            dma16(xtile + (int64_t)kt * 128 + (2 * p_) * bstep, voff, lds_x + buf + (2 * p_) * 4096);
-            dma16(xtile + (int64_t)kt * 128 + (2 * p_ + 1) * bstep, voff, lds_x + buf + (2 * p_ + 1) * 4096);
-        }
+        dma16(lx + (int64_t)lkt * 128 + (2 * p_) * lbstep, lvoff, lds_x + buf + (2 * p_) * 4096);
+        dma16(lx + (int64_t)lkt * 128 + (2 * p_ + 1) * lbstep, lvoff, lds_x + buf + (2 * p_ + 1) * 4096);
     };
-    auto issue_w1 = [&](auto I, unsigned buf, int kt) {
+    auto issue_w = [&](auto I, unsigned buf) {
         constexpr int p_ = decltype(I)::value;
-        if constexpr (p_ < LW) {
-            dma16(wtile + (int64_t)kt * 128 + (2 * p_) * bstep, voff, lds_w + buf + (2 * p_) * 4096);
-            dma16(wtile + (int64_t)kt * 128 + (2 * p_ + 1) * bstep, voff, lds_w + buf + (2 * p_ + 1) * 4096);
-        }
-    };
-    auto issue_x = [&](unsigned buf, int kt) { static_for<LX>([&](auto I) { issue_x1(I, buf, kt); }); };
-    auto issue_w = [&](unsigned buf, int kt) { static_for<LW>([&](auto I) { issue_w1(I, buf, kt); }); };
-
-    // a tile begins: its scales and its stages 0 and 1 are requested (activation buffers 0 and 1, weight buffers
-    // 0 and 1: every stage buffer is free when this is called).  In the memory counter's order: scales, stage 0,
-    // stage 1.  The scales go straight to their LDS area (wave w brings 64 of them: the BM row scales, then the BN
-    // column scales), so that no register has to hold them while the previous tile's epilogue runs.
-    auto begin_tile = [&](const v4i &e, unsigned scales_at) -> Epi {
-        const Problem &P = bt.p[e[0]];
-        const int K = P.K;
-        nk = K >> 7;
-        xtile = P.qx + (int64_t)e[1] * K;
-        wtile = P.qw + (int64_t)e[2] * K;
-        voff = lane_offset(K);
-        bstep = (int64_t)32 * K;   // four blocks of eight rows
-        if constexpr (DEQ) {
-            if (wave * 64 < BM + BN) {
-                const float *src = wave * 64 < BM ? P.sx + e[1] + wave * 64 : P.sw + e[2] + (wave * 64 - BM);
-                dma4(src, (unsigned)opaque(lane0) * 4u, lds_base + scales_at + wave * 256);
-            }
-        }
-        if (loader) {
-            issue_x(0u, 0);
-            issue_w(0u, 0);
-            if (nk > 1) {
-                issue_x((unsigned)XSTAGE, 1);
-                issue_w((unsigned)WSTAGE, 1);
-            }
-        }
-        Epi ep;
-        ep.out = P.out;
-        ep.N = P.N;
-        ep.K = K;
-        ep.m0 = e[1];
-        ep.n0 = e[2];
-        return ep;
+        dma16(lw + (int64_t)lkt * 128 + (2 * p_) * lbstep, lvoff, lds_w + buf + (2 * p_) * 4096);
+        dma16(lw + (int64_t)lkt * 128 + (2 * p_ + 1) * lbstep, lvoff, lds_w + buf + (2 * p_ + 1) * 4096);
     };
 
-    v4i xb[TM], wa[R];
-    int kt = 0;
-    unsigned xo = 0, wo = 0;   // this lane's fragment addresses in activation buffer 0 / weight buffer 0
+    // ---- read side: fragment (16 rows, 64 K bytes): lane (r = l%16, g = l/16) reads row r, chunk 4*half + g
+    v4i xb[TM], wa[4];
+    unsigned xo0 = 0, xo1 = 0, wo0 = 0, wo1 = 0;   // this lane's fragment addresses in buffer 0, K half 0 / 1
+    {
+        const int l = opaque(lane0);
+        const int r = l & 15, g_ = l >> 4;
+        const int rho = r & 7, bpar = r >> 3;
+        const int sigma = (bpar << 2) | (rho >> 1);
+        const unsigned roff0 = bpar * 1024 + ((8 * rho + ((0 + g_) ^ sigma)) << 4);
+        const unsigned roff1 = bpar * 1024 + ((8 * rho + ((4 + g_) ^ sigma)) << 4);
+        xo0 = lds_base + wm * TM * 2048 + roff0;
+        xo1 = lds_base + wm * TM * 2048 + roff1;
+        wo0 = lds_base + XAREA + wn * TN * 2048 + roff0;
+        wo1 = lds_base + XAREA + wn * TN * 2048 + roff1;
+    }
+    // stage s of the stream lives in activation buffer s % 2 and weight buffer s % 3, for the whole life of the workgroup
     unsigned xcur = 0, xnxt = XSTAGE, wcur = 0, wnxt = WSTAGE, wnn = 2 * WSTAGE;
+
+    // ---- the tile being computed
+    int kt = 0, nk = 0;
+    bool first_tile = true;   // no stores of a tile before this one are in flight
+    unsigned cur_scales = C::SCALES_AT;   // two scale areas, by tile parity: the next tile's scales are requested in
+                                          // its first stage, when a slower wave may still be reading this tile's
 
     // one stage.  There is ONE copy of this code and one loop around it: a fragment register is written by an LDS
     // read the compiler cannot follow (its data arrives later), so no value of xb / wa may ever have to be moved
-    // where two paths of the control flow meet.  The last stage of a tile therefore also requests "next" fragments
-    // (from a buffer that holds nothing new; they are never used), and the accumulators start a tile at zero
-    // (cleared by the epilogue that read them) instead of a first stage that writes them.
+    // where two paths of the control flow meet.  The last stage of a workgroup therefore also requests "next"
+    // fragments (from a buffer that holds nothing new; they are never used).
     auto stage = [&]() {
-        const unsigned aw = add_vs(wo, wcur);
-        const bool more2 = kt + 2 < nk;
-        const bool ld2 = loader && more2, ld3 = loader && kt + 3 < nk;
-        // Loads of a stage, one at the head of a group so that a wave never issues two in a row:
-        //   group 0: weight part 2 of stage kt+2;  groups 1..LX: the activation parts of stage kt+2 (behind B1);
-        //   group LX+1: weight part 3 of stage kt+2;  group TN-2 (behind B2) and TN-1: weight parts 0, 1 of stage kt+3
-        static_for<TN>([&](auto J) {
-            constexpr int j = decltype(J)::value;
-            if constexpr (j == 0) {
-                if (ld2) issue_w1(std::integral_constant<int, 2>{}, wnn, kt + 2);
-            } else if constexpr (j <= LX) {
-                if (ld2) issue_x1(std::integral_constant<int, j - 1>{}, xcur, kt + 2);
-            } else if constexpr (j == LX + 1 && LW > 3) {
-                static_assert(LW <= 4 && LX + 1 < TN - 2);
-                if (ld2) issue_w1(std::integral_constant<int, 3>{}, wnn, kt + 2);
-            } else if constexpr (j == TN - 1) {
-                if (ld3) issue_w1(std::integral_constant<int, 1>{}, wcur, kt + 3);
-            }
-            if constexpr (j + 2 < TN) ds_read128<(j + 2) * 2048>(wa[(j + 2) % R], aw);
-            if constexpr (j == 0) {
-                // LDS returns in order: wa[0], wa[1], the activation fragments, then the read issued just now
-                static_for<TM>([&](auto I) {
-                    constexpr int i = decltype(I)::value;
-                    wait_lgkm<TM - i>();
-                    vacc::mfma_acc<4 * i>(wa[0], xb[i]);
-                });
-                // B1: every wave holds its activation fragments: the activation buffer is free for stage kt + 2
-                __builtin_amdgcn_s_barrier();
-            } else {
-                if constexpr (j == TN - 2) {
-                    // all reads of the current weight buffer have been issued: drain them and, in a loading wave,
-                    // its share of the next stage (memory operations complete in order: the loads of later stages
-                    // may stay in flight; whatever this wave stored for its previous tile lies before them)
-                    if (loader) {
-                        if (more2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * (LX + LW)) : "memory");
-                        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                    } else {
-                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    }
-                    __builtin_amdgcn_s_barrier();   // B2: stage kt+1 is visible, the weight buffer of stage kt is free
-                    if (ld3) issue_w1(std::integral_constant<int, 0>{}, wcur, kt + 3);
-                } else if constexpr (j < TN - 2) {
-                    wait_lgkm<2>();   // wa[j] is in; wa[j+1] and the read issued just now may stay in flight
-                }
-                if constexpr (j == TN - 1) {
-                    const unsigned nax = add_vs(xo, xnxt);
-                    static_for<TM>([&](auto I) {
-                        constexpr int i = decltype(I)::value;
-                        vacc::mfma_acc<4 * (j * TM + i)>(wa[j % R], xb[i]);
-                        ds_read128<i * 2048>(xb[i], nax);   // xb[i] has been read
-                    });
-                } else {
-                    static_for<TM>([&](auto I) {
-                        constexpr int i = decltype(I)::value;
-                        vacc::mfma_acc<4 * (j * TM + i)>(wa[j % R], xb[i]);
-                    });
-                }
-                if constexpr (j == TN - 2) {   // wa[0] and wa[1] were last read by groups before this one
-                    const unsigned naw = add_vs(wo, wnxt);
-                    ds_read128<0>(wa[0], naw);
-                    ds_read128<2048>(wa[1], naw);
-                }
-            }
+        const bool ld = loader && ldv;
+        const unsigned aw0 = add_vs(wo0, wcur), aw1 = add_vs(wo1, wcur);
+        auto group = [&](auto J, auto SLOT) {   // weight fragment in slot SLOT against the four activation fragments
+            static_for<TM>([&](auto I) {
+                vacc::mfma_acc<4 * (decltype(J)::value * TM + decltype(I)::value)>(wa[decltype(SLOT)::value], xb[decltype(I)::value]);
+            });
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        // ---- K half 0.  LDS operations in flight, oldest first: W0, W1, xb0..3 (requested by the stage before)
+        if (ld) issue_w(I0{}, wnn);
+        ds_read128<2 * 2048>(wa[2], aw0);
+        static_for<TM>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            wait_lgkm<4 - i>();   // xb[i] is in (and W0 before it)
+            vacc::mfma_acc<4 * i>(wa[0], xb[i]);
         });
+        if (ld) issue_w(I1{}, wnn);
+        ds_read128<3 * 2048>(wa[3], aw0);
+        group(I1{}, I1{});
+        if (ld) issue_w(I2{}, wnn);
+        ds_read128<4 * 2048>(wa[0], aw0);
+        wait_lgkm<2>();   // W2 is in; W3 and W4 may stay in flight
+        group(I2{}, I2{});
+        ds_read128<5 * 2048>(wa[1], aw0);
+        wait_lgkm<2>();   // W3 is in
+        group(I3{}, I3{});
+        // the last two groups, interleaved; the fragments of K half 1 are requested behind them
+        if (kt == 0 && loader) {   // this tile's scales, for the end of the tile
+            if constexpr (DEQ) {
+                const Problem &P = bt.p[e_p];
+                const float *s0 = P.sx + e_m0 + pw * 64;                                     // row scales 64 pw ..
+                const float *s1 = pw < 3 ? P.sw + e_n0 + pw * 64 : P.sx + e_m0 + pw * 64;   // column scales 64 pw .. (wave 3: none left)
+                const unsigned lo4 = (unsigned)opaque(lane0) * 4u;
+                dma4(s0, lo4, lds_base + cur_scales + pw * 256);
+                dma4(s1, lo4, lds_base + cur_scales + (pw < 3 ? BM * 4 + pw * 256 : pw * 256));
+            }
+        }
+        ds_read128<0>(wa[2], aw1);
+        ds_read128<2048>(wa[3], aw1);
+        wait_lgkm<2>();   // W4, W5 are in
+        {
+            const unsigned ax1 = add_vs(xo1, xcur);
+            static_for<TM>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                vacc::mfma_acc<4 * (4 * TM + i)>(wa[0], xb[i]);
+                vacc::mfma_acc<4 * (5 * TM + i)>(wa[1], xb[i]);
+                ds_read128<i * 2048>(xb[i], ax1);   // xb[i] has been read for the last time
+            });
+        }
+        // ---- K half 1.  In flight: W0', W1', xb0..3
+        ds_read128<2 * 2048>(wa[0], aw1);
+        static_for<TM>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            wait_lgkm<4 - i>();
+            vacc::mfma_acc<4 * i>(wa[2], xb[i]);
+        });
+        // B1: every wave holds its activation fragments of both halves: the activation buffer is free for stage + 2
+        __builtin_amdgcn_s_barrier();
+        if (ld) issue_x(I0{}, xcur);
+        ds_read128<3 * 2048>(wa[1], aw1);
+        group(I1{}, I3{});
+        if (ld) issue_x(I1{}, xcur);
+        ds_read128<4 * 2048>(wa[2], aw1);
+        wait_lgkm<2>();   // W2' is in
+        group(I2{}, I0{});
+        if (ld) issue_x(I2{}, xcur);
+        ds_read128<5 * 2048>(wa[3], aw1);
+        wait_lgkm<2>();   // W3' is in
+        group(I3{}, I1{});
+        // B2.  All reads of the current buffers have been issued: drain them and, in a loading wave, its share of
+        // the next stage.  Memory operations complete in order; issued since the last load of the next stage (the
+        // fourth activation part, behind B2 of the stage before): in a tile's first stage the NACC stores of the
+        // tile before it; this stage's three weight parts; in a tile's first stage its scales; three activation parts.
+        if (loader) {
+            constexpr int SC = DEQ ? 2 : 0;
+            if (!ldv) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(12 + SC + NACC) : "memory");
+            else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(12 + SC) : "memory");
+            else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_s_barrier();   // the next stage is visible, the weight buffer of this stage is free
+        if (ld) issue_x(I3{}, xcur);
+        {
+            const unsigned naw0 = add_vs(wo0, wnxt), nax0 = add_vs(xo0, xnxt);
+            ds_read128<0>(wa[0], naw0);
+            ds_read128<2048>(wa[1], naw0);
+            static_for<TM>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                vacc::mfma_acc<4 * (4 * TM + i)>(wa[2], xb[i]);
+                vacc::mfma_acc<4 * (5 * TM + i)>(wa[3], xb[i]);
+                ds_read128<i * 2048>(xb[i], nax0);
+            });
+        }
         {
             const unsigned t = xcur; xcur = xnxt; xnxt = t;
             const unsigned u = wcur; wcur = wnxt; wnxt = wnn; wnn = u;
         }
     };
-    static_assert(LW >= 3 && (TN - 1) % R >= 2 && (TN - 2) % R != 0 && LX <= TN - 2,
-                  "the last group must not use wa[0] or wa[1], nor the one before it wa[0]");
+    static_assert(12 + 2 + NACC + 2 <= 63, "the memory counter has six bits");
 
-    // ---- the two partial sums of a wave tile meet.  Wave `half` finishes row tiles i in [half*IH, +IH) of every
-    // column tile; a round hands one row tile of two neighbouring column tiles to the partner (2 KB, two parcel
-    // areas in turn: one barrier a round), adds the partner's parcel to its own accumulators and stores the pair:
-    // 8 rows x 128 B per store instruction.  Both forms are compiled and a scalar branch picks one, so that every
-    // accumulator register is named by a constant.
-    auto finish = [&](auto HALF, const Epi &e, unsigned scales_at) {
-        constexpr int hf = decltype(HALF)::value;
-        constexpr int NR = IH * (TN / 2);   // rounds
+    // The tile's accumulators leave: converted, scaled by the row and the column scale, stored and cleared for the
+    // next tile; accumulator (j, i) is named at compile time.  Two neighbouring column tiles are paired and swap
+    // halves between lanes r and r ^ 8, so that a store instruction writes 8 rows x 128 B: whole cache lines
+    // (stores of 16 rows x 64 B, half lines, cost three times as much here and slowed the next tile's loads).  The first
+    // fragments of the next tile are in flight the whole time (6 LDS reads that the waits below count).
+    auto finish_tile = [&](const void *out, int N, int m0, int n0, unsigned scales_at) {
         const int l = opaque(lane0);
         const int r = l & 15, g_ = l >> 4;
-        const bool lo = r < 8;
-        const float *const s_sx = reinterpret_cast<const float *>(smem + scales_at);
-        const float *const s_sw = s_sx + BM;
-        float *const y = static_cast<float *>(e.out);
-        int32_t *const acc_out = static_cast<int32_t *>(e.out);
-        const int N = e.N;
-        const unsigned mine = lds_base + C::PARCELS_AT + wave * C::PARCEL + l * 16;
-        const unsigned theirs = lds_base + C::PARCELS_AT + (wave ^ 4) * C::PARCEL + l * 16;
-        const int ncol = e.n0 + wn * TN * 16 + (lo ? 0 : 16) + 4 * g_;
-        float4 sw4[TN / 2];
-#pragma unroll
-        for (int rd = 0; rd < TN / 2; ++rd) {
-            sw4[rd] = float4{1.0f, 1.0f, 1.0f, 1.0f};
-            if constexpr (DEQ) sw4[rd] = *reinterpret_cast<const float4 *>(s_sw + (wn * TN + 2 * rd) * 16 + (lo ? 0 : 16) + 4 * g_);
+        const unsigned asx = lds_base + scales_at + (unsigned)((wm * 64 + (r & 7)) * 4);
+        const unsigned asw = lds_base + scales_at + BM * 4 + (unsigned)((wn * 96 + 4 * g_) * 4);
+        float sxA[TM], sxB[TM];   // row r % 8 and row 8 + r % 8 of each 16-row tile
+        v4f sw4 = {1.0f, 1.0f, 1.0f, 1.0f};
+        if constexpr (DEQ) {
+            static_for<TM>([&](auto I) {
+                lds_read32(sxA[decltype(I)::value], asx + 64 * decltype(I)::value);
+                lds_read32(sxB[decltype(I)::value], asx + 64 * decltype(I)::value + 32);
+            });
         }
-        // round rnd = ii * (TN/2) + rd: row tile ii of this wave's half, column tiles 2rd and 2rd+1
-        auto hand_over = [&](auto RND) {
-            constexpr int rnd = decltype(RND)::value;
-            if constexpr (rnd < NR) {
-                constexpr int ii = rnd / (TN / 2), rd = rnd % (TN / 2);
-                constexpr int ip = (1 - hf) * IH + ii;
-                constexpr int area = (rnd & 1) * 8 * C::PARCEL;
-                vacc::acc_to_lds<4 * ((2 * rd) * TM + ip), area>(mine);
-                vacc::acc_to_lds<4 * ((2 * rd + 1) * TM + ip), area + 1024>(mine);
-            }
-        };
-        hand_over(std::integral_constant<int, 0>{});
-        static_for<NR>([&](auto RND) {
-            constexpr int rnd = decltype(RND)::value;
-            constexpr int ii = rnd / (TN / 2), rd = rnd % (TN / 2);
-            constexpr int i = hf * IH + ii, ip = (1 - hf) * IH + ii;
-            constexpr int area = (rnd & 1) * 8 * C::PARCEL;
-            // the parcels of this round are in LDS (the compiler does not count the asm's LDS writes), and every
-            // wave has read what it wanted from the round before the last: the other area is free again
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            v4i o0, o1;
-            ds_read128<area>(o0, theirs);
-            ds_read128<area + 1024>(o1, theirs);
-            hand_over(std::integral_constant<int, rnd + 1>{});   // under the latency of the reads above
-            float sxA = 1.0f, sxB = 1.0f;
+        const char *const base = static_cast<const char *>(out) + ((int64_t)m0 * N + n0) * 4;
+        const int64_t rows16 = (int64_t)64 * N;   // bytes from one 16-row tile to the next
+        const int64_t rows8 = (int64_t)32 * N;
+        const bool lo = r < 8;
+        // this lane's place in a store of 8 rows x 128 B: row r % 8, and the 16 bytes 4g of column tile j (lanes
+        // r < 8) or of column tile j + 1 (lanes r >= 8)
+        unsigned vo = (unsigned)(((wm * 64 + (r & 7)) * N + wn * 96 + (lo ? 0 : 16) + 4 * g_) * 4);
+        const unsigned asw2 = asw + (lo ? 0u : 64u);
+        static_for<TN / 2>([&](auto JP) {
+            constexpr int j = 2 * decltype(JP)::value;
             if constexpr (DEQ) {
-                const float *tsx = s_sx + (wm * TM + i) * 16;
-                sxA = tsx[r & 7];
-                sxB = tsx[8 + (r & 7)];
+                lds_read128f(sw4, asw2 + 64 * j);
+                wait_lgkm<0>();
             }
-            const int mA = e.m0 + (wm * TM + i) * 16 + (r & 7);
-            const int64_t at = (int64_t)mA * N + ncol + rd * 32;
-            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(rnd + 1 < NR ? 2 : 0) : "memory");   // o0, o1 are in
-            const v4i a0 = vacc::acc_plus<4 * ((2 * rd) * TM + i)>(o0);
-            const v4i a1 = vacc::acc_plus<4 * ((2 * rd + 1) * TM + i)>(o1);
-            v4i t0, t1;
+            // the matrix instructions of the stage's last two groups wrote column tiles 4 and 5 a moment ago
+            if constexpr (j == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+            static_for<TM>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                constexpr int r0 = vacc::ACC0 + 4 * (j * TM + i), r1 = vacc::ACC0 + 4 * ((j + 1) * TM + i);
+                const char *sbase = base + i * rows16 + j * 64;
+                const char *sbase8 = sbase + rows8;
+                const unsigned vo_ = vo;   // (named outside the asm so that the lambda captures it)
+                // a0: column tile j, a1: column tile j + 1 of row tile i, read and cleared
+                v4i a0, a1;
+                asm volatile("v_mov_b32 %0, v%c4\n\tv_mov_b32 %1, v%c5\n\tv_mov_b32 %2, v%c6\n\tv_mov_b32 %3, v%c7\n\t"
+                             "v_mov_b32 v%c4, 0\n\tv_mov_b32 v%c5, 0\n\tv_mov_b32 v%c6, 0\n\tv_mov_b32 v%c7, 0"
+                             : "=&v"(a0[0]), "=&v"(a0[1]), "=&v"(a0[2]), "=&v"(a0[3])
+                             : "n"(r0), "n"(r0 + 1), "n"(r0 + 2), "n"(r0 + 3));
+                asm volatile("v_mov_b32 %0, v%c4\n\tv_mov_b32 %1, v%c5\n\tv_mov_b32 %2, v%c6\n\tv_mov_b32 %3, v%c7\n\t"
+                             "v_mov_b32 v%c4, 0\n\tv_mov_b32 v%c5, 0\n\tv_mov_b32 v%c6, 0\n\tv_mov_b32 v%c7, 0"
+                             : "=&v"(a1[0]), "=&v"(a1[1]), "=&v"(a1[2]), "=&v"(a1[3])
+                             : "n"(r1), "n"(r1 + 1), "n"(r1 + 2), "n"(r1 + 3));
+                v4i t0, t1;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                t0[q] = ror8(a0[q]);
-                t1[q] = ror8(a1[q]);
-            }
-            const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile 2rd (own), lanes r>=8 tile 2rd+1 (from lane r-8)
-            const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile 2rd+1 (own), lanes r<8 tile 2rd (from lane r+8)
-            store4<DEQ>(y, acc_out, at, vA, sxA, sw4[rd]);
-            store4<DEQ>(y, acc_out, at + (int64_t)8 * N, vB, sxB, sw4[rd]);
-            // the two accumulators of this wave's own row tile have been read: they start the next tile at zero
-            // (the two that were handed over are cleared once their LDS writes are known to be done: next round)
-            vacc::acc_zero4<4 * ((2 * rd) * TM + i)>();
-            vacc::acc_zero4<4 * ((2 * rd + 1) * TM + i)>();
-        });
-        // every LDS write of the hand-overs has completed (each round waited for the previous ones)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        static_for<IH * TN>([&](auto Q) {
-            constexpr int q = decltype(Q)::value;
-            constexpr int j = q / IH, ii = q % IH;
-            vacc::acc_zero4<4 * (j * TM + (1 - hf) * IH + ii)>();
+                for (int q = 0; q < 4; ++q) {
+                    t0[q] = ror8(a0[q]);
+                    t1[q] = ror8(a1[q]);
+                }
+                const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
+                const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
+                if constexpr (DEQ) {
+                    // rows 0-7 use the scale of row r % 8, rows 8-15 that of row 8 + r % 8 of this 16-row tile
+                    v4f fA, fB;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        fA[q] = ((float)vA[q] * sxA[i]) * sw4[q];
+                        fB[q] = ((float)vB[q] * sxB[i]) * sw4[q];
+                    }
+                    asm volatile("global_store_dwordx4 %0, %1, %2" MI_STORE_MOD "\n\ts_nop 2" ::"v"(vo_), "v"(fA), "s"(sbase) : "memory");
+                    asm volatile("global_store_dwordx4 %0, %1, %2" MI_STORE_MOD "\n\ts_nop 2" ::"v"(vo_), "v"(fB), "s"(sbase8) : "memory");
+                } else {
+                    asm volatile("global_store_dwordx4 %0, %1, %2" MI_STORE_MOD "\n\ts_nop 2" ::"v"(vo_), "v"(vA), "s"(sbase) : "memory");
+                    asm volatile("global_store_dwordx4 %0, %1, %2" MI_STORE_MOD "\n\ts_nop 2" ::"v"(vo_), "v"(vB), "s"(sbase8) : "memory");
+                }
+                // (the wait states behind a store: a store of more than 8 bytes reads its data registers for a few
+                // cycles after it has issued, and the vector instruction behind an asm statement may already write
+                // them; the compiler pads this for its own stores only.  In front of it none are needed as long as the
+                // build lets no scalar be spilled: a scalar brought back by v_readlane may be read by a memory
+                // instruction only five wait states later, and the compiler cannot see the asm's memory instruction.)
+            });
         });
     };
 
-    Epi ce = begin_tile(ent, (unsigned)C::SCALES_AT);
-    bool first = true;
+    // ---- fill: stages 0 and 1 of the first tile, then its first fragments
+    cursor_to((v4i){e_p, e_m0, e_n0, 0});
+    nk = bt.p[e_p].K >> 7;
+    if (loader) {
+        static_for<4>([&](auto I) { issue_x(I, 0u); });
+        static_for<3>([&](auto I) { issue_w(I, 0u); });
+        lkt = 1;
+        static_for<4>([&](auto I) { issue_x(I, (unsigned)XSTAGE); });
+        static_for<3>([&](auto I) { issue_w(I, (unsigned)WSTAGE); });
+        wait_vm<14>();   // stage 0 has landed
+    }
+    lkt = 2;
+    __syncthreads();
+    ds_read128<0>(wa[0], wo0);
+    ds_read128<2048>(wa[1], wo0);
+    static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb[decltype(I)::value], xo0); });
+
     for (int it = 0;; ++it) {
-        const unsigned scales_at = (unsigned)(C::SCALES_AT + (it & 1) * C::SCALES);
-        // ---- stage 0 (and the scales before it) have landed when at most stage 1 and, behind it, the stores of
-        // the previous tile are still in flight
-        if (loader) {
-            if (first) {
-                if (nk > 1) wait_vm<2 * (LX + LW)>();
-                else wait_vm<0>();
-            } else {
-                if (nk > 1) wait_vm<2 * (LX + LW) + NS>();
-                else wait_vm<NS>();
-            }
-        } else {
-            if (first) wait_vm<0>();
-            else wait_vm<NS>();
-        }
-        __syncthreads();   // also: every wave has left the previous tile's last exchange round (third weight buffer)
+        cur_scales = (unsigned)(C::SCALES_AT + (it & 1) * C::SCALES);
+        // (the list is read again where the next entry is needed: it is not worth four scalar registers for a tile)
+        const bool more = sload4(my + it + 1)[0] >= 0;
+        bool in_cur = true;   // the cursor stands in this tile (it entered it two stages ago)
 #ifdef MI_GEMM_TIMELINE
         const unsigned long long tl_a = __builtin_amdgcn_s_memtime(), tl_ra = __builtin_amdgcn_s_memrealtime();
 #endif
-        xcur = 0; xnxt = XSTAGE; wcur = 0; wnxt = WSTAGE; wnn = 2 * WSTAGE;
-        voff = lane_offset(ce.K);
-        if (loader && nk > 2) {   // the first two parts of stage 2; stage 0 issues the rest (as stage kt does for kt + 2)
-            issue_w1(std::integral_constant<int, 0>{}, wnn, 2);
-            issue_w1(std::integral_constant<int, 1>{}, wnn, 2);
+        for (kt = 0; kt < nk; ++kt) {
+            stage();
+            // the cursor moves on: to the next stage of its tile, to the next tile, or off the end of the list
+            if (ldv && ++lkt == lnk) {
+                if (in_cur && more) cursor_to(sload4(my + it + 1));
+                else ldv = false;
+                in_cur = false;
+            }
         }
-        {   // read side: fragment (16 rows, this wave's K half): lane (r = l%16, g = l/16) reads row r, chunk 4*half + g
-            const int l = opaque(lane0);
-            const int r = l & 15, g_ = l >> 4;
-            const int rho = r & 7, bpar = r >> 3;
-            const int sigma = (bpar << 2) | (rho >> 1);
-            const unsigned roff = bpar * 1024 + ((8 * rho + ((4 * half + g_) ^ sigma)) << 4);
-            xo = lds_base + wm * TM * 2048 + roff;
-            wo = lds_base + XAREA + wn * TN * 2048 + roff;
-        }
-        {   // first fragments of stage 0, in the order every later stage requests them
-            ds_read128<0>(wa[0], wo);
-            ds_read128<2048>(wa[1], wo);
-            static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb[decltype(I)::value], xo); });
-        }
-#ifdef MI_GEMM_TIMELINE
-        const int nk_done = nk;
-#endif
-        for (kt = 0; kt < nk; ++kt) stage();
-        // everything of this wave is home; 2 x 16 wait states cover the longest MFMA-result -> read hazard
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\ns_nop 15\ns_nop 15" ::: "memory");
-        __syncthreads();   // every wave is done with the stage buffers
 #ifdef MI_GEMM_TIMELINE
         const unsigned long long tl_b = __builtin_amdgcn_s_memtime();
 #endif
-
-        // ---- the next tile's first stages go out, then this tile's sums meet and leave
-        ent = sload4(my + it + 1);
-        const bool more = ent[0] >= 0;
-        Epi ne = ce;
-        if (more) ne = begin_tile(ent, (unsigned)(C::SCALES_AT + ((it + 1) & 1) * C::SCALES));
-#ifdef MI_GEMM_TIMELINE
-        const unsigned long long tl_b2 = __builtin_amdgcn_s_memtime();
-#endif
-        if (half == 0) finish(std::integral_constant<int, 0>{}, ce, scales_at);
-        else finish(std::integral_constant<int, 1>{}, ce, scales_at);
+        {
+            const Problem &P = bt.p[e_p];
+            if (!more) {
+                // nothing follows: the scales must be visible whatever the tile's length, and no load is in flight
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
+            finish_tile(P.out, P.N, e_m0, e_n0, cur_scales);
+        }
 #ifdef MI_GEMM_TIMELINE
         {
             const unsigned long long tl_c = __builtin_amdgcn_s_memtime(), tl_rc = __builtin_amdgcn_s_memrealtime();
             if (wave == 0 && opaque(lane0) == 0 && blockIdx.x < TL_WGS && it < TL_TILES) {
                 unsigned long long *o = g_list_timeline + ((size_t)blockIdx.x * TL_TILES + it) * 8;
-                o[0] = tl_a;    // first stage in LDS (ticks)
-                o[1] = tl_b;    // stage loop done
-                o[2] = tl_c;    // last store issued, next tile's first stages requested
+                o[0] = tl_a;    // first stage begins (ticks)
+                o[1] = tl_b;    // last stage issued
+                o[2] = tl_c;    // last store issued
                 o[3] = tl_ra;   // real time (100 MHz) at o[0]
                 o[4] = tl_rc;   // real time at o[2]
-                o[5] = (unsigned long long)nk_done;
+                o[5] = (unsigned long long)nk;
                 o[6] = 1;
-                o[7] = tl_b2;   // next tile's first stages requested
+                o[7] = tl_b;
             }
         }
 #endif
         if (!more) break;
-        ce = ne;
-        first = false;
+        first_tile = false;
+        const v4i e = sload4(my + it + 1);
+        e_p = e[0];
+        e_m0 = e[1];
+        e_n0 = e[2];
+        nk = bt.p[e_p].K >> 7;
     }
 }
 
@@ -476,7 +503,7 @@ struct Tile {
     int p, m0, n0, cost;
 };
 
-// cost of a tile in K stages: its stage loop plus the exchange and stores
+// cost of a tile in K stages, plus its conversion and stores (measured: 8.7 k ticks against 2.3 k a stage)
 static inline int tile_cost(int64_t K) { return (int)(K / 128) + 4; }
 
 template <int BM, int BN>
@@ -529,15 +556,14 @@ static int64_t build_lists(const int64_t *mnk, int n, int cus, std::vector<v4i> 
     return (int64_t)cus * per_wg * (int64_t)sizeof(v4i);
 }
 
-constexpr int TM_ = 8, TN_ = 6;
-using LC = Cfg<TM_, TN_>;
+using LC = Cfg;
 
 static int32_t check_shapes(const int64_t *mnk, int32_t n)
 {
     if (!mnk || n < 1 || n > MAX_PROBLEMS) return MI_EINVAL;
     for (int p = 0; p < n; ++p) {
         const int64_t M = mnk[3 * p], N = mnk[3 * p + 1], K = mnk[3 * p + 2];
-        if (M < LC::BM || N < LC::BN || K < 128 || K % 128 || N % 16) return MI_EINVAL;
+        if (M < LC::BM || N < LC::BN || K < 128 * LC::MIN_STAGES || K % 128 || N % 16) return MI_EINVAL;
         if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MI_ERANGE;
         if ((int64_t)127 * 127 * K > 0x7fffffffLL) return MI_ERANGE;   // int32 accumulator bound
     }
@@ -641,12 +667,12 @@ static int32_t batch_run(mi_gemm_batch *b, const mi_gemm_problem *p, void *strea
     int dev = -1;
     MI_HIP(hipGetDevice(&dev));
     if (dev != b->device) return MI_EINVAL;   // the list lives in that device's memory
-    const void *fn = reinterpret_cast<const void *>(&list::k_w8a8_list<list::TM_, list::TN_, DEQ>);
+    const void *fn = reinterpret_cast<const void *>(&list::k_w8a8_list<DEQ>);
     if (!b->attr_set[DEQ].load(std::memory_order_acquire)) {
         MI_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, list::LC::LDS));
         b->attr_set[DEQ].store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((list::k_w8a8_list<list::TM_, list::TN_, DEQ>), dim3((unsigned)b->grid), dim3(512), list::LC::LDS,
+    hipLaunchKernelGGL((list::k_w8a8_list<DEQ>), dim3((unsigned)b->grid), dim3(512), list::LC::LDS,
                        as_stream(stream), bt, b->lists, b->per_wg);
     return launch_status();
 }

@@ -25,22 +25,24 @@ def make_ops(dev, shapes, seed, dtype):
     return ops, host
 
 
-# K of 1 to 7 stages walks every branch of the prologue, of the waits of a tile's first stages and of its last
-# stages; shapes that are no multiple of the tile exercise the tiles that are moved inwards (rows: 300 = 256 + 44,
-# columns: 272 = 192 + 80, 14336 = 74 * 192 + 128); several tiles per workgroup exercise the prefetch of the next
-# tile under the exchange of the current one and the hand-over of the accumulators at zero.
+# K of 3 to 7 stages (short tiles: the tile before them is not drained by the time they end) and of 24, 25 and 32
+# (the previous tile's 24 accumulators leave one per stage); shapes that are no multiple of the tile exercise the
+# tiles that are moved inwards (rows: 300 = 256 + 44, columns: 272 = 192 + 80, 14336 = 74 * 192 + 128); several tiles
+# per workgroup exercise the load stream across tile boundaries, both accumulator sets and the clearing of a
+# drained set; mixed K in one batch exercises a cursor that changes its stride between tiles.
 @pytest.mark.parametrize("shapes", [
-    [(256, 192, 128)],
-    [(256, 192, 256)],
     [(256, 192, 384)],
-    [(300, 272, 512)],
-    [(2048, 6144, 128)],
-    [(2048, 6144, 640)],
-    [(2048, 14336, 256)],
-    [(4096, 4096, 384)],
-    [(512, 384, 896), (256, 208, 128)],
-    [(2048, 6144, 256), (2048, 4096, 896), (264, 14336, 128)],
-    [(1024, 1152, 256)] * 8,
+    [(256, 192, 512)],
+    [(300, 272, 640)],
+    [(2048, 6144, 384)],
+    [(2048, 6144, 896)],
+    [(2048, 14336, 384)],
+    [(4096, 4096, 512)],
+    [(2048, 4608, 3072)],
+    [(2048, 6144, 3200)],
+    [(512, 384, 896), (256, 208, 384)],
+    [(2048, 6144, 384), (2048, 4096, 4096), (264, 14336, 512)],
+    [(1024, 1152, 768)] * 8,
 ])
 def test_batch_accumulators_bit_exact(mi, dev, orc, shapes):
     mark = dev.mark()
@@ -57,9 +59,10 @@ def test_batch_accumulators_bit_exact(mi, dev, orc, shapes):
 
 
 @pytest.mark.parametrize("shapes", [
-    [(256, 192, 128)],
+    [(256, 192, 384)],
     [(300, 272, 512)],
     [(2048, 6144, 384), (520, 4096, 1024)],
+    [(2048, 6144, 4096)],
 ])
 def test_batch_dequant_equals_the_oracle_and_the_single_call(mi, dev, orc, shapes):
     mark = dev.mark()
@@ -110,16 +113,17 @@ def test_batch_rejects_what_it_cannot_run(mi, dev):
         arr = (i64 * (3 * len(shapes)))(*[v for s in shapes for v in s])
         return mi.lib.mi_gemm_batch_plan_bytes(arr, len(shapes))
 
-    assert plan_bytes([(255, 192, 128)]) == mi.EINVAL      # fewer rows than a tile
-    assert plan_bytes([(256, 176, 128)]) == mi.EINVAL      # fewer columns than a tile
-    assert plan_bytes([(256, 200, 128)]) == mi.EINVAL      # N % 16
-    assert plan_bytes([(256, 192, 192)]) == mi.EINVAL      # K % 128
-    assert plan_bytes([(256, 192, 128)] * 9) == mi.EINVAL  # more than eight problems
+    assert plan_bytes([(255, 192, 384)]) == mi.EINVAL      # fewer rows than a tile
+    assert plan_bytes([(256, 176, 384)]) == mi.EINVAL      # fewer columns than a tile
+    assert plan_bytes([(256, 200, 384)]) == mi.EINVAL      # N % 16
+    assert plan_bytes([(256, 192, 448)]) == mi.EINVAL      # K % 128
+    assert plan_bytes([(256, 192, 256)]) == mi.EINVAL      # fewer than three K stages
+    assert plan_bytes([(256, 192, 384)] * 9) == mi.EINVAL  # more than eight problems
     assert plan_bytes([(256, 192, 1 << 18)]) == mi.ERANGE  # the int32 accumulator could overflow
-    assert plan_bytes([(256, 192, 128)]) > 0
+    assert plan_bytes([(256, 192, 384)]) > 0
     mark = dev.mark()
-    batch = mi.GemmBatch(dev, [(256, 192, 128)])
-    qx, qw, out = dev.empty((256, 256), np.int8), dev.empty((192, 256), np.int8), dev.empty((256, 192), np.int32)
+    batch = mi.GemmBatch(dev, [(256, 192, 384)])
+    qx, qw, out = dev.empty((256, 512), np.int8), dev.empty((192, 512), np.int8), dev.empty((256, 192), np.int32)
     with pytest.raises(mi.MiError) as e:   # K differs from the batch's
         batch.run_i32([(qx, None, qw, None, out)])
     assert e.value.status == mi.EINVAL
