@@ -23,13 +23,12 @@
 //
 // Waves: 8 = 4 (rows) x 2 (columns), two per SIMD; wave tile 4 x 6 matrix-instruction tiles.  A 128-byte K stage
 // is two halves of 64 bytes; a half is six groups (one weight fragment against the four activation fragments).
-// LDS layout, swizzle and load shapes are those of gemm_pair.hip.  Per wave and half: 6 weight fragment reads
-// (through four register slots, two groups ahead) and 4 activation fragment reads (each right behind the last
-// matrix instruction that reads the old fragment; the last two groups of a half are interleaved so that the first
-// reload is 6 instructions ahead of its use).
+// LDS layout, swizzle and load shapes are those of gemm_pair.hip.  Per wave and half: 6 weight and 4 activation
+// fragment reads, all of them requested half a stage before they are used (see the stage below), and ONE barrier
+// a stage.
 //
-// Registers: v[64..159] are the accumulators, named by hand; the kernel is limited to v0..v63 for everything the
-// compiler places (see gemm_pair_ops.h).
+// Registers: v[160..255] are the accumulators, named by hand; the kernel is limited to v0..v159 for everything the
+// compiler places (see gemm_pair_ops.h): fragments for two K halves and the addresses.
 //
 // Memory operations complete in issue order (one counter for loads and stores), and every wait below is written
 // against that order.  Only waves 0..3 (the ones the matrix pipe serves first) issue loads; every wave stores its
@@ -153,9 +152,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     constexpr int XSTAGE = C::XSTAGE, WSTAGE = C::WSTAGE, XAREA = C::XAREA;
     constexpr int NACC = C::NACC;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    // v[64 .. 255] are this kernel's accumulators, named by hand: the attribute above keeps everything the compiler
-    // places below v64, and this clobber makes the wave's register count cover them
-    asm volatile("" ::: "v64", "v255");
+    // v[160 .. 255] are this kernel's accumulators, named by hand: the attribute above keeps everything the compiler
+    // places below v160, and this clobber makes the wave's register count cover them
+    asm volatile("" ::: "v160", "v255");
 
     const int tid = threadIdx.x, lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -211,7 +210,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     };
 
     // ---- read side: fragment (16 rows, 64 K bytes): lane (r = l%16, g = l/16) reads row r, chunk 4*half + g
-    v4i xb[TM], wa[4];
+    v4i xa[TM], xc[TM], w[TN];   // activation fragments of a first / second K half, weight fragments
     unsigned xo0 = 0, xo1 = 0, wo0 = 0, wo1 = 0;   // this lane's fragment addresses in buffer 0, K half 0 / 1
     {
         const int l = opaque(lane0);
@@ -235,106 +234,83 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                                           // its first stage, when a slower wave may still be reading this tile's
 
     // one stage.  There is ONE copy of this code and one loop around it: a fragment register is written by an LDS
-    // read the compiler cannot follow (its data arrives later), so no value of xb / wa may ever have to be moved
+    // read the compiler cannot follow (its data arrives later), so no value of xa / xc / w may ever have to be moved
     // where two paths of the control flow meet.  The last stage of a workgroup therefore also requests "next"
     // fragments (from a buffer that holds nothing new; they are never used).
+    //
+    // Fragments are requested half a stage ahead: while the six groups of a K half run, the four activation
+    // fragments of the next half arrive in the other activation set (xa: first halves, xc: second halves) and weight
+    // fragment k of the next half is requested into w[k] right behind group k, the last reader of the old w[k].
+    // One barrier a stage, behind the first group of the second half: by then every read of this stage's buffers has
+    // been issued (the second half's fragments during the first half) and, at the barrier, has landed; behind it the
+    // next stage's buffers are read, the activation buffer takes the loads of stage + 2, and the weight buffer is
+    // free for the stage after that (its loads are issued during the next stage's first half).
     auto stage = [&]() {
         const bool ld = loader && ldv;
-        const unsigned aw0 = add_vs(wo0, wcur), aw1 = add_vs(wo1, wcur);
-        auto group = [&](auto J, auto SLOT) {   // weight fragment in slot SLOT against the four activation fragments
-            static_for<TM>([&](auto I) {
-                vacc::mfma_acc<4 * (decltype(J)::value * TM + decltype(I)::value)>(wa[decltype(SLOT)::value], xb[decltype(I)::value]);
-            });
-        };
         using I0 = std::integral_constant<int, 0>;
         using I1 = std::integral_constant<int, 1>;
         using I2 = std::integral_constant<int, 2>;
         using I3 = std::integral_constant<int, 3>;
-        // ---- K half 0.  LDS operations in flight, oldest first: W0, W1, xb0..3 (requested by the stage before)
-        if (ld) issue_w(I0{}, wnn);
-        ds_read128<2 * 2048>(wa[2], aw0);
-        static_for<TM>([&](auto I) {
-            constexpr int i = decltype(I)::value;
-            wait_lgkm<4 - i>();   // xb[i] is in (and W0 before it)
-            vacc::mfma_acc<4 * i>(wa[0], xb[i]);
-        });
-        if (ld) issue_w(I1{}, wnn);
-        ds_read128<3 * 2048>(wa[3], aw0);
-        group(I1{}, I1{});
-        if (ld) issue_w(I2{}, wnn);
-        ds_read128<4 * 2048>(wa[0], aw0);
-        wait_lgkm<2>();   // W2 is in; W3 and W4 may stay in flight
-        group(I2{}, I2{});
-        ds_read128<5 * 2048>(wa[1], aw0);
-        wait_lgkm<2>();   // W3 is in
-        group(I3{}, I3{});
-        // the last two groups, interleaved; the fragments of K half 1 are requested behind them
-        if (kt == 0 && loader) {   // this tile's scales, for the end of the tile
-            if constexpr (DEQ) {
-                const Problem &P = bt.p[e_p];
-                const float *s0 = P.sx + e_m0 + pw * 64;                                     // row scales 64 pw ..
-                const float *s1 = pw < 3 ? P.sw + e_n0 + pw * 64 : P.sx + e_m0 + pw * 64;   // column scales 64 pw .. (wave 3: none left)
-                const unsigned lo4 = (unsigned)opaque(lane0) * 4u;
-                dma4(s0, lo4, lds_base + cur_scales + pw * 256);
-                dma4(s1, lo4, lds_base + cur_scales + (pw < 3 ? BM * 4 + pw * 256 : pw * 256));
-            }
-        }
-        ds_read128<0>(wa[2], aw1);
-        ds_read128<2048>(wa[3], aw1);
-        wait_lgkm<2>();   // W4, W5 are in
+        // ---- K half 0 (fragments xa, w).  In flight, oldest first, from the stage before:
+        //      W0 | x0 W1 | x1 W2 | x2 W3 | x3 W4 | W5
         {
-            const unsigned ax1 = add_vs(xo1, xcur);
-            static_for<TM>([&](auto I) {
-                constexpr int i = decltype(I)::value;
-                vacc::mfma_acc<4 * (4 * TM + i)>(wa[0], xb[i]);
-                vacc::mfma_acc<4 * (5 * TM + i)>(wa[1], xb[i]);
-                ds_read128<i * 2048>(xb[i], ax1);   // xb[i] has been read for the last time
+            const unsigned ax1 = add_vs(xo1, xcur), aw1 = add_vs(wo1, wcur);
+            static_for<TN>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                if constexpr (j < TM) ds_read128<j * 2048>(xc[j], ax1);
+                if constexpr (j < 3) {
+                    if (ld) issue_w(J, wnn);
+                }
+                if constexpr (j == 0) wait_lgkm<3>();        // x0..x3 and W0..W3 are in; W4, W5 and the read above may not be
+                if constexpr (j >= 4) wait_lgkm<9>();        // W4 (W5) is in: 8 reads of this half and W5 (W4') are younger
+                if constexpr (j == 4) {
+                    if (kt == 0 && loader) {   // this tile's scales, for the end of the tile
+                        if constexpr (DEQ) {
+                            const Problem &P = bt.p[e_p];
+                            const float *s0 = P.sx + e_m0 + pw * 64;                                     // row scales 64 pw ..
+                            const float *s1 = pw < 3 ? P.sw + e_n0 + pw * 64 : P.sx + e_m0 + pw * 64;   // column scales 64 pw .. (wave 3: none left)
+                            const unsigned lo4 = (unsigned)opaque(lane0) * 4u;
+                            dma4(s0, lo4, lds_base + cur_scales + pw * 256);
+                            dma4(s1, lo4, lds_base + cur_scales + (pw < 3 ? BM * 4 + pw * 256 : pw * 256));
+                        }
+                    }
+                }
+                static_for<TM>([&](auto I) {
+                    vacc::mfma_acc<4 * (j * TM + decltype(I)::value)>(w[j], xa[decltype(I)::value]);
+                });
+                ds_read128<j * 2048>(w[j], aw1);   // w[j] has been read for the last time
             });
         }
-        // ---- K half 1.  In flight: W0', W1', xb0..3
-        ds_read128<2 * 2048>(wa[0], aw1);
-        static_for<TM>([&](auto I) {
-            constexpr int i = decltype(I)::value;
-            wait_lgkm<4 - i>();
-            vacc::mfma_acc<4 * i>(wa[2], xb[i]);
-        });
-        // B1: every wave holds its activation fragments of both halves: the activation buffer is free for stage + 2
-        __builtin_amdgcn_s_barrier();
-        if (ld) issue_x(I0{}, xcur);
-        ds_read128<3 * 2048>(wa[1], aw1);
-        group(I1{}, I3{});
-        if (ld) issue_x(I1{}, xcur);
-        ds_read128<4 * 2048>(wa[2], aw1);
-        wait_lgkm<2>();   // W2' is in
-        group(I2{}, I0{});
-        if (ld) issue_x(I2{}, xcur);
-        ds_read128<5 * 2048>(wa[3], aw1);
-        wait_lgkm<2>();   // W3' is in
-        group(I3{}, I1{});
-        // B2.  All reads of the current buffers have been issued: drain them and, in a loading wave, its share of
-        // the next stage.  Memory operations complete in order; issued since the last load of the next stage (the
-        // fourth activation part, behind B2 of the stage before): in a tile's first stage the NACC stores of the
-        // tile before it; this stage's three weight parts; in a tile's first stage its scales; three activation parts.
-        if (loader) {
-            constexpr int SC = DEQ ? 2 : 0;
-            if (!ldv) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(12 + SC + NACC) : "memory");
-            else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(12 + SC) : "memory");
-            else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
-        } else {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        }
-        __builtin_amdgcn_s_barrier();   // the next stage is visible, the weight buffer of this stage is free
-        if (ld) issue_x(I3{}, xcur);
+        // ---- K half 1 (fragments xc, w).  In flight: x0 W0 | x1 W1 | x2 W2 | x3 W3 | W4 | W5
         {
-            const unsigned naw0 = add_vs(wo0, wnxt), nax0 = add_vs(xo0, xnxt);
-            ds_read128<0>(wa[0], naw0);
-            ds_read128<2048>(wa[1], naw0);
-            static_for<TM>([&](auto I) {
-                constexpr int i = decltype(I)::value;
-                vacc::mfma_acc<4 * (4 * TM + i)>(wa[2], xb[i]);
-                vacc::mfma_acc<4 * (5 * TM + i)>(wa[3], xb[i]);
-                ds_read128<i * 2048>(xb[i], nax0);
+            wait_lgkm<3>();   // x0..x3 and W0..W2 are in
+            static_for<TM>([&](auto I) { vacc::mfma_acc<4 * decltype(I)::value>(w[0], xc[decltype(I)::value]); });
+            // The barrier.  Every read of this stage's buffers has landed in this wave, and a loading wave's share of
+            // the next stage as well.  Memory operations complete in order; issued since the last load of the next
+            // stage (its fourth activation part, in the stage before): in a tile's first stage the NACC stores of
+            // the tile before it; this stage's three weight parts; in a tile's first stage its scales.
+            if (loader) {
+                constexpr int SC = DEQ ? 2 : 0;
+                if (!ldv) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(6 + SC + NACC) : "memory");
+                else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(6 + SC) : "memory");
+                else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();
+            const unsigned nax0 = add_vs(xo0, xnxt), naw0 = add_vs(wo0, wnxt);
+            ds_read128<0>(w[0], naw0);
+            static_for<TN - 1>([&](auto J1) {
+                constexpr int j = decltype(J1)::value + 1;
+                if constexpr (j - 1 < TM) {
+                    ds_read128<(j - 1) * 2048>(xa[j - 1], nax0);
+                    if (ld) issue_x(std::integral_constant<int, j - 1>{}, xcur);
+                }
+                static_for<TM>([&](auto I) {
+                    vacc::mfma_acc<4 * (j * TM + decltype(I)::value)>(w[j], xc[decltype(I)::value]);
+                });
+                ds_read128<j * 2048>(w[j], naw0);
             });
         }
         {
@@ -342,7 +318,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
             const unsigned u = wcur; wcur = wnxt; wnxt = wnn; wnn = u;
         }
     };
-    static_assert(12 + 2 + NACC + 2 <= 63, "the memory counter has six bits");
+    static_assert(6 + 2 + NACC + 8 <= 63, "the memory counter has six bits");
 
     // The tile's accumulators leave: converted, scaled by the row and the column scale, stored and cleared for the
     // next tile; accumulator (j, i) is named at compile time.  Two neighbouring column tiles are paired and swap
@@ -438,9 +414,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     }
     lkt = 2;
     __syncthreads();
-    ds_read128<0>(wa[0], wo0);
-    ds_read128<2048>(wa[1], wo0);
-    static_for<TM>([&](auto I) { ds_read128<decltype(I)::value * 2048>(xb[decltype(I)::value], xo0); });
+    // the first fragments, in the order in which every second half requests them for the next stage
+    ds_read128<0>(w[0], wo0);
+    static_for<TN - 1>([&](auto J1) {
+        constexpr int j = decltype(J1)::value + 1;
+        if constexpr (j - 1 < TM) ds_read128<(j - 1) * 2048>(xa[j - 1], xo0);
+        ds_read128<j * 2048>(w[j], wo0);
+    });
 
     for (int it = 0;; ++it) {
         cur_scales = (unsigned)(C::SCALES_AT + (it & 1) * C::SCALES);
@@ -503,8 +483,9 @@ struct Tile {
     int p, m0, n0, cost;
 };
 
-// cost of a tile in K stages, plus its conversion and stores (measured: 8.7 k ticks against 2.3 k a stage)
-static inline int tile_cost(int64_t K) { return (int)(K / 128) + 4; }
+// cost of a tile in K stages, plus what does not grow with K (conversion and stores, and the slower stages behind
+// them: a tile of 112 stages was measured at 2.9 times a tile of 32)
+static inline int tile_cost(int64_t K) { return (int)(K / 128) + 10; }
 
 template <int BM, int BN>
 static int64_t build_lists(const int64_t *mnk, int n, int cus, std::vector<v4i> *lists, int *per_wg_out)

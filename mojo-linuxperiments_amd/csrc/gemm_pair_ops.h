@@ -72,11 +72,12 @@ __device__ __forceinline__ void acc_zero()
 // accumulation registers.  A kernel that carries __attribute__((amdgpu_num_vgpr(ACC0 / 2))) and uses no
 // accumulation register is limited to v0 .. v(ACC0-1) for everything the compiler places (a spill goes to scratch
 // memory, which the build checks for), while v[ACC0 .. 255] are named by hand in the asm below and claimed for the
-// wave by a clobber of v255 (the register count of the kernel's descriptor).  Unlike accumulation registers, which
+// wave by a clobber of v255 (the register count of the kernel's descriptor).  ACC0 = 160 leaves the compiler 160
+// registers (fragments two K halves deep) and 96 accumulators.  Unlike accumulation registers, which
 // the register allocator may use to split a live range whenever ordinary registers run short, nothing but this
 // code can write them.
 namespace vacc {
-constexpr int ACC0 = 64;
+constexpr int ACC0 = 160;
 template <int LO>
 __device__ __forceinline__ void mfma_acc(const v4i &a, const v4i &b)
 {

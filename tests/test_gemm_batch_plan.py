@@ -38,7 +38,7 @@ def test_every_output_is_covered_once_or_with_equal_tiles(mi, shapes, cus):
             assert not ended, "an entry behind the end mark"
             M, N, K = shapes[p]
             assert 0 <= m0 <= M - BM and 0 <= n0 <= N - BN and n0 % 16 == 0
-            assert cost == K // 128 + 4
+            assert cost == K // 128 + 10
             cover[p][m0:m0 + BM, n0:n0 + BN] += 1
         assert ended, "every list ends with a mark"
     for c, (M, N, K) in zip(cover, shapes):
