@@ -203,7 +203,9 @@ def main():
         shapes[(K, N)] = bufs
         del w
     acts = {K: dev.upload(wl.activations(2025, M, K, stream=K)) for K in (4096, 14336)}
-    ybuf = dev.empty((M, 14336), np.float32)
+    # every projection writes an output of its own (318 MB in all: more than the memory-side cache holds)
+    ybufs = {name: dev.empty((M, N), np.float32) for name, K, N in wl.PROJECTIONS}
+    ybuf = ybufs["gate"]
     lin_ws = dev.empty(lib.mi_w8a8_linear_workspace_bytes(M, 14336, 14336), np.uint8)
     dev.sync()
 
@@ -216,10 +218,29 @@ def main():
 
     # One cfg3 step = the four projections of a decoder layer's prefill.  gate and up read the same activation
     # matrix (as they do in the layer), so its rotate + quantize prologue runs once and both contractions take the
-    # codes; qkv and down each quantize their own input.  Three prologues and four GEMM launches per step.
+    # codes; qkv and down each quantize their own input.  Three prologues, then ONE launch for the four
+    # contractions (mi_gemm_batch_*: a workgroup per compute unit walks a balanced list of 256 x 192 tiles drawn from
+    # all four problems).  The same step with four launches (one per projection, the single-problem kernels) and as
+    # four whole linears (a prologue each) is timed beside it.
     qx_ws = {K: (dev.empty((M, K), np.int8), dev.empty(M, np.float32)) for K in (4096, 14336)}
+    qx_qkv = (dev.empty((M, 4096), np.int8), dev.empty(M, np.float32))
+    batch = mi.GemmBatch(dev, [(M, N, K) for _, K, N in wl.PROJECTIONS])
+
+    def batch_ops(codes_of):
+        ops = []
+        for name, K, N in wl.PROJECTIONS:
+            qw, sw = next_w(K, N)
+            cx, cs = codes_of(name, K)
+            ops.append((cx, cs, qw, sw, ybufs[name]))
+        return ops
 
     def prefill_step():
+        mi.fwht_quant(acts[4096], *qx_qkv, wl.HADAMARD_BLOCK, stream=s)            # qkv's input
+        mi.fwht_quant(acts[4096], *qx_ws[4096], wl.HADAMARD_BLOCK, stream=s)       # gate's and up's input
+        mi.fwht_quant(acts[14336], *qx_ws[14336], wl.HADAMARD_BLOCK, stream=s)     # down's input
+        batch.run_f32(batch_ops(lambda name, K: qx_qkv if name == "qkv" else qx_ws[K]), stream=s)
+
+    def prefill_step_four_launches():
         last_quantized = None
         for name, K, N in wl.PROJECTIONS:
             qw, sw = next_w(K, N)
@@ -227,7 +248,13 @@ def main():
             if not (name == "up" and last_quantized == "gate"):
                 mi.fwht_quant(acts[K], cx, cs, wl.HADAMARD_BLOCK, stream=s)
             last_quantized = name
-            mi.check(lib.mi_w8a8_gemm_dequant_f32(cx.ptr, cs.ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, s))
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(cx.ptr, cs.ptr, qw.ptr, sw.ptr, ybufs[name].ptr, M, N, K, s))
+
+    def prefill_step_four_linears():
+        for name, K, N in wl.PROJECTIONS:
+            qw, sw = next_w(K, N)
+            mi.check(lib.mi_w8a8_linear_f32(acts[K].ptr, qw.ptr, sw.ptr, ybufs[name].ptr, M, N, K, wl.HADAMARD_BLOCK,
+                                            lin_ws.ptr, lin_ws.nbytes, s))
 
     log("headline: prefill step x%d (+%d warm-up)" % (args.steps, args.warmup))
     timer.settle(prefill_step)
@@ -241,21 +268,32 @@ def main():
     # The declared method: the same K steps recorded once into a graph (the weight rotation is baked in) and
     # replayed as one launch, exactly K steps inside the timed region and no host work between kernels.  The eager
     # figure is reported beside it and never picked.
+    def graph_ms(step):
+        with mi.Graph.capture(s) as g:
+            for _ in range(args.steps):
+                step()
+        timer.settle(lambda: g.launch())
+        ms = timer.run(lambda: g.launch(), 1) / args.steps
+        g.destroy()
+        return ms
+
     if NO_GRAPH:
         ms_graph = None
         ms_step = ms_eager
+        timer.settle(prefill_step_four_launches)
+        ms_four_launches = timer.run(prefill_step_four_launches, args.steps)
+        timer.settle(prefill_step_four_linears)
+        ms_four_linears = timer.run(prefill_step_four_linears, args.steps)
     else:
-        with mi.Graph.capture(s) as g:
-            for _ in range(args.steps):
-                prefill_step()
-        timer.settle(lambda: g.launch())
-        ms_graph = timer.run(lambda: g.launch(), 1) / args.steps
-        g.destroy()
+        ms_graph = graph_ms(prefill_step)
         ms_step = ms_graph
+        ms_four_launches = graph_ms(prefill_step_four_launches)
+        ms_four_linears = graph_ms(prefill_step_four_linears)
     step_ops = sum(wl.gemm_ops(M, N, K) for _, K, N in wl.PROJECTIONS)
     value = step_ops / (ms_step * 1e-3) / 1e12
 
-    # ---- the dominant kernel alone: the tiled MFMA GEMM on already-quantized activations
+    # ---- the dominant kernel alone: the batched GEMM (one launch, four problems) on already-quantized activations,
+    # and, for comparison, each projection as a launch of its own (the single-problem kernels)
     gemm_ms, gemm_samples = {}, {}
     qx = {K: dev.empty((M, K), np.int8) for K in (4096, 14336)}
     sx = {K: dev.empty(M, np.float32) for K in (4096, 14336)}
@@ -263,38 +301,56 @@ def main():
         mi.fwht_quant(acts[K], qx[K], sx[K], wl.HADAMARD_BLOCK, stream=s)
     quant_ms = {K: timer.run(lambda K=K: mi.fwht_quant(acts[K], qx[K], sx[K], wl.HADAMARD_BLOCK, stream=s), 20)
                 for K in qx}
+
+    def batch_only():
+        batch.run_f32(batch_ops(lambda name, K: (qx[K], sx[K])), stream=s)
+    timer.settle(batch_only)
+    batch_ms = timer.run(batch_only, max(10, args.steps))
+    batch_samples = sorted(timer.samples(batch_only, max(10, args.steps)))
     for name, K, N in wl.PROJECTIONS:
-        def one(K=K, N=N):
+        def one(name=name, K=K, N=N):
             qw, sw = next_w(K, N)
-            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx[K].ptr, sx[K].ptr, qw.ptr, sw.ptr, ybuf.ptr, M, N, K, s))
+            mi.check(lib.mi_w8a8_gemm_dequant_f32(qx[K].ptr, sx[K].ptr, qw.ptr, sw.ptr, ybufs[name].ptr, M, N, K, s))
         timer.settle(one)
         gemm_ms[name] = timer.run(one, max(10, args.steps))
         gemm_samples[name] = sorted(timer.samples(one, max(10, args.steps)))
     gemm_total_ms = sum(gemm_ms.values())
-    gemm_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
+    gemm_tops = step_ops / (batch_ms * 1e-3) / 1e12
+    single_tops = step_ops / (gemm_total_ms * 1e-3) / 1e12
     # HBM-side bytes per launch of the tiled GEMM, measured with hardware counters in a separate run
     traffic, traffic_total = None, None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as fh:
-            per = json.load(fh)["tiled_gemm_bytes_per_launch"]
-        traffic = {k: v["fetch"] + v["write"] for k, v in per.items()}
-        traffic_total = sum(traffic.values())
+            rec = json.load(fh)
+        if "batched_gemm_bytes_per_launch" in rec:
+            traffic = rec["batched_gemm_bytes_per_launch"]
+            traffic_total = traffic["fetch"] + traffic["write"]
     roofline = {
-        "kernel": "k_w8a8_pair (qkv, down) / k_w8a8_tiled (gate, up), v_mfma_i32_16x16x64_i8, four cfg3 shapes, ops-weighted",
+        "kernel": "k_w8a8_list, v_mfma_i32_16x16x64_i8: ONE launch for the four cfg3 contractions (1,632 tiles of "
+                  "256 x 192 on a balanced work list), dequantization fused",
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_total,
-        "traffic_unit": "bytes over the four launches (fetched + written), rocprofv3 PMC, calibrated",
+        "traffic_unit": "bytes per launch (fetched + written), rocprofv3 PMC, calibrated",
         "traffic_source": "profiles/hbm_traffic_pmc.md (a separate rocprofv3 --pmc run of bench.py --pmc-probe, "
                           "not this run)",
-        "traffic_per_shape": traffic,
-        "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
-        "per_shape_us_median": {k: round(v[len(v) // 2] * 1e3, 2) for k, v in gemm_samples.items()},
-        "per_shape_us_min": {k: round(v[0] * 1e3, 2) for k, v in gemm_samples.items()},
-        "per_shape_samples": "median / min over single launches, each between two event records (the records add "
-                             "1-3 us per launch to these two rows; per_shape_us is one pair of events around the whole run)",
-        "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
-                           for name, K, N in wl.PROJECTIONS},
+        "traffic_fetch_write": traffic,
+        "launch_us": round(batch_ms * 1e3, 2),
+        "launch_us_median": round(batch_samples[len(batch_samples) // 2] * 1e3, 2),
+        "launch_us_min": round(batch_samples[0] * 1e3, 2),
+        "launch_samples": "median / min over single launches, each between two event records; launch_us is one pair "
+                          "of events around back-to-back launches",
+        "algorithmic_ops_per_launch": step_ops,
+        "single_problem_launches": {
+            "what": "the same four contractions as four launches of the single-problem kernels (k_w8a8_pair for qkv "
+                    "and down, k_w8a8_tiled for gate and up)",
+            "tops": round(single_tops, 1), "frac": round(single_tops / PEAK_INT8_TOPS, 4),
+            "per_shape_us": {k: round(v * 1e3, 2) for k, v in gemm_ms.items()},
+            "per_shape_us_median": {k: round(v[len(v) // 2] * 1e3, 2) for k, v in gemm_samples.items()},
+            "per_shape_us_min": {k: round(v[0] * 1e3, 2) for k, v in gemm_samples.items()},
+            "per_shape_frac": {name: round(wl.gemm_ops(M, N, K) / (gemm_ms[name] * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
+                               for name, K, N in wl.PROJECTIONS},
+        },
     }
     # what the matrix pipe sustains here with nothing else in the way (power-limited clock): context for `frac`,
     # which stays against the published peak
@@ -318,15 +374,21 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "cfg3 prefill: the 4 rotated W8A8 projections of a layer (4096->6144, 4096->14336 x2, "
                                "14336->4096) at M=2048, Hadamard block 128, rotate+quant prologues included; gate and up share "
-                               "one input, which is rotated and quantized once (3 prologues + 4 GEMMs per step); all four "
-                               "write one 117 MB output buffer (it stays in the memory-side cache; weights rotate through "
-                               ">256 MB of copies); the K steps are recorded into one HIP graph and replayed - the timed "
-                               "method; eager launches from Python are reported beside it; about 60 ms of the same steps "
-                               "run untimed before the W warm-up steps so that timing starts at the sustained clock",
+                               "one input, which is rotated and quantized once (3 prologues per step), and the four "
+                               "contractions run as ONE launch (mi_gemm_batch_run_f32); every projection writes an output of "
+                               "its own (318 MB per step; weights rotate through >256 MB of copies); the K steps are recorded "
+                               "into one HIP graph and replayed - the timed method; eager launches from Python are reported "
+                               "beside it; about 60 ms of the same steps run untimed before the W warm-up steps so that "
+                               "timing starts at the sustained clock",
                    "tokens": M, "ops_per_step": step_ops, "tokens_per_s": round(M / (ms_step * 1e-3), 1),
                    "wall_ms_per_step": round(wall_ms, 4),
                    "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
-                   "method": "eager (--no-graph)" if NO_GRAPH else "graph replay"},
+                   "method": "eager (--no-graph)" if NO_GRAPH else "graph replay",
+                   "ms_per_step_four_launches": round(ms_four_launches, 4),
+                   "ms_per_step_four_linears": round(ms_four_linears, 4),
+                   "other_forms": "ms_per_step_four_launches: the same step with one launch per projection (3 prologues "
+                                  "+ 4 single-problem GEMM launches); ms_per_step_four_linears: four whole linears, a "
+                                  "prologue each (4 + 4 launches)"},
         "roofline": roofline,
         "host": host_topology(),
     }
@@ -362,8 +424,8 @@ def main():
 
 def pmc_probe(mi, wl):
     """Three launches each of: the rotation-only kernel on fp32 [2048,14336] (reads and writes exactly
-    117,440,512 B: the calibration for the FETCH_SIZE / WRITE_SIZE counters), the tiled GEMM on the four cfg3
-    shapes, the decode GEMV (M=1, 4096->14336), decode attention (cfg2) and the MoE layer (cfg4)."""
+    117,440,512 B: the calibration for the FETCH_SIZE / WRITE_SIZE counters), the single-problem GEMMs on the cfg3
+    shapes and the batched GEMM over all four (k_w8a8_list), the decode GEMV (M=1, 4096->14336), decode attention (cfg2) and the MoE layer (cfg4)."""
     lib = mi.lib
     dev = mi.Device(arena_bytes=8 << 30)
     M = wl.PREFILL_M
@@ -374,18 +436,24 @@ def pmc_probe(mi, wl):
         mi.fwht(a, b, 128)
     dev.sync()
     y = dev.empty((M, 14336), np.float32)
+    bops = []
     for name, K, N in wl.PROJECTIONS:
-        if name == "up":
-            continue
         qx = dev.upload(g.integers(-127, 128, (M, K)).astype(np.int8))
         qw = dev.upload(g.integers(-127, 128, (N, K)).astype(np.int8))
         sx, sw = dev.upload(np.ones(M, np.float32)), dev.upload(np.ones(N, np.float32))
+        bops.append((qx, sx, qw, sw, dev.empty((M, N), np.float32)))
+        if name == "up":
+            continue
         for _ in range(3):
             mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, y.ptr, M, N, K, None))
         if name == "gate":
             for _ in range(3):
                 mi.check(lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, y.ptr, 1, N, K, None))
         dev.sync()
+    batch = mi.GemmBatch(dev, [(M, N, K) for _, K, N in wl.PROJECTIONS])   # the four contractions as one launch
+    for _ in range(3):
+        batch.run_f32(bops)
+    dev.sync()
     timer = Timer(mi, None)
     print(json.dumps({"probe": "done", "attention": decode_attention(mi, wl, dev, None, timer, reps=1, graph=False),
                       "moe": moe_layer(mi, wl, dev, None, timer, reps=1, graph=False)}), flush=True)
