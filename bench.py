@@ -578,12 +578,27 @@ def decode_attention(mi, wl, dev, s, timer, reps=20, graph=True):
         mi.check(lib.mi_gqa_decode_attn_paged(dq.ptr, k[0].ptr, k[1].ptr, k[2].ptr, k[3].ptr, do.ptr, dtab.ptr,
                                               max_pages, P, B, Hq, Hkv, D, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
     ms_paged = run([(lambda k=k: paged(k)) for k in sets])
+    # the tiled caches read as pools of 64-token pages (one key block and one value block per kv head) under a
+    # shuffled block table: the same kernel, one table look-up per block
+    pages64 = T // 64
+    dtab64 = dev.upload(np.random.default_rng(4).permutation(B * pages64).astype(np.int32).reshape(B, pages64))
+
+    def paged_tiled(k, append):
+        if append:
+            mi.check(lib.mi_kv_append_tiled_paged_f32_i8(knew.ptr, vnew.ptr, Hkv * D, k[4].ptr, k[1].ptr, k[5].ptr, k[3].ptr,
+                                                         dtab64.ptr, pages64, dpos.ptr, B, Hkv, D, s))
+        mi.check(lib.mi_gqa_decode_attn_tiled_paged(dq.ptr, k[4].ptr, k[1].ptr, k[5].ptr, k[3].ptr, do.ptr, dtab64.ptr,
+                                                    pages64, B, Hq, Hkv, D, dlen.ptr, T, 0, ws.ptr, ws.nbytes, s))
+    ms_paged64 = run([(lambda k=k: paged_tiled(k, False)) for k in sets])
+    ms_paged64_app = run([(lambda k=k: paged_tiled(k, True)) for k in sets])
     dev.reset_to(mark)
     return {"cfg2_decode_attention": {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                       "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                       "tokens_per_s": round(B / (ms * 1e-3), 1), "algorithmic_bytes": nbytes,
                                       "cache_layout": "keys in 16-token tiles, values in transposed 64-token blocks",
                                       "with_kv_append_us": round(ms_app * 1e3, 2),
+                                      "paged_64_token_pages_shuffled_table_us": round(ms_paged64 * 1e3, 2),
+                                      "paged_64_token_pages_with_kv_append_us": round(ms_paged64_app * 1e3, 2),
                                       "row_major_cache_us": round(ms_rows * 1e3, 2),
                                       "row_major_with_kv_append_us": round(ms_rows_app * 1e3, 2),
                                       "row_major_paged_16_token_pages_us": round(ms_paged * 1e3, 2)}}
@@ -842,7 +857,7 @@ def decode_layer_chain(mi, wl, dev, s, timer, reps=10, batch=None, nlayers=3):
                             enumerate((((Hq + 2 * Hkv) * D, H), (H, Hq * D), (2 * I, H), (H, I)))]
             csrc[li % 3] = wl.normal(600 + li, (B * Hkv * T, D), 0)
         w = wsrc[li % 3]
-        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, w[0], w[1], w[2], w[3], g1, g1, cos, sin)
+        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, w[0], w[1], w[2], w[3], g1, g1, cos, sin, tiled=True)
         if li + 3 >= nlayers:
             wsrc[li % 3] = None
         # a cache of real rows: rotate + quantize N(0,1) keys and values
@@ -906,7 +921,7 @@ def moe_decode_layer_chain(mi, wl, dev, s, timer, reps=10, nlayers=3):
             dev.sync(s)
             dev.reset_to(keep)
             moe["w" + name], moe["s" + name] = q, sc
-        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, wq, wo, None, None, g1, g1, cos, sin, moe=moe)
+        L = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T, wq, wo, None, None, g1, g1, cos, sin, tiled=True, moe=moe)
         m2 = dev.mark()
         src = dev.upload(wl.normal(900 + li, (B * Hkv * T, D), 0))
         L.fill_cache_from_rows(src, T, s)

@@ -341,6 +341,45 @@ MI_API int32_t mi_rope_kv_append_tiled_f32_i8(const float *qkv, int64_t row_stri
                                               int8_t *vt, float *vs, const int32_t *pos,
                                               int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                                               void *stream);
+/* Paged form of the tiled cache: pools of 64-token pages.  A page holds, per kv head, one 8 KB key block (four
+ * 16-token tiles in the layout above) and one 8 KB transposed value block, plus 64 key and 64 value scales:
+ *   kt_pool, vt_pool int8 [pages, Hkv, 8192];  ks_pool, vs_pool fp32 [pages, Hkv, 64]
+ * Tokens [64 i, 64 i + 64) of sequence b live in page block_table[b * max_pages + i] (int32 in device memory; every
+ * entry that covers a token below seq_len[b], resp. the position being appended, must be a valid page of the pool:
+ * the kernels cannot check it; entries behind a sequence's last block may hold anything).  The attention kernel's
+ * loads stay 1 KB contiguous and a block costs it one scalar table look-up; arithmetic and results are those of the
+ * dense tiled layout, bit for bit.  seq_len is required.  No upstream counterpart: the allocator idea of one slab
+ * handing out fixed pieces (threading/numa_arena.mojo:40-55) applied to the cache. */
+MI_API int32_t mi_gqa_decode_attn_tiled_paged(const float *q, const int8_t *kt_pool, const float *ks_pool,
+                                              const int8_t *vt_pool, const float *vs_pool, float *o,
+                                              const int32_t *block_table, int64_t max_pages,
+                                              int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                              const int32_t *seq_len, int64_t T_max, int32_t out_rotated,
+                                              void *workspace, int64_t workspace_bytes, void *stream);
+MI_API int32_t mi_gqa_decode_attn_tiled_paged_quant_i8(const float *q, const int8_t *kt_pool, const float *ks_pool,
+                                                       const int8_t *vt_pool, const float *vs_pool, float *o_rot,
+                                                       int8_t *oq, float *oscale,
+                                                       const int32_t *block_table, int64_t max_pages,
+                                                       int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                                       const int32_t *seq_len, int64_t T_max,
+                                                       void *workspace, int64_t workspace_bytes, void *stream);
+MI_API int32_t mi_kv_append_tiled_paged_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                               int8_t *kt_pool, float *ks_pool, int8_t *vt_pool, float *vs_pool,
+                                               const int32_t *block_table, int64_t max_pages, const int32_t *pos,
+                                               int64_t B, int64_t Hkv, int64_t D, void *stream);
+MI_API int32_t mi_rope_kv_append_tiled_paged_f32_i8(const float *qkv, int64_t row_stride, const float *rope_cos,
+                                                    const float *rope_sin, float *q_out,
+                                                    int8_t *kt_pool, float *ks_pool, int8_t *vt_pool, float *vs_pool,
+                                                    const int32_t *block_table, int64_t max_pages, const int32_t *pos,
+                                                    int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
+/* Gate helper for the tiled layout: the split kernel of mi_gqa_decode_attn_tiled alone, which also writes out the
+ * int8 query codes [B,Hq,D], their scales [B,Hq] and the raw int32 scores [B,Hq,T] it works from (no merge, no o;
+ * every sequence holds T tokens). */
+MI_API int32_t mi_gqa_decode_scores_tiled_i32(const float *q, const int8_t *kt, const float *ks,
+                                              const int8_t *vt, const float *vs,
+                                              int8_t *qq, float *sq, int32_t *dots,
+                                              int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap, int64_t T,
+                                              void *workspace, int64_t workspace_bytes, void *stream);
 /* Gate helper: runs the same split kernel and also writes out the int8 query
  * codes [B,Hq,D], their scales [B,Hq] and the raw int32 scores [B,Hq,T] it
  * works from (no merge, no o). */

@@ -57,6 +57,15 @@ struct Params {
     float score_scale;        // log2(e) / sqrt(D)
     float *o;                 // DIRECT kernels: the output rows [B, Hq, 128]
     int out_rotated;
+    // paged cache: kq / vt are pools of 8 KB blocks [page][kv head], ks / vs pools of 64 scales [page][kv head];
+    // 64-token block i of sequence b lives in page block_table[b * max_pages + i].  Null: the dense layout.
+    const int32_t *block_table;
+    int max_pages;
+    // gate outputs (null in production): the int8 query codes [B, Hq, 128], their scales [B, Hq] and the raw int32
+    // dots [B, Hq, T] this kernel works from
+    int8_t *dbg_qq;
+    float *dbg_sq;
+    int32_t *dbg_dots;
 };
 
 template <int MASK>
@@ -117,9 +126,18 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
     // ---- loads, in the order they are needed: the span's scales, the query rows, then the ring
     const int sidx = 4 * tid;   // one float4 of each scale array per thread
     float4 ks4 = make_float4(0.f, 0.f, 0.f, 0.f), vs4 = ks4;
-    {
-        const int tk = min(t_lo + sidx, p.Tstride - 4);   // the row's own memory; tokens past the end are masked
-        if (sidx < SPAN) {
+    const int last_blk = (T - 1) >> 6;   // the last block that holds a token of this sequence
+    if (sidx < SPAN) {
+        if (p.block_table) {
+            // four consecutive tokens lie in one page; blocks past the sequence's last one (their table entries may
+            // hold anything) fall back on it, and their tokens are masked like any token past the end
+            const int tb = min((t_lo + sidx) >> 6, last_blk);
+            const int64_t page = p.block_table[(int64_t)b * p.max_pages + tb];
+            const int64_t at = (page * p.Hkv + kvh) * 64 + ((t_lo + sidx) & 63);
+            ks4 = *reinterpret_cast<const float4 *>(p.ks + at);
+            vs4 = *reinterpret_cast<const float4 *>(p.vs + at);
+        } else {
+            const int tk = min(t_lo + sidx, p.Tstride - 4);   // the row's own memory; tokens past the end are masked
             ks4 = *reinterpret_cast<const float4 *>(p.ks + (int64_t)bkv * p.Tstride + tk);
             vs4 = *reinterpret_cast<const float4 *>(p.vs + (int64_t)bkv * p.Tstride + tk);
         }
@@ -138,7 +156,14 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
     const int8_t *kblk[NT], *vblk[NT];   // the wave's blocks: 8 KB each, at the same offset in both arrays
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-        const int64_t off = ((int64_t)bkv * nblk_row + min(blk_lo + NW * j + wave, nblk_row - 1)) * 8192;
+        int64_t off;
+        if (p.block_table) {   // one scalar table look-up per block
+            const int page = __builtin_amdgcn_readfirstlane(
+                p.block_table[(int64_t)b * p.max_pages + min(blk_lo + NW * j + wave, last_blk)]);
+            off = ((int64_t)page * p.Hkv + kvh) * 8192;
+        } else {
+            off = ((int64_t)bkv * nblk_row + min(blk_lo + NW * j + wave, nblk_row - 1)) * 8192;
+        }
         kblk[j] = p.kq + off;
         vblk[j] = p.vt + off;
     }
@@ -182,9 +207,16 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
         a = fmax_xor<1>(a); a = fmax_xor<2>(a); a = fmax_xor<4>(a); a = fmax_xor<8>(a);
         const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
         const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
-        *reinterpret_cast<uint32_t *>(&s_q[wave][hr][4 * jj]) = quant4(v[0], v[1], v[2], v[3], inv);
-        *reinterpret_cast<uint32_t *>(&s_q[wave][hr][64 + 4 * jj]) = quant4(v[4], v[5], v[6], v[7], inv);
+        const uint32_t c0 = quant4(v[0], v[1], v[2], v[3], inv), c1 = quant4(v[4], v[5], v[6], v[7], inv);
+        *reinterpret_cast<uint32_t *>(&s_q[wave][hr][4 * jj]) = c0;
+        *reinterpret_cast<uint32_t *>(&s_q[wave][hr][64 + 4 * jj]) = c1;
         if (jj == 0) s_sq[wave][hr] = sc;
+        if (p.dbg_qq && split == 0 && wave == 0 && hr < G) {
+            int8_t *dq = p.dbg_qq + ((int64_t)b * p.Hq + head) * D;
+            *reinterpret_cast<uint32_t *>(dq + 4 * jj) = c0;
+            *reinterpret_cast<uint32_t *>(dq + 64 + 4 * jj) = c1;
+            if (jj == 0) p.dbg_sq[(int64_t)b * p.Hq + head] = sc;
+        }
     }
     // LDS only: the ring's loads stay in flight across this barrier
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -217,6 +249,12 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
             __builtin_amdgcn_sched_barrier(0);
             const float4 kk = *reinterpret_cast<const float4 *>(s_ks + sbase + 16 * sub + 4 * c4);
             const int tt = tok0 + 16 * sub + 4 * c4;
+            if (p.dbg_dots && r16 < G) {
+                int32_t *dd = p.dbg_dots + ((int64_t)b * p.Hq + kvh * G + r16) * p.T;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (tt + e < t_end) dd[tt + e] = dots[e];
+            }
             float4 sc;
             sc.x = (float)dots[0] * (kk.x * cq);
             sc.y = (float)dots[1] * (kk.y * cq);
@@ -420,7 +458,8 @@ __global__ __launch_bounds__(256) void k_kv_append_vt(const float *__restrict__ 
                                                       const float *__restrict__ sn, float *__restrict__ q_out,
                                                       int8_t *__restrict__ kq, float *__restrict__ ks,
                                                       int8_t *__restrict__ vt, float *__restrict__ vs,
-                                                      const int32_t *__restrict__ pos, int B, int Hq, int Hkv, int T_cap)
+                                                      const int32_t *__restrict__ pos, int B, int Hq, int Hkv, int T_cap,
+                                                      const int32_t *__restrict__ block_table, int max_pages)
 {
     constexpr int LPB = 16;
     const int t = threadIdx.x, j = t % LPB;
@@ -477,17 +516,19 @@ __global__ __launch_bounds__(256) void k_kv_append_vt(const float *__restrict__ 
     const float sc = (a == 0.0f) ? 1.0f : a / 127.0f;
     const float inv = (a == 0.0f) ? 0.0f : 127.0f / a;
     if (live && !is_q) {
-        const int64_t row = ((int64_t)b * Hkv + h) * T_cap + tp;
+        // first token of the 64-token block that holds tp: in the sequence's own row, or in its page of the pool
+        const int64_t blk0 = block_table ? ((int64_t)block_table[(int64_t)b * max_pages + (tp >> 6)] * Hkv + h) * 64
+                                         : ((int64_t)b * Hkv + h) * T_cap + (tp & ~63);
         const uint32_t c0 = quant4(v[0], v[1], v[2], v[3], inv), c1 = quant4(v[4], v[5], v[6], v[7], inv);
-        if (j == 0) (is_v ? vs : ks)[row] = sc;
+        if (j == 0) (is_v ? vs : ks)[blk0 + (tp & 63)] = sc;
         if (!is_v) {
             // codes 4j .. 4j+3: chunk j/4, bytes 4*(j%4) .. of token tp % 16 in tile tp / 16; codes 64 + 4j ..: chunk 4 + j/4
-            int8_t *q = kq + (((int64_t)b * Hkv + h) * T_cap + (tp & ~15)) * D + (j >> 2) * 256 + (tp & 15) * 16 + 4 * (j & 3);
+            int8_t *q = kq + (blk0 + (tp & 48)) * D + (j >> 2) * 256 + (tp & 15) * 16 + 4 * (j & 3);
             *reinterpret_cast<uint32_t *>(q) = c0;
             *reinterpret_cast<uint32_t *>(q + 1024) = c1;
         } else {
             // code d of token tp: block tp / 64, piece d / 16, token chunk (tp % 64) / 16, row d % 16, byte tp % 16
-            int8_t *blk = vt + (((int64_t)b * Hkv + h) * T_cap + (tp & ~63)) * D + (j >> 2) * 1024 + ((tp & 63) >> 4) * 256 +
+            int8_t *blk = vt + blk0 * D + (j >> 2) * 1024 + ((tp & 63) >> 4) * 256 +
                           4 * (j & 3) * 16 + (tp & 15);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -541,11 +582,22 @@ using namespace mi;
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+struct ScoreGate {
+    int8_t *qq;
+    float *sq;
+    int32_t *dots;
+};
+
 static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, const int8_t *vt, const float *vs, float *o,
                       int8_t *oq, float *oscale, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap,
                       const int32_t *seq_len, int64_t T_max, int32_t out_rotated, void *workspace,
-                      int64_t workspace_bytes, hipStream_t s)
+                      int64_t workspace_bytes, hipStream_t s, const int32_t *block_table = nullptr,
+                      int64_t max_pages = 0, const ScoreGate *dbg = nullptr)
 {
+    if (block_table) {   // paged: the capacity of a sequence is its share of the table
+        if (max_pages <= 0 || max_pages > (1 << 18) || !seq_len || !aligned4(block_table)) return MI_EINVAL;
+        T_cap = max_pages * 64;
+    }
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || T_cap <= 0 || T_max <= 0 || T_max > T_cap) return MI_EINVAL;
     if (D != avt::D || Hq % Hkv || Hq / Hkv > 4 || T_cap % 64) return MI_EINVAL;
     if (T_cap > (1LL << 24) || B * Hkv > 65535) return MI_ERANGE;
@@ -555,7 +607,8 @@ static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, cons
     if (seq_len && !aligned4(seq_len)) return MI_EINVAL;
     if (workspace_bytes < mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max)) return MI_ENOSPC;
     const avt::Plan plan = avt::pick(B, Hkv, T_max);
-    const bool direct = plan.splits == 1 && !oq;   // one workgroup sees the whole sequence: it writes the output rows
+    // one workgroup sees the whole sequence: it writes the output rows (the gate takes the split form: it wants no o)
+    const bool direct = plan.splits == 1 && !oq && !dbg;
     avt::Params p;
     p.q = q; p.kq = kq; p.ks = ks; p.vt = vt; p.vs = vs;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.G = (int)(Hq / Hkv); p.T = (int)T_max;
@@ -563,6 +616,10 @@ static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, cons
     p.seq_len = seq_len;
     p.score_scale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
     p.o = o; p.out_rotated = out_rotated;
+    p.block_table = block_table; p.max_pages = (int)max_pages;
+    p.dbg_qq = dbg ? dbg->qq : nullptr;
+    p.dbg_sq = dbg ? dbg->sq : nullptr;
+    p.dbg_dots = dbg ? dbg->dots : nullptr;
     p.part_o = static_cast<float *>(workspace);
     p.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) +
                                           align_up(B * Hkv * plan.splits * 4 * avt::D * 4, 256));
@@ -573,7 +630,7 @@ static int32_t run_tiled(const float *q, const int8_t *kq, const float *ks, cons
     if (direct) { if (nt <= 1) MI_TILED(1, true); else if (nt <= 2) MI_TILED(2, true); else MI_TILED(4, true); }
     else { if (nt <= 1) MI_TILED(1, false); else if (nt <= 2) MI_TILED(2, false); else MI_TILED(4, false); }
 #undef MI_TILED
-    if (direct) return launch_status();
+    if (direct || dbg) return launch_status();
     int32_t rc = launch_status();
     if (rc) return rc;
     return attn::launch_merge(p.part_o, p.part_ml, o, oq, oscale, B, Hq, Hkv, plan.splits, out_rotated, s);
@@ -599,6 +656,19 @@ extern "C" int32_t mi_gqa_decode_attn_tiled_quant_i8(const float *q, const int8_
     if (Hq > 64) return MI_ERANGE;
     return run_tiled(q, kq, ks, vt, vs, o_rot, oq, oscale, B, Hq, Hkv, D, T_cap, seq_len, T_max, 1, workspace,
                   workspace_bytes, as_stream(stream));
+}
+
+// Gate helper for this layout: the split kernel alone, which also writes out the int8 query codes, their scales and
+// the raw int32 dots it works from (no merge, no o).
+extern "C" int32_t mi_gqa_decode_scores_tiled_i32(const float *q, const int8_t *kt, const float *ks, const int8_t *vt,
+                                                  const float *vs, int8_t *qq, float *sq, int32_t *dots, int64_t B,
+                                                  int64_t Hq, int64_t Hkv, int64_t D, int64_t T_cap, int64_t T,
+                                                  void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!qq || !sq || !dots || !aligned4(qq) || !aligned4(sq) || !aligned4(dots)) return MI_EINVAL;
+    const ScoreGate g = {qq, sq, dots};
+    return run_tiled(q, kt, ks, vt, vs, nullptr, nullptr, nullptr, B, Hq, Hkv, D, T_cap, nullptr, T, 1, workspace,
+                     workspace_bytes, as_stream(stream), nullptr, 0, &g);
 }
 
 namespace mi {
@@ -688,7 +758,7 @@ extern "C" int32_t mi_kv_append_tiled_f32_i8(const float *k_new, const float *v_
     const dim3 grid((unsigned)((B * Hkv + 15) / 16), 2);
     hipLaunchKernelGGL(avt::k_kv_append_vt<false>, grid, dim3(256), 0, as_stream(stream), k_new, v_new, row_stride,
                        (const float *)nullptr, (const float *)nullptr, (float *)nullptr, kq, ks, vt, vs, pos, (int)B, 0,
-                       (int)Hkv, (int)T_cap);
+                       (int)Hkv, (int)T_cap, (const int32_t *)nullptr, 0);
     return launch_status();
 }
 
@@ -704,6 +774,69 @@ extern "C" int32_t mi_rope_kv_append_tiled_f32_i8(const float *qkv, int64_t row_
     const int64_t heads = B * (Hq + 2 * Hkv);
     hipLaunchKernelGGL(avt::k_kv_append_vt<true>, dim3((unsigned)((heads + 15) / 16)), dim3(256), 0, as_stream(stream),
                        qkv, (const float *)nullptr, row_stride, rope_cos, rope_sin, q_out, kq, ks, vt, vs, pos, (int)B,
-                       (int)Hq, (int)Hkv, (int)T_cap);
+                       (int)Hq, (int)Hkv, (int)T_cap, (const int32_t *)nullptr, 0);
+    return launch_status();
+}
+
+// ---- the paged form of the tiled cache: pools of 64-token pages, one page = one 8 KB key block (four 16-token tiles)
+// and one 8 KB transposed value block per kv head, so the attention kernel's loads stay 1 KB contiguous and a block
+// costs it one scalar table look-up.
+extern "C" int32_t mi_gqa_decode_attn_tiled_paged(const float *q, const int8_t *kt_pool, const float *ks_pool,
+                                                  const int8_t *vt_pool, const float *vs_pool, float *o,
+                                                  const int32_t *block_table, int64_t max_pages, int64_t B,
+                                                  int64_t Hq, int64_t Hkv, int64_t D, const int32_t *seq_len,
+                                                  int64_t T_max, int32_t out_rotated, void *workspace,
+                                                  int64_t workspace_bytes, void *stream)
+{
+    if (!o || !aligned16(o) || !block_table) return MI_EINVAL;
+    return run_tiled(q, kt_pool, ks_pool, vt_pool, vs_pool, o, nullptr, nullptr, B, Hq, Hkv, D, 0, seq_len, T_max,
+                     out_rotated, workspace, workspace_bytes, as_stream(stream), block_table, max_pages);
+}
+
+extern "C" int32_t mi_gqa_decode_attn_tiled_paged_quant_i8(const float *q, const int8_t *kt_pool, const float *ks_pool,
+                                                           const int8_t *vt_pool, const float *vs_pool, float *o_rot,
+                                                           int8_t *oq, float *oscale, const int32_t *block_table,
+                                                           int64_t max_pages, int64_t B, int64_t Hq, int64_t Hkv,
+                                                           int64_t D, const int32_t *seq_len, int64_t T_max,
+                                                           void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!oq || !oscale || !aligned4(oq) || !aligned4(oscale) || (o_rot && !aligned16(o_rot)) || !block_table) return MI_EINVAL;
+    if (Hq > 64) return MI_ERANGE;
+    return run_tiled(q, kt_pool, ks_pool, vt_pool, vs_pool, o_rot, oq, oscale, B, Hq, Hkv, D, 0, seq_len, T_max, 1,
+                     workspace, workspace_bytes, as_stream(stream), block_table, max_pages);
+}
+
+extern "C" int32_t mi_kv_append_tiled_paged_f32_i8(const float *k_new, const float *v_new, int64_t row_stride,
+                                                   int8_t *kt_pool, float *ks_pool, int8_t *vt_pool, float *vs_pool,
+                                                   const int32_t *block_table, int64_t max_pages, const int32_t *pos,
+                                                   int64_t B, int64_t Hkv, int64_t D, void *stream)
+{
+    if (!block_table || !aligned4(block_table) || max_pages <= 0 || max_pages > (1 << 18)) return MI_EINVAL;
+    int32_t rc = check_append(k_new, v_new, kt_pool, ks_pool, vt_pool, vs_pool, pos, B, Hkv, D, max_pages * 64);
+    if (rc) return rc;
+    if (row_stride < Hkv * D || row_stride % 4) return MI_EINVAL;
+    const dim3 grid((unsigned)((B * Hkv + 15) / 16), 2);
+    hipLaunchKernelGGL(avt::k_kv_append_vt<false>, grid, dim3(256), 0, as_stream(stream), k_new, v_new, row_stride,
+                       (const float *)nullptr, (const float *)nullptr, (float *)nullptr, kt_pool, ks_pool, vt_pool,
+                       vs_pool, pos, (int)B, 0, (int)Hkv, (int)(max_pages * 64), block_table, (int)max_pages);
+    return launch_status();
+}
+
+extern "C" int32_t mi_rope_kv_append_tiled_paged_f32_i8(const float *qkv, int64_t row_stride, const float *rope_cos,
+                                                        const float *rope_sin, float *q_out, int8_t *kt_pool,
+                                                        float *ks_pool, int8_t *vt_pool, float *vs_pool,
+                                                        const int32_t *block_table, int64_t max_pages,
+                                                        const int32_t *pos, int64_t B, int64_t Hq, int64_t Hkv,
+                                                        int64_t D, void *stream)
+{
+    if (!block_table || !aligned4(block_table) || max_pages <= 0 || max_pages > (1 << 18)) return MI_EINVAL;
+    int32_t rc = check_append(qkv, q_out, kt_pool, ks_pool, vt_pool, vs_pool, pos, B, Hkv, D, max_pages * 64);
+    if (rc) return rc;
+    if (!rope_cos || !rope_sin || !aligned16(rope_cos) || !aligned16(rope_sin) || Hq <= 0) return MI_EINVAL;
+    if (row_stride < (Hq + 2 * Hkv) * D || row_stride % 4) return MI_EINVAL;
+    const int64_t heads = B * (Hq + 2 * Hkv);
+    hipLaunchKernelGGL(avt::k_kv_append_vt<true>, dim3((unsigned)((heads + 15) / 16)), dim3(256), 0, as_stream(stream),
+                       qkv, (const float *)nullptr, row_stride, rope_cos, rope_sin, q_out, kt_pool, ks_pool, vt_pool,
+                       vs_pool, pos, (int)B, (int)Hq, (int)Hkv, (int)(max_pages * 64), block_table, (int)max_pages);
     return launch_status();
 }

@@ -235,7 +235,9 @@ struct DecodeAttention {
 // (the loop that produces them runs on the device side of the stream, not on the host).
 // tiled: the codes live in the layouts the int8 matrix instruction loads straight from memory (keys in 16-token
 // tiles, values in transposed 64-token blocks; capacity a multiple of 64 tokens): the fast attention path.
-// Otherwise both halves are row-major [B, Hkv, T_cap, 128].  Same arithmetic, same codes, same scales.
+// Otherwise both halves are row-major [B, Hkv, T_cap, 128].  Same arithmetic, same codes, same scales.  The layout is
+// the caller's choice at prepare() and never follows from the capacity; code that fills kq / vq itself must write
+// the layout it chose (load_rows() converts row-major codes).
 struct KvCache {
     int64_t B = 0, Hq = 0, Hkv = 0, D = 128, T_cap = 0;
     bool tiled = false;
@@ -258,11 +260,6 @@ struct KvCache {
         vs = arena.template alloc<float>(B * Hkv * T_cap);
         workspace = arena.template alloc<uint8_t>(workspace_bytes);
         return kq && vq && ks && vs && workspace;
-    }
-    template <typename Arena>
-    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t t_cap)
-    {
-        return prepare(arena, b, hq, hkv, t_cap, t_cap % 64 == 0);
     }
     explicit operator bool() const { return workspace != nullptr; }
     // k_new / v_new: head h of sequence b at + b*row_stride + h*128 floats (slices of a fused QKV row are fine)
@@ -319,17 +316,24 @@ struct KvCache {
 
 // The same cache as pools of pages shared by all sequences: tokens [i*P, (i+1)*P) of sequence b live in page
 // table[b*max_pages + i].  The table is the caller's (int32 in device memory): a scheduler hands pages out.
+// tiled (pages of 64 tokens only): a page holds, per kv head, one 8 KB block of key tiles and one 8 KB transposed
+// value block, the layouts of the tiled KvCache, so attention runs the matrix-instruction kernel at the dense
+// layout's speed; otherwise pages are row-major [page_size, 128] per kv head.
 struct PagedKvCache {
     int64_t B = 0, Hq = 0, Hkv = 0, D = 128, pages = 0, page_size = 0, max_pages = 0;
+    bool tiled = false;
     int8_t *kq = nullptr, *vq = nullptr;
     float *ks = nullptr, *vs = nullptr;
     void *workspace = nullptr;
     int64_t workspace_bytes = 0;
 
     template <typename Arena>
-    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t n_pages, int64_t p_size, int64_t max_pages_per_seq)
+    bool prepare(Arena &arena, int64_t b, int64_t hq, int64_t hkv, int64_t n_pages, int64_t p_size, int64_t max_pages_per_seq,
+                 bool use_tiled_layouts)
     {
         B = b; Hq = hq; Hkv = hkv; pages = n_pages; page_size = p_size; max_pages = max_pages_per_seq;
+        tiled = use_tiled_layouts;
+        if (tiled && page_size != 64) return false;
         workspace_bytes = mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, max_pages * page_size);
         if (workspace_bytes <= 0) return false;
         kq = arena.template alloc<int8_t>(pages * Hkv * page_size * D);
@@ -343,14 +347,34 @@ struct PagedKvCache {
     int32_t append(const float *k_new, const float *v_new, int64_t row_stride, const int32_t *table, const int32_t *pos,
                    void *stream) const
     {
-        return mi_kv_append_paged_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, table, max_pages, page_size, pos, B, Hkv,
-                                         D, stream);
+        return tiled ? mi_kv_append_tiled_paged_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, table, max_pages, pos, B,
+                                                       Hkv, D, stream)
+                     : mi_kv_append_paged_f32_i8(k_new, v_new, row_stride, kq, ks, vq, vs, table, max_pages, page_size, pos,
+                                                 B, Hkv, D, stream);
+    }
+    // a fused QKV row per sequence: rotary embedding, queries out, keys and values appended (tiled pages only)
+    int32_t rope_append(const float *qkv, int64_t row_stride, const float *rope_cos, const float *rope_sin, float *q_out,
+                        const int32_t *table, const int32_t *pos, void *stream) const
+    {
+        if (!tiled) return MI_EINVAL;
+        return mi_rope_kv_append_tiled_paged_f32_i8(qkv, row_stride, rope_cos, rope_sin, q_out, kq, ks, vq, vs, table,
+                                                    max_pages, pos, B, Hq, Hkv, D, stream);
     }
     int32_t attend(const float *q, float *o, const int32_t *table, const int32_t *seq_len, int64_t t_max, bool out_rotated,
                    void *stream) const
     {
-        return mi_gqa_decode_attn_paged(q, kq, ks, vq, vs, o, table, max_pages, page_size, B, Hq, Hkv, D, seq_len, t_max,
-                                        out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+        return tiled ? mi_gqa_decode_attn_tiled_paged(q, kq, ks, vq, vs, o, table, max_pages, B, Hq, Hkv, D, seq_len, t_max,
+                                                      out_rotated ? 1 : 0, workspace, workspace_bytes, stream)
+                     : mi_gqa_decode_attn_paged(q, kq, ks, vq, vs, o, table, max_pages, page_size, B, Hq, Hkv, D, seq_len,
+                                                t_max, out_rotated ? 1 : 0, workspace, workspace_bytes, stream);
+    }
+    // the merge fused with the output projection's row quantizer (tiled pages only)
+    int32_t attend_quant(const float *q, float *o_rot, int8_t *oq, float *oscale, const int32_t *table, const int32_t *seq_len,
+                         int64_t t_max, void *stream) const
+    {
+        if (!tiled) return MI_EINVAL;
+        return mi_gqa_decode_attn_tiled_paged_quant_i8(q, kq, ks, vq, vs, o_rot, oq, oscale, table, max_pages, B, Hq, Hkv, D,
+                                                       seq_len, t_max, workspace, workspace_bytes, stream);
     }
 };
 
@@ -404,7 +428,7 @@ struct DecoderLayer {
     // fp32 weights in device memory: wqkv [(Hq+2Hkv)*128, H], wo [H, Hq*128], wgu [2I, H] (gate rows, then up
     // rows), wd [H, I]; norm weights g1, g2 [H]; rotary tables [T_cap, 64].  false if the arena is exhausted.
     template <typename Arena>
-    bool prepare(Arena &arena, int64_t b, int64_t h, int64_t hq, int64_t hkv, int64_t i, int64_t t_cap,
+    bool prepare(Arena &arena, int64_t b, int64_t h, int64_t hq, int64_t hkv, int64_t i, int64_t t_cap, bool tiled_cache,
                  const float *wqkv, const float *wo, const float *wgu, const float *wd, const float *norm1,
                  const float *norm2, const float *cos_table, const float *sin_table, float epsilon, void *stream,
                  bool trace = false)
@@ -415,7 +439,7 @@ struct DecoderLayer {
         // wgu == wd == nullptr: the FFN half will be an MoE (use_moe)
         bool ok = qkv.prepare(arena, wqkv, nqkv, H, B, stream) && o.prepare(arena, wo, H, Hq * 128, B, stream) &&
                   (!wgu || gate_up.prepare(arena, wgu, 2 * I, H, B, stream)) &&
-                  (!wd || down.prepare(arena, wd, H, I, B, stream)) && cache.prepare(arena, B, Hq, Hkv, T_cap);
+                  (!wd || down.prepare(arena, wd, H, I, B, stream)) && cache.prepare(arena, B, Hq, Hkv, T_cap, tiled_cache);
         h0 = arena.template alloc<float>(B * H);
         qkv_out = arena.template alloc<float>(B * nqkv);
         q = arena.template alloc<float>(B * Hq * 128);

@@ -121,6 +121,12 @@ SIGNATURES = {
     "mi_kv_tiled_from_rows_i8": (i32, [vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_kv_append_tiled_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
     "mi_rope_kv_append_tiled_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
+    "mi_gqa_decode_attn_tiled_paged": (i32, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64, i32, vp, i64, vp]),
+    "mi_gqa_decode_attn_tiled_paged_quant_i8": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, i64,
+                                                       vp, i64, vp]),
+    "mi_kv_append_tiled_paged_f32_i8": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, i64, vp, i64, i64, i64, vp]),
+    "mi_rope_kv_append_tiled_paged_f32_i8": (i32, [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, vp, i64, i64, i64, i64, vp]),
+    "mi_gqa_decode_scores_tiled_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_gqa_decode_scores_i32": (i32, [vp] * 8 + [i64, i64, i64, i64, i64, vp, i64, vp]),
     "mi_moe_route_workspace_bytes": (i64, [i64, i64]),
     "mi_moe_route": (i32, [vp, vp, vp, vp, i64, i64, i64, i32, vp, i64, vp]),
@@ -473,15 +479,18 @@ class DecoderLayer:
     (xn, att, hn, act) so that a test can gate every stage."""
 
     def __init__(self, dev, B, H, Hq, Hkv, I, T_cap, wqkv, wo, wgu, wd, g1, g2, rope_cos, rope_sin, eps=1e-5,
-                 block=128, trace=False, tiled=None, moe=None):
+                 block=128, trace=False, *, tiled, moe=None):
         """moe: None for the dense FFN (wgu, wd), or the experts of an MoE FFN in its place (wgu = wd = None):
         dict(wr fp32 [E,H], wg/wu int8 [E,I,H], sg/su fp32 [E,I], wd int8 [E,H,I], sd fp32 [E,H], topk), prepared codes.
         The second half of the layer is then residual + RMSNorm -> router, dispatch and grouped expert FFN ->
         residual."""
         D = 128
         self.moe = None
-        # the cache lives in the matrix-pipe layouts whenever its capacity allows (a multiple of 64 tokens)
-        self.tiled = (T_cap % 64 == 0) if tiled is None else bool(tiled)
+        # tiled (required, no default): the cache lives in the matrix-pipe layouts (capacity a multiple of 64 tokens)
+        # or row-major; the layout never follows from the capacity
+        self.tiled = bool(tiled)
+        if self.tiled and T_cap % 64:
+            raise MiError(EINVAL, "DecoderLayer: a tiled cache needs a capacity that is a multiple of 64 tokens")
         self.dev, self.B, self.H, self.Hq, self.Hkv, self.I, self.T_cap, self.eps, self.block = \
             dev, B, H, Hq, Hkv, I, T_cap, eps, block
         self.NQKV = (Hq + 2 * Hkv) * D

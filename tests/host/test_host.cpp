@@ -239,7 +239,7 @@ static void test_kv_cache(const Context &ctx, int64_t T_cap, const char *name)
     const int64_t B = 2, Hq = 8, Hkv = 2, D = 128;
     DeviceArena<256> arena(ctx, 64 << 20);
     KvCache cache;
-    bool ok = cache.prepare(arena, B, Hq, Hkv, T_cap) && (bool)cache;
+    bool ok = cache.prepare(arena, B, Hq, Hkv, T_cap, T_cap % 64 == 0) && (bool)cache;
     Rng rng{11};
     std::vector<int8_t> rkq(B * Hkv * T_cap * D, 0), rvq(B * Hkv * T_cap * D, 0);
     std::vector<float> rks(B * Hkv * T_cap, 0.0f), rvs(B * Hkv * T_cap, 0.0f);
@@ -301,6 +301,55 @@ static void test_kv_cache(const Context &ctx, int64_t T_cap, const char *name)
     report(name, ok && err <= 2e-3f, "max-abs " + std::to_string(err));
 }
 
+// PagedKvCache against KvCache: the same three decode steps, the paged cache under a table that hands its pages
+// out in reverse; outputs must be equal bit for bit in either layout.
+static void test_paged_kv_cache(const Context &ctx, bool tiled, const char *name)
+{
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 128, P = 64, max_pages = 3, T_cap = P * max_pages, pages = B * max_pages + 1;
+    DeviceArena<256> arena(ctx, 64 << 20);
+    KvCache dense;
+    PagedKvCache paged;
+    bool ok = dense.prepare(arena, B, Hq, Hkv, T_cap, tiled) && paged.prepare(arena, B, Hq, Hkv, pages, P, max_pages, tiled) &&
+              (bool)paged && paged.tiled == tiled;
+    // a cache that was never appended to must read as zero codes with zero scales in both
+    ok = ok && mi_fill_u32(dense.kq, 0, B * Hkv * T_cap * D / 4, nullptr) == MI_OK &&
+         mi_fill_u32(dense.vq, 0, B * Hkv * T_cap * D / 4, nullptr) == MI_OK &&
+         mi_fill_u32(dense.ks, 0, B * Hkv * T_cap, nullptr) == MI_OK && mi_fill_u32(dense.vs, 0, B * Hkv * T_cap, nullptr) == MI_OK &&
+         mi_fill_u32(paged.kq, 0, pages * Hkv * P * D / 4, nullptr) == MI_OK &&
+         mi_fill_u32(paged.vq, 0, pages * Hkv * P * D / 4, nullptr) == MI_OK &&
+         mi_fill_u32(paged.ks, 0, pages * Hkv * P, nullptr) == MI_OK && mi_fill_u32(paged.vs, 0, pages * Hkv * P, nullptr) == MI_OK;
+    std::vector<int32_t> table((size_t)(B * max_pages));
+    for (size_t i = 0; i < table.size(); ++i) table[i] = (int32_t)(pages - 1 - i);
+    int32_t *dtable = upload(arena, table);
+    Rng rng{21};
+    int32_t *dpos = arena.alloc<int32_t>(B), *dlen = arena.alloc<int32_t>(B);
+    float *dq = arena.alloc<float>(B * Hq * D), *dk = arena.alloc<float>(B * Hkv * D), *dv = arena.alloc<float>(B * Hkv * D);
+    float *o1 = arena.alloc<float>(B * Hq * D), *o2 = arena.alloc<float>(B * Hq * D);
+    ok = ok && dtable && dpos && dlen && dq && dk && dv && o1 && o2;
+    const int32_t start[2] = {62, 127};   // both sequences cross a page boundary within the three steps
+    bool same = true;
+    for (int step = 0; ok && step < 3; ++step) {
+        std::vector<float> q(B * Hq * D), k(B * Hkv * D), v(B * Hkv * D);
+        for (auto &e : q) e = rng.normal();
+        for (auto &e : k) e = rng.normal();
+        for (auto &e : v) e = rng.normal();
+        int32_t pos[2] = {start[0] + step, start[1] + step}, len[2] = {pos[0] + 1, pos[1] + 1};
+        mi_memcpy_h2d(dpos, pos, sizeof(pos), nullptr);
+        mi_memcpy_h2d(dlen, len, sizeof(len), nullptr);
+        mi_memcpy_h2d(dq, q.data(), (int64_t)q.size() * 4, nullptr);
+        mi_memcpy_h2d(dk, k.data(), (int64_t)k.size() * 4, nullptr);
+        mi_memcpy_h2d(dv, v.data(), (int64_t)v.size() * 4, nullptr);
+        ok = ok && dense.append(dk, dv, Hkv * D, dpos, nullptr) == MI_OK &&
+             paged.append(dk, dv, Hkv * D, dtable, dpos, nullptr) == MI_OK &&
+             dense.attend(dq, o1, dlen, len[1], false, nullptr) == MI_OK &&
+             paged.attend(dq, o2, dtable, dlen, len[1], false, nullptr) == MI_OK;
+        same = same && download(o1, (size_t)(B * Hq * D)) == download(o2, (size_t)(B * Hq * D));
+    }
+    // the calls that exist for tiled pages only say so for row-major ones
+    const int32_t rc = paged.attend_quant(dq, o2, nullptr, nullptr, dtable, dlen, 1, nullptr);
+    report(name, ok && same && (tiled || rc == MI_EINVAL), same ? "outputs equal" : "outputs differ");
+}
+
 // DecoderLayer::step against the oracle's operators chained in the same order, every stage fed what the device
 // fed its next kernel (integer stages equal, fp32 stages to 2e-6 relative; attention to 2e-5 absolute)
 static void test_decoder_layer(const Context &ctx)
@@ -321,7 +370,7 @@ static void test_decoder_layer(const Context &ctx)
             sn[t * 64 + i] = (float)std::sin(a);
         }
     DecoderLayer layer;
-    bool ok = layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, upload(arena, wqkv), upload(arena, wo), upload(arena, wgu),
+    bool ok = layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, T_cap % 64 == 0, upload(arena, wqkv), upload(arena, wo), upload(arena, wgu),
                             upload(arena, wd), upload(arena, g1), upload(arena, g2), upload(arena, cs), upload(arena, sn),
                             1e-5f, nullptr, true);
     const std::vector<int32_t> pos = {0, 9}, len = {1, 10};
@@ -440,8 +489,8 @@ static void test_decoder_stack(const Context &ctx)
         float *a = upload(arena, wqkv), *b = upload(arena, wo), *c = upload(arena, wgu), *d = upload(arena, wd),
               *e = upload(arena, g1), *f = upload(arena, g2);
         ok = a && b && c && d && e && f &&
-             stack.add(arena, B, H, Hq, Hkv, I, T_cap, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr) &&
-             solo[l].prepare(arena, B, H, Hq, Hkv, I, T_cap, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr);
+             stack.add(arena, B, H, Hq, Hkv, I, T_cap, false, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr) &&
+             solo[l].prepare(arena, B, H, Hq, Hkv, I, T_cap, false, a, b, c, d, e, f, dcs, dsn, 1e-5f, nullptr);
     }
     std::vector<float> x = gauss(B * H, 1.0f);
     const std::vector<int32_t> pos = {0, 5}, len = {1, 6};
@@ -449,7 +498,7 @@ static void test_decoder_stack(const Context &ctx)
     float *dx = upload(arena, x), *dout = arena.alloc<float>(B * H), *dref = arena.alloc<float>(B * H),
           *dmid = arena.alloc<float>(B * H);
     ok = ok && dpos && dlen && dx && dout && dref && dmid && stack.count == 3;
-    const bool refuses = ok && [&] { DecoderStack<1> one; one.count = 1; return !one.add(arena, B, H, Hq, Hkv, I, T_cap, dx, dx, dx, dx, dx, dx, dcs, dsn, 1e-5f, nullptr); }();
+    const bool refuses = ok && [&] { DecoderStack<1> one; one.count = 1; return !one.add(arena, B, H, Hq, Hkv, I, T_cap, false, dx, dx, dx, dx, dx, dx, dcs, dsn, 1e-5f, nullptr); }();
     if (!ok) { report("decoder_stack", false, "set-up failed"); return; }
     // by hand: every layer closes with its own residual add, the next one starts from that sum
     bool good = solo[0].step(dx, nullptr, dpos, dlen, T_cap, dmid, nullptr) == MI_OK &&
@@ -502,7 +551,7 @@ static void test_moe_decoder_layer(const Context &ctx)
     ok = ok && ffn.prepare(arena, B, H, I, E, topk);
     ffn.wr = upload(arena, wr); ffn.wg = wg; ffn.sg = sg; ffn.wu = wu; ffn.su = su; ffn.wd = wd; ffn.sd = sd;
     DecoderLayer layer;
-    ok = ok && layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, upload(arena, wqkv), upload(arena, wo), (const float *)nullptr,
+    ok = ok && layer.prepare(arena, B, H, Hq, Hkv, I, T_cap, T_cap % 64 == 0, upload(arena, wqkv), upload(arena, wo), (const float *)nullptr,
                              (const float *)nullptr, upload(arena, g1), upload(arena, g2), upload(arena, cs),
                              upload(arena, sn), 1e-5f, nullptr);
     ok = ok && layer.use_moe(arena, ffn) && layer.cache.tiled;
@@ -534,6 +583,8 @@ int main()
     test_decode_attention(ctx);
     test_kv_cache(ctx, 40, "kv_cache_append_attend_vs_oracle");
     test_kv_cache(ctx, 64, "kv_cache_tiled_layouts_append_attend_vs_oracle");
+    test_paged_kv_cache(ctx, false, "paged_kv_cache_row_major_equals_dense");
+    test_paged_kv_cache(ctx, true, "paged_kv_cache_tiled_equals_dense");
     test_decoder_layer(ctx);
     test_decoder_stack(ctx);
     test_moe_decoder_layer(ctx);

@@ -279,3 +279,117 @@ def test_vt_attention_with_projection_is_the_two_calls(mi, dev, B, Hq, Hkv, T_ca
     assert np.isfinite(a).all() and np.abs(a).max() > 0
     assert np.array_equal(r0, r1)
     assert np.array_equal(a, b) and np.array_equal(a, c)
+
+
+# ---- the paged form of the tiled cache, and the gate on the tiled kernel's own integers
+
+def to_pages(dense, table, Hkv, per_page):
+    """dense [B, Hkv, nblk, per_page...] -> pool [pages, Hkv, per_page...] under table [B, max_pages] (unused pages: junk)"""
+    B, _, nblk = dense.shape[:3]
+    pages = int(table.max()) + 1
+    pool = np.random.default_rng(5).integers(-100, 100, (pages, Hkv) + dense.shape[3:]).astype(dense.dtype)
+    for b in range(B):
+        for i in range(nblk):
+            if table[b, i] >= 0:
+                pool[table[b, i]] = dense[b, :, i]
+    return pool
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T_cap,lens", [
+    (2, 8, 2, 256, [256, 256]), (3, 8, 2, 512, [512, 65, 300]), (4, 16, 4, 1024, [1000, 1, 64, 129]),
+    (16, 32, 8, 4096, [4096] * 16),            # the decode-attention configuration at full size
+    (1, 32, 8, 2048, [1999]),                  # one sequence: many splits
+])
+def test_paged_tiled_attention_equals_dense(mi, dev, orc, B, Hq, Hkv, T_cap, lens):
+    """The same cache cut into 64-token pages that lie in a shuffled pool: the output equals the dense layout's bit
+    for bit (and the oracle within the gate, through the dense test above); table entries behind a sequence's last
+    block are poisoned."""
+    mark = dev.mark()
+    lens = np.array(lens, np.int32)
+    q, kq, ks, vq, vs, _, _ = make_cache(mi, dev, 900 + T_cap, B, Hq, Hkv, T_cap, T_cap)
+    dkt, dvt = convert(mi, dev, kq, vq, T_cap, T_cap)
+    nblk = T_cap // 64
+    g = np.random.default_rng(B + T_cap)
+    table = g.permutation(B * nblk + 7)[:B * nblk].reshape(B, nblk).astype(np.int32)
+    kt_pool = to_pages(dev.download(dkt).reshape(B, Hkv, nblk, 8192), table, Hkv, 8192)
+    vt_pool = to_pages(dev.download(dvt).reshape(B, Hkv, nblk, 8192), table, Hkv, 8192)
+    ks_pool = to_pages(ks.reshape(B, Hkv, nblk, 64), table, Hkv, 64)
+    vs_pool = to_pages(vs.reshape(B, Hkv, nblk, 64), table, Hkv, 64)
+    poisoned = table.copy()
+    for b in range(B):
+        poisoned[b, (int(lens[b]) + 63) // 64:] = 0x3FFFFFF   # never looked up
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, 128, T_cap), np.uint8)
+    dq, dks, dvs, dl = dev.upload(q), dev.upload(ks), dev.upload(vs), dev.upload(lens)
+    dense_o, paged_o = dev.empty((B, Hq, 128), np.float32), dev.empty((B, Hq, 128), np.float32)
+    mi.check(mi.lib.mi_gqa_decode_attn_tiled(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, dense_o.ptr, B, Hq, Hkv, 128, T_cap,
+                                             dl.ptr, T_cap, 0, ws.ptr, ws.nbytes, None))
+    dev.sync()
+    args = (dev.upload(kt_pool), dev.upload(ks_pool), dev.upload(vt_pool), dev.upload(vs_pool))
+    mi.check(mi.lib.mi_gqa_decode_attn_tiled_paged(dq.ptr, args[0].ptr, args[1].ptr, args[2].ptr, args[3].ptr, paged_o.ptr,
+                                                   dev.upload(poisoned).ptr, nblk, B, Hq, Hkv, 128, dl.ptr, T_cap, 0,
+                                                   ws.ptr, ws.nbytes, None), "mi_gqa_decode_attn_tiled_paged")
+    od, op = dev.download(dense_o), dev.download(paged_o)
+    assert np.array_equal(od, op)
+    for b in range(B):   # and the dense result is the oracle's, sequence by sequence
+        L = int(lens[b])
+        oo = orc.gqa_decode(q[b:b + 1], kq[b:b + 1, :, :L], ks[b:b + 1, :, :L], vq[b:b + 1, :, :L], vs[b:b + 1, :, :L])
+        assert np.max(np.abs(op[b:b + 1] - oo)) <= 2e-5
+    dev.reset_to(mark)
+
+
+def test_paged_tiled_append_equals_dense_append(mi, dev):
+    """Tokens appended one decode step at a time into a paged pool land exactly where the dense append puts them."""
+    mark = dev.mark()
+    B, Hkv, T_cap, D = 3, 2, 192, 128
+    nblk = T_cap // 64
+    g = np.random.default_rng(3)
+    table = g.permutation(B * nblk + 3)[:B * nblk].reshape(B, nblk).astype(np.int32)
+    pages = int(table.max()) + 1
+    dkt, dvt = dev.empty((B, Hkv, nblk, 8192), np.int8), dev.empty((B, Hkv, nblk, 8192), np.int8)
+    dks, dvs = dev.empty((B, Hkv, T_cap), np.float32), dev.empty((B, Hkv, T_cap), np.float32)
+    pkt, pvt = dev.empty((pages, Hkv, 8192), np.int8), dev.empty((pages, Hkv, 8192), np.int8)
+    pks, pvs = dev.empty((pages, Hkv, 64), np.float32), dev.empty((pages, Hkv, 64), np.float32)
+    for buf in (dkt, dvt, dks, dvs, pkt, pvt, pks, pvs):
+        mi.check(mi.lib.mi_fill_u32(buf.ptr, 0, buf.nbytes // 4, None))
+    dtab = dev.upload(table)
+    positions = [np.array([0, 63, 64], np.int32), np.array([1, 64, 191], np.int32), np.array([70, 5, 130], np.int32)]
+    for step, pos in enumerate(positions):
+        k_new = workload.normal(40 + step, (B, Hkv * D), 0)
+        v_new = workload.normal(40 + step, (B, Hkv * D), 1)
+        dk, dv, dp = dev.upload(k_new), dev.upload(v_new), dev.upload(pos)
+        mi.check(mi.lib.mi_kv_append_tiled_f32_i8(dk.ptr, dv.ptr, Hkv * D, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, dp.ptr,
+                                                  B, Hkv, D, T_cap, None))
+        mi.check(mi.lib.mi_kv_append_tiled_paged_f32_i8(dk.ptr, dv.ptr, Hkv * D, pkt.ptr, pks.ptr, pvt.ptr, pvs.ptr,
+                                                        dtab.ptr, nblk, dp.ptr, B, Hkv, D, None),
+                 "mi_kv_append_tiled_paged_f32_i8")
+    dev.sync()
+    kt, vt, ks, vs = (dev.download(x) for x in (dkt, dvt, dks, dvs))
+    gkt, gvt, gks, gvs = (dev.download(x) for x in (pkt, pvt, pks, pvs))
+    for b in range(B):
+        for i in range(nblk):
+            pg = table[b, i]
+            assert np.array_equal(gkt[pg], kt[b, :, i]) and np.array_equal(gvt[pg], vt[b, :, i])
+            assert np.array_equal(gks[pg], ks[b, :, 64 * i:64 * i + 64]) and np.array_equal(gvs[pg], vs[b, :, 64 * i:64 * i + 64])
+    dev.reset_to(mark)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,T_cap", [
+    (2, 8, 2, 256, 256), (1, 4, 1, 16, 64), (1, 32, 8, 1000, 1024), (3, 6, 3, 77, 128), (1, 8, 2, 4096, 4096),
+])
+def test_tiled_kernel_scores_are_the_oracles_integers(mi, dev, orc, B, Hq, Hkv, T, T_cap):
+    """The tiled kernel's own query codes, query scales and raw int32 dots (the products of its matrix instructions
+    on the tiled keys), against the oracle's: bit for bit."""
+    mark = dev.mark()
+    q, kq, ks, vq, vs, ks_c, vs_c = make_cache(mi, dev, 500 + T, B, Hq, Hkv, T, T_cap)
+    dkt, dvt = convert(mi, dev, kq, vq, T, T_cap)
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, 128, T_cap), np.uint8)
+    dqq, dsq, ddots = dev.empty((B, Hq, 128), np.int8), dev.empty((B, Hq), np.float32), dev.empty((B, Hq, T), np.int32)
+    mi.check(mi.lib.mi_fill_u32(ddots.ptr, 0x7F7F7F7F, ddots.nbytes // 4, None))
+    mi.check(mi.lib.mi_gqa_decode_scores_tiled_i32(dev.upload(q).ptr, dkt.ptr, dev.upload(ks_c).ptr, dvt.ptr,
+                                                   dev.upload(vs_c).ptr, dqq.ptr, dsq.ptr, ddots.ptr, B, Hq, Hkv, 128,
+                                                   T_cap, T, ws.ptr, ws.nbytes, None), "mi_gqa_decode_scores_tiled_i32")
+    _, qq, sq, dots = orc.gqa_decode(q, kq, ks, vq, vs, want_debug=True)
+    assert np.array_equal(dev.download(dqq), qq)
+    assert np.array_equal(dev.download(dsq), sq)
+    assert np.array_equal(dev.download(ddots), dots)
+    dev.reset_to(mark)

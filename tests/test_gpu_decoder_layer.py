@@ -199,7 +199,7 @@ def test_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B, H, 
     g1 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
     g2 = (1 + 0.1 * g.standard_normal(H)).astype(np.float32)
     layer = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T_cap, fw["qkv"], fw["o"], fw["gu"], fw["d"], g1, g2, cos, sin, eps,
-                            trace=True)
+                            trace=True, tiled=T_cap % 64 == 0)
     W = {k: orc.rotate_quant_rows(v, 128) for k, v in fw.items()}
     for k, dv in (("qkv", layer.wqkv), ("o", layer.wo), ("gu", layer.wgu), ("d", layer.wd)):
         assert np.array_equal(dev.download(dv[0]), W[k][0]) and np.array_equal(dev.download(dv[1]), W[k][1])
@@ -428,7 +428,7 @@ def test_moe_decoder_layer_decode_steps_follow_the_oracle_chain(mi, dev, orc, B,
         q, sc = orc.rotate_quant_rows(workload.weights(45, E * n, k, len(name) + n), b)
         moe["w" + name], moe["s" + name] = q.reshape(E, n, k), sc.reshape(E, n)
     layer = mi.DecoderLayer(dev, B, H, Hq, Hkv, I, T_cap, fw["qkv"], fw["o"], None, None, g1, g2, cos, sin, eps,
-                            trace=True, moe=moe)
+                            trace=True, tiled=T_cap % 64 == 0, moe=moe)
     W = {k: orc.rotate_quant_rows(v, 128) for k, v in fw.items()}
     W["g1"], W["g2"] = g1, g2
     start = np.array(start, np.int32)
