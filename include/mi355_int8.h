@@ -291,9 +291,14 @@ MI_API int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, int64
  *   vt int8 [B, Hkv, T_cap/64, 8, 4, 16, 16]  block of 64 tokens, transposed, in 16 x 16 pieces:
  *                                          byte (d / 16, (t % 64) / 16, d % 16, t % 16) = code d of token t
  * ks, vs fp32 [B, Hkv, T_cap] as above (16-byte aligned); T_cap % 64 == 0.  Both products of the attention run on
- * the int8 matrix pipe (the softmax weights times the V scales enter as 28-bit fixed-point numbers, finer than
- * fp32's mantissa, so the result is that of the fp32 accumulation to within rounding): the fast layout, and the one
- * the decode-layer chain uses.  seq_len may be NULL (every sequence holds T_max tokens).  Workspace:
+ * the int8 matrix pipe.  The softmax weights times the V scales enter the second one as 28-bit fixed-point numbers:
+ * w_t = exp2(s_t - m) * vs_t is rounded to the nearest multiple of u = vmax * 2^-28, vmax the largest V scale among
+ * the tokens of one split (at most 1024 of them), so a token whose V scale is vmax / r keeps 28 - log2(r) bits of
+ * its weight.  Against the fp32 accumulation of the row-major kernel an output element therefore differs by at most
+ * (tokens of the split) * 127 * u / 2 per split before the division by the softmax sum (which is >= 1), i.e. by
+ * T * 127 * 2^-29 * vmax in all (a worst case with every rounding the same way): invisible while the V scales of a split lie within
+ * two or three decades of each other (what a Hadamard-rotated cache holds), and a loss of precision that grows
+ * with the spread beyond that.  This is the fast layout, and the one the decode-layer chain uses.  seq_len may be NULL (every sequence holds T_max tokens).  Workspace:
  * mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T_max) (one query serves both layouts).  Bytes that belong to tokens
  * at or past a sequence's length are never used (they may hold anything).  No upstream counterpart. */
 MI_API int32_t mi_gqa_decode_attn_tiled(const float *q, const int8_t *kt, const float *ks,

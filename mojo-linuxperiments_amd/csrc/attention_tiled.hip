@@ -13,7 +13,8 @@
 //   P.V      o[h, d]    = sum_t p[t, h] * vs[t] * vq[t, d]   A = 16 rows x 64 tokens, B = a vt piece (64 t x 16 d)
 //
 // For the second product the fp32 weights a[t, h] = exp2(s[t, h] - m[h]) * vs[t] are written as fixed-point
-// numbers of 28 bits relative to the largest V scale of the workgroup's span (finer than the fp32 mantissa) and
+// numbers of 28 bits relative to the largest V scale of the workgroup's span (rounded to nearest: a token whose V
+// scale is 1/r of that largest one keeps 28 - log2(r) bits of its weight, more than fp32's 24 while r < 16) and
 // cut into four 7-bit digits; digit k of head h is row 4*k + h of A, so that ONE instruction multiplies all four
 // digits of the four heads with the block, and the four int32 partial sums are recombined in fp32 when the wave is
 // done.  Inside a wave the sums are exact integers (any order), across waves and splits fp32 as before.
@@ -302,7 +303,7 @@ __global__ __launch_bounds__(64 * NW) void k_gqa_tiled_split(Params p)
             const float pe = __builtin_amdgcn_exp2f(ss[e] - m_h);       // masked token: exp2(-inf) = 0
             lsum += pe;
             const float a = (pe == 0.0f) ? 0.0f : pe * (vv[e] * fix);   // (a masked token's scale may be anything)
-            code[e] = min((unsigned)a, 0x0fffffffu);
+            code[e] = min((unsigned)(a + 0.5f), 0x0fffffffu);           // to nearest; the clamp covers a = 2^28
         }
         v4i pa;
         static_for<4>([&](auto K) {

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <utility>
 
 #include "../../include/mi355_int8.h"
@@ -37,6 +38,32 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 int32_t compute_units();   // of the current device, cached
+int32_t lds_limit();       // largest LDS allocation of one workgroup on the current device, cached
+
+// A kernel's dynamic-LDS limit is a setting of the (kernel, device) pair: raised once for every device that the
+// kernel is launched on, and refused where the device cannot give that much.  One LdsOptIn per kernel
+// instantiation (a function-local static); a race between two first launches only repeats the call.
+struct LdsOptIn {
+    std::atomic<uint64_t> devices{0};
+};
+inline int32_t lds_opt_in(LdsOptIn &st, const void *kernel, int bytes)
+{
+    int dev = 0;
+    MI_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return MI_EINVAL;
+    const uint64_t bit = 1ull << dev;
+    if (st.devices.load(std::memory_order_acquire) & bit) return MI_OK;
+    if (bytes > lds_limit()) return MI_ENOSPC;
+    MI_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    st.devices.fetch_or(bit, std::memory_order_release);
+    return MI_OK;
+}
+#define MI_LDS_OPT_IN(kernel, bytes)                                                              \
+    do {                                                                                          \
+        static ::mi::LdsOptIn _st;                                                                \
+        const int32_t _rc = ::mi::lds_opt_in(_st, reinterpret_cast<const void *>(kernel), bytes); \
+        if (_rc != MI_OK) return _rc;                                                             \
+    } while (0)
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));

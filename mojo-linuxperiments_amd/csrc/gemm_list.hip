@@ -562,7 +562,6 @@ struct mi_gemm_batch {
     int32_t grid, per_wg;
     int64_t mnk[3 * list::MAX_PROBLEMS];
     const v4i *lists;   // device memory of the caller
-    std::atomic<bool> attr_set[2];
 };
 
 extern "C" int64_t mi_gemm_batch_plan_bytes(const int64_t *mnk, int32_t n)
@@ -613,7 +612,6 @@ extern "C" int32_t mi_gemm_batch_create(const int64_t *mnk, int32_t n, void *pla
     b->per_wg = per_wg;
     for (int i = 0; i < 3 * n; ++i) b->mnk[i] = mnk[i];
     b->lists = static_cast<const v4i *>(plan);
-    b->attr_set[0] = b->attr_set[1] = false;
     *out = b;
     return MI_OK;
 }
@@ -648,11 +646,7 @@ static int32_t batch_run(mi_gemm_batch *b, const mi_gemm_problem *p, void *strea
     int dev = -1;
     MI_HIP(hipGetDevice(&dev));
     if (dev != b->device) return MI_EINVAL;   // the list lives in that device's memory
-    const void *fn = reinterpret_cast<const void *>(&list::k_w8a8_list<DEQ>);
-    if (!b->attr_set[DEQ].load(std::memory_order_acquire)) {
-        MI_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, list::LC::LDS));
-        b->attr_set[DEQ].store(true, std::memory_order_release);
-    }
+    MI_LDS_OPT_IN((&list::k_w8a8_list<DEQ>), list::LC::LDS);
     hipLaunchKernelGGL((list::k_w8a8_list<DEQ>), dim3((unsigned)b->grid), dim3(512), list::LC::LDS,
                        as_stream(stream), bt, b->lists, b->per_wg);
     return launch_status();

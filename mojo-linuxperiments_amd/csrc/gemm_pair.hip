@@ -370,12 +370,9 @@ static int32_t launch(const int8_t *qx, const float *sx, const int8_t *qw, const
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
     constexpr int LDS = Cfg<TM, TN>::LDS;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_w8a8_pair<TM, TN, DEQ>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        attr_set = true;
-    }
+    // the kernel has no bounds checks: its direct-to-LDS loads and its stores address whole tiles and whole stages
+    if (M <= 0 || N <= 0 || M % BM != 0 || N % BN != 0 || K < 128 || K % 128 != 0) return MI_EINVAL;
+    MI_LDS_OPT_IN((&k_w8a8_pair<TM, TN, DEQ>), LDS);
     Grid gg;
     gg.tiles_m = (M + BM - 1) / BM;
     gg.tiles_n = (N + BN - 1) / BN;

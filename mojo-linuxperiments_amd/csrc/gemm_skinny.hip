@@ -388,12 +388,7 @@ static int32_t launch_fused(const float *x, const int8_t *qw, const float *sw, f
     constexpr int R = (16 / CW) < 1 ? 1 : (16 / CW);
     constexpr int V = pow2_ceil(R * MB);
     const size_t lds = (size_t)MB * K + (MB + 4 + 4 * CQ) * sizeof(float) + 4 * V * sizeof(int);
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_fused<MB, CW, CQ, NORM, ROT>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        attr_set = true;
-    }
+    MI_LDS_OPT_IN((&k_gemv_fused<MB, CW, CQ, NORM, ROT>), 96 * 1024);
     // Every workgroup reads the whole activation row (with the norm: the residual and the gain too, 48 KB at
     // K = 4096) before its first dot product.  Beyond two workgroups per compute unit a workgroup therefore takes
     // several groups of rows in turn, the next group's weights on their way while it works on the current one.
@@ -642,12 +637,7 @@ static int32_t launch_dot4(const int8_t *qx, const float *sx, const int8_t *qw, 
                            float *y, int M, int N, int K, hipStream_t s)
 {
     const size_t lds = (size_t)MB * K;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemv_dot4<MB, DEQ>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
-    }
+    MI_LDS_OPT_IN((&k_gemv_dot4<MB, DEQ>), 160 * 1024);
     const int cus = compute_units();
     // one or two workgroups per compute unit, each with a contiguous span of at least 8 rows
     int grid = lds <= 64 * 1024 ? 2 * cus : cus;
@@ -690,12 +680,7 @@ static int32_t launch_ring(const int8_t *qx, const float *sx, const int8_t *qw, 
     size_t lds = (size_t)nwave * D * STAGE;
     const size_t part = (size_t)nwave * NG * MT * 4 * 64 * sizeof(int);
     if (part > lds) lds = part;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_skinny_ring<NG, MT, D, DEQ>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
-    }
+    MI_LDS_OPT_IN((&k_skinny_ring<NG, MT, D, DEQ>), 160 * 1024);
     const unsigned grid = (unsigned)((N + 16 * NG - 1) / (16 * NG));
     hipLaunchKernelGGL((k_skinny_ring<NG, MT, D, DEQ>), dim3(grid), dim3((unsigned)(64 * nwave)), lds, s, qx, qw, sx,
                        sw, acc, y, M, N, K);

@@ -393,12 +393,10 @@ static int32_t launch_shape(const int8_t *qx, const float *sx, const int8_t *qw,
 {
     constexpr int BM = 32 * TM, BN = 32 * TN;
     constexpr int LDS = TiledCfg<TM, TN>::LDS;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_w8a8_tiled<TM, TN, DEQ>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        attr_set = true;
-    }
+    // ragged M and N are the kernel's to clamp; the K loop moves whole 128-byte stages and the stores whole
+    // 16-column groups, which nothing behind this line checks again
+    if (M <= 0 || N <= 0 || N % 16 != 0 || K < 128 || K % 128 != 0) return MI_EINVAL;
+    MI_LDS_OPT_IN((&k_w8a8_tiled<TM, TN, DEQ>), LDS);
     GemmGrid gg;
     gg.tiles_m = (M + BM - 1) / BM;
     gg.tiles_n = (N + BN - 1) / BN;

@@ -943,12 +943,7 @@ static int32_t launch_dispatch(const int32_t *idx, int32_t *perm, int32_t *seg_o
     if (T * topk > (1LL << 24) || E > 65535) return MI_ERANGE;
     const int64_t words = 2 * E * ((T + 31) / 32) + E + 1;
     if (words > moe::DISPATCH_MAX_WORDS) return MI_ERANGE;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_dispatch),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)(moe::DISPATCH_MAX_WORDS * 4)));
-        attr_set = true;
-    }
+    MI_LDS_OPT_IN((&moe::k_moe_dispatch), (int)(moe::DISPATCH_MAX_WORDS * 4));
     hipLaunchKernelGGL(moe::k_moe_dispatch, dim3(1), dim3(1024), (size_t)words * 4, as_stream(stream), idx, perm,
                        seg_off, order, (int)T, (int)E, (int)topk);
     return launch_status();
@@ -1014,14 +1009,8 @@ static int32_t run_ffn(const float *x, const int32_t *idx, const float *w, const
         rc = mi_fwht_quant_f32_i8(x, qx, sx, T, H, 128, stream);
         if (rc) return rc;
     }
-    static bool attr_set = false;  // idempotent; a race only repeats the calls
-    if (!attr_set) {
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_gemm<false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, moe::EXPERT_LDS));
-        MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_gemm<true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, moe::EXPERT_LDS));
-        attr_set = true;
-    }
+    MI_LDS_OPT_IN((&moe::k_moe_expert_gemm<false>), moe::EXPERT_LDS);
+    MI_LDS_OPT_IN((&moe::k_moe_expert_gemm<true>), moe::EXPERT_LDS);
     // Row chunks per workgroup: with the activation fragments in registers a workgroup walks several chunks
     // against them; about four workgroups per compute unit keep the stream dense.
     const int cus = compute_units();
@@ -1037,12 +1026,7 @@ static int32_t run_ffn(const float *x, const int32_t *idx, const float *w, const
         const dim3 grid((unsigned)(y_split * wpe + (E - y_split) * wpe2));
 #define MI_RX_GU(NS)                                                                                            \
     do {                                                                                                        \
-        static bool set = false;                                                                                \
-        if (!set) {                                                                                             \
-            MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<false, NS>),        \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::rx_lds(false)));        \
-            set = true;                                                                                         \
-        }                                                                                                       \
+        MI_LDS_OPT_IN((&moe::k_moe_expert_rx<false, NS>), moe::rx_lds(false));                                        \
         hipLaunchKernelGGL((moe::k_moe_expert_rx<false, NS>), grid, dim3(256), moe::rx_lds(false), s, qx, sx, perm, seg, \
                            wg, sg, wu, su, h, (int)H, (int)I, (int)I, (int)topk, nch, order, chunks, y_split);  \
     } while (0)
@@ -1067,12 +1051,7 @@ static int32_t run_ffn(const float *x, const int32_t *idx, const float *w, const
         const dim3 grid((unsigned)(y_split * wpe + (E - y_split) * wpe2));
 #define MI_RX_DN(NS)                                                                                            \
     do {                                                                                                        \
-        static bool set = false;                                                                                \
-        if (!set) {                                                                                             \
-            MI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&moe::k_moe_expert_rx<true, NS>),         \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, moe::rx_lds(true)));         \
-            set = true;                                                                                         \
-        }                                                                                                       \
+        MI_LDS_OPT_IN((&moe::k_moe_expert_rx<true, NS>), moe::rx_lds(true));                                        \
         hipLaunchKernelGGL((moe::k_moe_expert_rx<true, NS>), grid, dim3(256), moe::rx_lds(true), s, hq, hs, perm, seg, wd, \
                            sd, (const int8_t *)nullptr, (const float *)nullptr, out, (int)I, (int)H, (int)H,    \
                            (int)topk, nch, order, chunks, y_split);                                             \

@@ -28,6 +28,19 @@ int32_t compute_units()
     return cached[dev];
 }
 
+int32_t lds_limit()
+{
+    static int32_t cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 64 * 1024;
+    if (cached[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || v <= 0) v = 64 * 1024;
+        cached[dev] = v;
+    }
+    return cached[dev];
+}
+
 int32_t linear_scratch_bind(int device, unsigned char **out);   // gemm.hip: address of the static scratch array
 
 __global__ void k_fill_u32(uint32_t *dst, uint32_t value, int64_t count)

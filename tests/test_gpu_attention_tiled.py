@@ -393,3 +393,37 @@ def test_tiled_kernel_scores_are_the_oracles_integers(mi, dev, orc, B, Hq, Hkv, 
     assert np.array_equal(dev.download(dsq), sq)
     assert np.array_equal(dev.download(ddots), dots)
     dev.reset_to(mark)
+
+
+def test_vt_weights_with_v_scales_over_six_decades(mi, dev, orc):
+    """The fixed-point weights are relative to the largest V scale of a split.  Here the V scales spread over six
+    decades and the softmax mass sits on the tokens with the SMALLEST scales (their keys are the query scaled up),
+    so their weights keep only about 28 - 20 bits: the output must stay inside the bound the header states,
+    T * 127 * 2^-29 * vmax, and, the roundings being to nearest, well inside it (1 % of the output's size)."""
+    mark = dev.mark()
+    B, Hq, Hkv, T, D = 1, 4, 1, 1024, 128
+    g = np.random.default_rng(15)
+    q = g.standard_normal((B, Hq, D)).astype(np.float32)
+    q[0, 1:] = q[0, 0]                               # one direction, so that the same tokens win for every head
+    mag = np.exp(g.uniform(-7.0, 7.0, (T, 1)))
+    v = (g.standard_normal((T, D)) * mag).astype(np.float32)
+    k = g.standard_normal((T, D)).astype(np.float32)
+    small = np.argsort(mag[:, 0])[:48]
+    k[small] = 3.0 * q[0, 0]
+    kq, ks = orc.rotate_quant_rows(k, D)
+    vq, vs = orc.rotate_quant_rows(v, D)
+    kq, vq = kq.reshape(B, Hkv, T, D), vq.reshape(B, Hkv, T, D)
+    ks, vs = ks.reshape(B, Hkv, T), vs.reshape(B, Hkv, T)
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, D, T), np.uint8)
+    do = dev.empty((B, Hq, D), np.float32)
+    mi.check(mi.lib.mi_gqa_decode_attn_tiled(dev.upload(q).ptr, dev.upload(to_tiles(kq, T)).ptr, dev.upload(ks).ptr,
+                                             dev.upload(to_blocks(vq, T)).ptr, dev.upload(vs).ptr, do.ptr, B, Hq, Hkv, D,
+                                             T, None, T, 1, ws.ptr, ws.nbytes, None))
+    o = dev.download(do)
+    oo = orc.gqa_decode(q, kq, ks, vq, vs, out_rotated=True)
+    size = float(np.max(np.abs(oo)))
+    assert size < 1e-3 * float(vs.max()) * 127          # the mass really is on the small-scale tokens
+    err = float(np.max(np.abs(o - oo)))
+    assert err <= T * 127 * 2.0 ** -29 * float(vs.max())
+    assert err <= 1e-2 * size, (err, size)
+    dev.reset_to(mark)
