@@ -649,7 +649,7 @@ def gemm_timeline(mi, wl):
     lib = mi.lib
     if not hasattr(lib, "mi_debug_gemm_timeline"):
         sys.exit("bench.py --gemm-timeline-child needs the instrumented library (run bench.py --gemm-timeline)")
-    dev = mi.Device(arena_bytes=4 << 30)
+    dev = mi.Device(arena_bytes=6 << 30)
     pool = mi.StreamPool(dev, 1)
     s = pool.stream(0)
     M = wl.PREFILL_M
@@ -698,12 +698,85 @@ def gemm_timeline(mi, wl):
             "end_skew_us": round(float(t[:, :, 7].max() - t[:, :, 7].min()) / 100.0, 2),
         }
         dev.reset_to(mark)
+    out["batch"] = list_timeline(mi, wl, dev, s)
     print(json.dumps({"gemm_timeline": out, "M": M,
                       "note": "k_w8a8_pair, clock ticks = s_memtime read by waves 0 and 4 of every workgroup in the "
                               "last of 440 launches; real time = s_memrealtime (100 MHz); instrumented build "
                               "(libmi355_int8_timeline.so), five clock reads a wave outside the stage loop"}), flush=True)
     pool.destroy()
     dev.close()
+
+
+def list_timeline(mi, wl, dev, s):
+    """The batched GEMM (k_w8a8_list) on the four cfg3 projections as one launch: 240 launches on the benchmark's
+    codes, then the clock reads one more launch left for every tile of every workgroup: first stage begins, last
+    stage issued, last store of the tile issued."""
+    import ctypes as C
+    lib = mi.lib
+    M = wl.PREFILL_M
+    shapes = [(M, 6144, 4096), (M, 14336, 4096), (M, 14336, 4096), (M, 4096, 14336)]
+    mark = dev.mark()
+    ops = []
+    for i, (_, N, K) in enumerate(shapes):
+        m2 = dev.mark()
+        qx, sx = dev.empty((M, K), np.int8), dev.empty(M, np.float32)
+        mi.fwht_quant(dev.upload(wl.activations(2025, M, K, stream=K)), qx, sx, wl.HADAMARD_BLOCK)
+        qw, sw = dev.empty((N, K), np.int8), dev.empty(N, np.float32)
+        mi.fwht_quant(dev.upload(wl.weights(2025, N, K, stream=K + N + i)), qw, sw, wl.HADAMARD_BLOCK)
+        dev.sync()
+        host = [dev.download(b) for b in (qx, sx, qw, sw)]
+        dev.reset_to(m2)
+        ops.append(tuple(dev.upload(h) for h in host) + (dev.empty((M, N), np.float32),))
+    batch = mi.GemmBatch(dev, shapes)
+    for _ in range(200):
+        batch.run_f32(ops, stream=s)
+    e0, e1 = mi.Event(), mi.Event()
+    e0.record(s)
+    for _ in range(40):
+        batch.run_f32(ops, stream=s)
+    e1.record(s)
+    e1.synchronize()
+    us = e0.elapsed_ms(e1) / 40 * 1e3
+    WGS, TILES = 512, 16
+    f = lib.mi_debug_gemm_list_timeline
+    f.restype, f.argtypes = C.c_int32, [C.c_void_p, C.c_int32, C.c_int32]
+    mi.check(f(None, 0, 1))
+    batch.run_f32(ops, stream=s)
+    dev.sync(s)
+    buf = np.zeros(WGS * TILES * 8, np.uint64)
+    mi.check(f(buf.ctypes.data, buf.size, 0))
+    t = buf.reshape(WGS, TILES, 8).astype(np.int64)
+    valid = t[:, :, 6] == 1
+    wgs = int(valid.any(axis=1).sum())
+    nk = t[:, :, 5][valid]
+    loop = (t[:, :, 1] - t[:, :, 0])[valid]
+    fin = (t[:, :, 2] - t[:, :, 1])[valid]
+    real_us = (t[:, :, 4] - t[:, :, 3])[valid] / 100.0
+    first = np.broadcast_to(np.arange(TILES)[None, :] == 0, valid.shape)[valid]
+    per_k = {}
+    for k in np.unique(nk):
+        sel = nk == k
+        rec = {"tiles": int(sel.sum()), "loop_ticks_per_stage": round(float(loop[sel].mean() / k)),
+               "tile_us": round(float(real_us[sel].mean()), 2)}
+        for name, which in (("first_tile_of_a_workgroup", first), ("later_tiles", ~first)):
+            if (sel & which).any():
+                rec["loop_ticks_per_stage_" + name] = round(float(loop[sel & which].mean() / k))
+        per_k["stages_%d" % k] = rec
+    start = t[:, :, 3][valid].min()
+    ends = np.array([t[w, np.where(valid[w])[0][-1], 4] for w in range(WGS) if valid[w].any()])
+    res = {"kernel_us_event": round(us, 2), "workgroups": wgs, "tiles": int(valid.sum()),
+           "clock_mhz": round(float(((t[:, :, 2] - t[:, :, 0])[valid] / real_us).mean())),
+           "per_tile_depth": per_k, "mfma_per_simd_and_stage": 4 * 6 * 2 * 2,
+           "convert_and_store_ticks_per_tile": round(float(fin.mean())),
+           "loop_ticks_all_tiles": int(loop.sum()), "convert_and_store_ticks_all_tiles": int(fin.sum()),
+           "first_tile_start_to_last_store_us": round(float(ends.max() - start) / 100.0, 2),
+           "workgroup_end_before_the_last_one_us": {"mean": round(float(ends.max() - ends.mean()) / 100.0, 2),
+                                                    "p10": round(float(ends.max() - np.percentile(ends, 10)) / 100.0, 2)},
+           "note": "k_w8a8_list, one launch over the four cfg3 projections; clock ticks = s_memtime read by wave 0 of "
+                   "every workgroup at three points of every tile; instrumented build"}
+    batch.destroy()
+    dev.reset_to(mark)
+    return res
 
 
 def mfma_probe():
