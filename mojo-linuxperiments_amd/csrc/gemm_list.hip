@@ -31,8 +31,7 @@
 // compiler places (see gemm_pair_ops.h): fragments for two K halves and the addresses.
 //
 // Memory operations complete in issue order (one counter for loads and stores), and every wait below is written
-// against that order.  Only waves 0..3 (the ones the matrix pipe serves first) issue loads; every wave stores its
-// own results.
+// against that order.  Every wave issues an eighth of the loads and stores its own results.
 //
 // The list itself is made on the host when the batch is created (longest tiles first, each to the least loaded
 // workgroup of its XCD; tiles that run at the same time on one XCD are neighbours in column-major order, so they
@@ -80,7 +79,7 @@ struct Cfg {
     static constexpr int SCALES = (BM + BN) * 4;        // of one tile: BM row scales, then BN column scales
     static constexpr int SCALES_AT = STAGES;
     static constexpr int LDS = SCALES_AT + 2 * SCALES;  // two scale areas, by tile parity
-    static constexpr int LX = NBX / 8, LW = NBW / 8;    // parts (pairs of loads) per loading wave and stage
+    static constexpr int LX = NBX / 8, LW = NBW / 8;    // loads of a wave per stage
     static constexpr int NACC = TM * TN;                // accumulators of a set
     static constexpr int MIN_STAGES = 3;                // the loads run up to three stages ahead, into the next tile at most
     static_assert(LX == 4 && LW == 3, "the stage's load slots are written out for four and three parts");
@@ -109,6 +108,9 @@ __device__ __forceinline__ void dma16(const int8_t *sbase, unsigned voff, unsign
 #ifdef MI_GEMM_TIMELINE
 // Built only into libmi355_int8_timeline.so (bench.py --gemm-timeline): wave 0 of every workgroup leaves, per tile,
 // the clock ticks (s_memtime) and the 100 MHz real time at which the tile's first and last stage began and ended.
+#ifndef MI_TL_WAVE
+#define MI_TL_WAVE 0
+#endif
 constexpr int TL_WGS = 512, TL_TILES = 16;
 __device__ unsigned long long g_list_timeline[TL_WGS * TL_TILES * 8];
 #endif
@@ -158,11 +160,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
 
     const int tid = threadIdx.x, lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int pw = wave & 3;
     const int wm = wave >> 1, wn = wave & 1;   // wave tile: rows wm*64.., columns wn*96..
-    const bool loader = wave < 4;              // the waves the matrix pipe serves first issue every load
     const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
-    const unsigned lds_x = lds_base + pw * 1024, lds_w = lds_base + XAREA + pw * 1024;
+    const unsigned lds_x = lds_base + wave * 1024, lds_w = lds_base + XAREA + wave * 1024;
 
     const v4i *const my = lists + (int64_t)blockIdx.x * per_wg;
     // {problem or -1, first row, first column, -}: the tile the matrix pipe works on (three scalars, not the entry's four)
@@ -177,10 +177,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     static_for<NACC>([&](auto I) { vacc::acc_zero4<4 * decltype(I)::value>(); });
 
     // ---- load side.  The load cursor (a tile and a stage of it) runs two stages ahead of the matrix instructions.
-    // lane l = 8*rho + c fetches the 16-byte chunk c ^ sigma of row rho of a block; wave pw fills blocks pw + 4q,
-    // so one lane offset serves every block on a uniform base that moves with q
+    // lane l = 8*rho + c fetches the 16-byte chunk c ^ sigma of row rho of a block; wave w fills blocks w + 8q of
+    // a stage (four of the activations, three of the weights): every wave issues the same share of the loads, and
+    // one lane offset serves every block of a tile: base of the tile (two scalars) + this lane's offset + a scalar
+    // that moves with q and with the stage (one scalar and one vector addition a load; 64-bit scalar address
+    // arithmetic for every load, on four waves only, made those four waves the last at every barrier by 500 ticks)
     const int8_t *lx = nullptr, *lw = nullptr;
-    int64_t lbstep = 0;
+    unsigned lbstep = 0;
     unsigned lvoff = 0;
     int lkt = 0, lnk = 0;
     bool ldv = false;   // the cursor stands on a stage that exists
@@ -191,22 +194,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
         lkt = 0;
         lx = P.qx + (int64_t)e[1] * K;
         lw = P.qw + (int64_t)e[2] * K;
-        lbstep = (int64_t)32 * K;   // four blocks of eight rows
+        lbstep = 64u * (unsigned)K;   // eight blocks of eight rows
         const int l = opaque(lane0);
-        const int lrow = pw * 8 + (l >> 3);
-        const unsigned lchunk = (unsigned)(((l & 7) ^ (((pw & 1) << 2) | (l >> 4))) << 4);
+        const int lrow = wave * 8 + (l >> 3);
+        const unsigned lchunk = (unsigned)(((l & 7) ^ (((wave & 1) << 2) | (l >> 4))) << 4);
         lvoff = (unsigned)lrow * (unsigned)K + lchunk;
         ldv = true;
     };
     auto issue_x = [&](auto I, unsigned buf) {   // part p of the cursor's stage
         constexpr int p_ = decltype(I)::value;
-        dma16(lx + (int64_t)lkt * 128 + (2 * p_) * lbstep, lvoff, lds_x + buf + (2 * p_) * 4096);
-        dma16(lx + (int64_t)lkt * 128 + (2 * p_ + 1) * lbstep, lvoff, lds_x + buf + (2 * p_ + 1) * 4096);
+        dma16(lx, add_vs(lvoff, (unsigned)lkt * 128u + p_ * lbstep), lds_x + buf + p_ * 8192);
     };
     auto issue_w = [&](auto I, unsigned buf) {
         constexpr int p_ = decltype(I)::value;
-        dma16(lw + (int64_t)lkt * 128 + (2 * p_) * lbstep, lvoff, lds_w + buf + (2 * p_) * 4096);
-        dma16(lw + (int64_t)lkt * 128 + (2 * p_ + 1) * lbstep, lvoff, lds_w + buf + (2 * p_ + 1) * 4096);
+        dma16(lw, add_vs(lvoff, (unsigned)lkt * 128u + p_ * lbstep), lds_w + buf + p_ * 8192);
     };
 
     // ---- read side: fragment (16 rows, 64 K bytes): lane (r = l%16, g = l/16) reads row r, chunk 4*half + g
@@ -245,8 +246,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     // been issued (the second half's fragments during the first half) and, at the barrier, has landed; behind it the
     // next stage's buffers are read, the activation buffer takes the loads of stage + 2, and the weight buffer is
     // free for the stage after that (its loads are issued during the next stage's first half).
+#ifdef MI_GEMM_TIMELINE
+    unsigned tl_wait = 0, tl_bar = 0;   // ticks of a tile spent in the wait in front of the barrier / in the barrier
+#endif
     auto stage = [&]() {
-        const bool ld = loader && ldv;
+        const bool ld = ldv;
         using I0 = std::integral_constant<int, 0>;
         using I1 = std::integral_constant<int, 1>;
         using I2 = std::integral_constant<int, 2>;
@@ -264,14 +268,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                 if constexpr (j == 0) wait_lgkm<3>();        // x0..x3 and W0..W3 are in; W4, W5 and the read above may not be
                 if constexpr (j >= 4) wait_lgkm<9>();        // W4 (W5) is in: 8 reads of this half and W5 (W4') are younger
                 if constexpr (j == 4) {
-                    if (kt == 0 && loader) {   // this tile's scales, for the end of the tile
+                    if (kt == 0) {   // this tile's scales, for the end of the tile
                         if constexpr (DEQ) {
+                            // waves 0..3: row scales 64 w ..; waves 4..6: column scales 64 (w - 4) ..; wave 7 has
+                            // none left and fetches wave 3's again (every wave counts the same memory operations)
                             const Problem &P = bt.p[e_p];
-                            const float *s0 = P.sx + e_m0 + pw * 64;                                     // row scales 64 pw ..
-                            const float *s1 = pw < 3 ? P.sw + e_n0 + pw * 64 : P.sx + e_m0 + pw * 64;   // column scales 64 pw .. (wave 3: none left)
+                            const int part = wave < 7 ? wave : 3;
+                            const float *s0 = part < 4 ? P.sx + e_m0 + part * 64 : P.sw + e_n0 + (part - 4) * 64;
                             const unsigned lo4 = (unsigned)opaque(lane0) * 4u;
-                            dma4(s0, lo4, lds_base + cur_scales + pw * 256);
-                            dma4(s1, lo4, lds_base + cur_scales + (pw < 3 ? BM * 4 + pw * 256 : pw * 256));
+                            dma4(s0, lo4, lds_base + cur_scales + (part < 4 ? part * 256 : BM * 4 + (part - 4) * 256));
                         }
                     }
                 }
@@ -289,16 +294,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
             // the next stage as well.  Memory operations complete in order; issued since the last load of the next
             // stage (its fourth activation part, in the stage before): in a tile's first stage the NACC stores of
             // the tile before it; this stage's three weight parts; in a tile's first stage its scales.
-            if (loader) {
-                constexpr int SC = DEQ ? 2 : 0;
+#ifdef MI_GEMM_TIMELINE
+            const unsigned tl_s0 = (unsigned)__builtin_amdgcn_s_memtime();
+#endif
+            {
+                constexpr int SC = DEQ ? 1 : 0, LW = C::LW;
                 if (!ldv) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(6 + SC + NACC) : "memory");
-                else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(6 + SC) : "memory");
-                else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
-            } else {
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LW + SC + NACC) : "memory");
+                else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LW + SC) : "memory");
+                else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LW) : "memory");
             }
+#ifdef MI_GEMM_TIMELINE
+            const unsigned tl_s1 = (unsigned)__builtin_amdgcn_s_memtime();
+#endif
             __builtin_amdgcn_s_barrier();
+#ifdef MI_GEMM_TIMELINE
+            tl_wait += tl_s1 - tl_s0;
+            tl_bar += (unsigned)__builtin_amdgcn_s_memtime() - tl_s1;
+#endif
             const unsigned nax0 = add_vs(xo0, xnxt), naw0 = add_vs(wo0, wnxt);
             ds_read128<0>(w[0], naw0);
             static_for<TN - 1>([&](auto J1) {
@@ -318,7 +331,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
             const unsigned u = wcur; wcur = wnxt; wnxt = wnn; wnn = u;
         }
     };
-    static_assert(6 + 2 + NACC + 8 <= 63, "the memory counter has six bits");
+    static_assert(C::LW + 1 + NACC + C::LX <= 63, "the memory counter has six bits");
 
     // The tile's accumulators leave: converted, scaled by the row and the column scale, stored and cleared for the
     // next tile; accumulator (j, i) is named at compile time.  Two neighbouring column tiles are paired and swap
@@ -404,13 +417,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     // ---- fill: stages 0 and 1 of the first tile, then its first fragments
     cursor_to((v4i){e_p, e_m0, e_n0, 0});
     nk = bt.p[e_p].K >> 7;
-    if (loader) {
+    {
         static_for<4>([&](auto I) { issue_x(I, 0u); });
         static_for<3>([&](auto I) { issue_w(I, 0u); });
         lkt = 1;
         static_for<4>([&](auto I) { issue_x(I, (unsigned)XSTAGE); });
         static_for<3>([&](auto I) { issue_w(I, (unsigned)WSTAGE); });
-        wait_vm<14>();   // stage 0 has landed
+        wait_vm<7>();   // stage 0 has landed
     }
     lkt = 2;
     __syncthreads();
@@ -454,7 +467,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
 #ifdef MI_GEMM_TIMELINE
         {
             const unsigned long long tl_c = __builtin_amdgcn_s_memtime(), tl_rc = __builtin_amdgcn_s_memrealtime();
-            if (wave == 0 && opaque(lane0) == 0 && blockIdx.x < TL_WGS && it < TL_TILES) {
+            if (wave == MI_TL_WAVE && opaque(lane0) == 0 && blockIdx.x < TL_WGS && it < TL_TILES) {
                 unsigned long long *o = g_list_timeline + ((size_t)blockIdx.x * TL_TILES + it) * 8;
                 o[0] = tl_a;    // first stage begins (ticks)
                 o[1] = tl_b;    // last stage issued
@@ -463,8 +476,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                 o[4] = tl_rc;   // real time at o[2]
                 o[5] = (unsigned long long)nk;
                 o[6] = 1;
-                o[7] = tl_b;
+                o[7] = ((unsigned long long)tl_bar << 32) | tl_wait;
             }
+            tl_wait = tl_bar = 0;
         }
 #endif
         if (!more) break;
