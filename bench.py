@@ -116,6 +116,8 @@ def main():
                     help="context only: what a loop of v_mfma_i32_16x16x64_i8 alone sustains on this machine "
                          "(operands in registers, with and without the GEMM's LDS fragment reads, zeros and "
                          "activation-like codes); one JSON line")
+    ap.add_argument("--grid-wait-probe", action="store_true",
+                    help="time a grid-wide wait as a cooperative and as a plain launch (its own executable), then exit")
     ap.add_argument("--gemm-timeline", action="store_true",
                     help="context only: where the eight-wave GEMM's time goes (prologue / stage loop / stores, in "
                          "clock ticks read inside the kernel), from the instrumented build of the library; one JSON line")
@@ -144,6 +146,9 @@ def main():
 
     if args.mfma_probe:
         print(json.dumps(mfma_probe()), flush=True)
+        return
+    if args.grid_wait_probe:
+        print(json.dumps(run_probe("grid_wait_probe", "grid_wide_wait")), flush=True)
         return
     if args.gemm_timeline_child:
         return gemm_timeline(mi, wl)
@@ -779,17 +784,22 @@ def list_timeline(mi, wl, dev, s):
     return res
 
 
-def mfma_probe():
-    """Runs the matrix-pipe probe (its own process, csrc/probe_mfma_peak.hip) and returns its JSON, or None with
-    the reason when the executable is not built.  Context for the roofline, never part of `value`."""
+def run_probe(exe_name, key):
+    """Runs one of the measurement executables built by `make bench` (its own process) and returns its JSON line,
+    or {key: None, reason} when it is not built or fails."""
     import subprocess
-    exe = os.path.join(ROOT, "mojo-linuxperiments_amd", "mfma_peak_probe")
+    exe = os.path.join(ROOT, "mojo-linuxperiments_amd", exe_name)
     if not os.path.exists(exe):
-        return {"mfma_power_limited_peak": None, "reason": "mfma_peak_probe is not built (make -C mojo-linuxperiments_amd/csrc)"}
+        return {key: None, "reason": "%s is not built (make -C mojo-linuxperiments_amd/csrc bench)" % exe_name}
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     if r.returncode != 0:
-        return {"mfma_power_limited_peak": None, "reason": "probe failed: " + r.stderr.strip()[-200:]}
+        return {key: None, "reason": "probe failed: " + r.stderr.strip()[-200:]}
     return json.loads(r.stdout.strip().splitlines()[-1])
+
+
+def mfma_probe():
+    """The matrix-pipe probe (csrc/probe_mfma_peak.hip).  Context for the roofline, never part of `value`."""
+    return run_probe("mfma_peak_probe", "mfma_power_limited_peak")
 
 
 VENDOR_CHILD = r"""

@@ -100,24 +100,47 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) xr[tt] = x + (int64_t)min(t0 + tt, T - 1) * H + 4 * lane;
     const float *wp = wr + (int64_t)e0 * H + 4 * lane;
-    for (int j = 0; j < H / 256; ++j) {
-        float4 xv[4];
+    // Eight experts at a time: while the 128 FMAs of one half run, the weights of the next half (and, behind a
+    // second half, the token rows of the next round) are already on their way; with one wave per SIMD the loop is
+    // otherwise a chain of memory round trips.  Every dot product still takes its terms in the same order.
+    const int nj = H / 256;
+    float4 xv[4], xn[4], wa[8], wb[8];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * j);
-        float4 wv[16];
+    for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt]);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) wv[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H + 256 * j);
+    for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H);
+    for (int j = 0; j < nj; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wb[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)(8 + e) * H + 256 * j);
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
+            for (int e = 0; e < 8; ++e) {
                 float a = p[tt * 16 + e];
-                a = __builtin_fmaf(xv[tt].x, wv[e].x, a);
-                a = __builtin_fmaf(xv[tt].y, wv[e].y, a);
-                a = __builtin_fmaf(xv[tt].z, wv[e].z, a);
-                a = __builtin_fmaf(xv[tt].w, wv[e].w, a);
+                a = __builtin_fmaf(xv[tt].x, wa[e].x, a);
+                a = __builtin_fmaf(xv[tt].y, wa[e].y, a);
+                a = __builtin_fmaf(xv[tt].z, wa[e].z, a);
+                a = __builtin_fmaf(xv[tt].w, wa[e].w, a);
                 p[tt * 16 + e] = a;
             }
+        const int jn = min(j + 1, nj - 1);   // (the last round fetches itself again: no branch around loads)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H + 256 * jn);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) xn[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * jn);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float a = p[tt * 16 + 8 + e];
+                a = __builtin_fmaf(xv[tt].x, wb[e].x, a);
+                a = __builtin_fmaf(xv[tt].y, wb[e].y, a);
+                a = __builtin_fmaf(xv[tt].z, wb[e].z, a);
+                a = __builtin_fmaf(xv[tt].w, wb[e].w, a);
+                p[tt * 16 + 8 + e] = a;
+            }
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) xv[tt] = xn[tt];
     }
     fold<32, 32>(p, lane);
     fold<16, 16>(p, lane);

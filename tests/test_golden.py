@@ -130,6 +130,36 @@ def test_gpu_attention(mi, dev, gold):
 
 
 @pytest.mark.gpu
+def test_gpu_attention_tiled_layouts(mi, dev, gold):
+    """The same fixture through the cache in the matrix-pipe layouts (37 tokens in a cache of 64, junk scales behind
+    them): the kernel's own query codes, scales and int32 scores against the committed ones, bit for bit; outputs
+    within the gate."""
+    mark = dev.mark()
+    B, Hq, Hkv, T, _ = gen.ATTN
+    T_cap = 64
+    q, kq, ks, vq, vs = gen.attn_inputs()
+    pad = lambda a, fill: np.concatenate([a, np.full(a.shape[:2] + (T_cap - T,) + a.shape[3:], fill, a.dtype)], axis=2)
+    dkq, dvq = dev.upload(pad(kq, 77)), dev.upload(pad(vq, -77))
+    dks, dvs = dev.upload(pad(ks, np.nan)), dev.upload(pad(vs, np.nan))
+    dkt, dvt = dev.empty((B, Hkv, T_cap, 128), np.int8), dev.empty((B, Hkv, T_cap, 128), np.int8)
+    mi.check(mi.lib.mi_kv_tiled_from_rows_i8(dkq.ptr, dvq.ptr, dkt.ptr, dvt.ptr, B * Hkv, T, T_cap, T_cap, None))
+    dq = dev.upload(q)
+    ws = dev.empty(mi.lib.mi_gqa_decode_workspace_bytes(B, Hq, Hkv, 128, T_cap), np.uint8)
+    dqq, dsq, ddots = dev.empty((B, Hq, 128), np.int8), dev.empty((B, Hq), np.float32), dev.empty((B, Hq, T), np.int32)
+    mi.check(mi.lib.mi_gqa_decode_scores_tiled_i32(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, dqq.ptr, dsq.ptr, ddots.ptr,
+                                                   B, Hq, Hkv, 128, T_cap, T, ws.ptr, ws.nbytes, None))
+    assert np.array_equal(dev.download(dqq), gold["attn_qq"]) and np.array_equal(dev.download(dsq), gold["attn_sq"])
+    assert np.array_equal(dev.download(ddots), gold["attn_dots"])
+    do = dev.empty((B, Hq, 128), np.float32)
+    dlen = dev.upload(np.full(B, T, np.int32))
+    for rot, key in ((0, "attn_o"), (1, "attn_o_rot")):
+        mi.check(mi.lib.mi_gqa_decode_attn_tiled(dq.ptr, dkt.ptr, dks.ptr, dvt.ptr, dvs.ptr, do.ptr, B, Hq, Hkv, 128, T_cap,
+                                                 dlen.ptr, T, rot, ws.ptr, ws.nbytes, None))
+        assert np.max(np.abs(dev.download(do) - gold[key])) <= 2e-5
+    dev.reset_to(mark)
+
+
+@pytest.mark.gpu
 def test_gpu_moe(mi, dev, gold):
     mark = dev.mark()
     T, H, I, E, topk, _ = gen.MOE
