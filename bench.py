@@ -757,12 +757,16 @@ def list_timeline(mi, wl, dev, s):
     loop = (t[:, :, 1] - t[:, :, 0])[valid]
     fin = (t[:, :, 2] - t[:, :, 1])[valid]
     real_us = (t[:, :, 4] - t[:, :, 3])[valid] / 100.0
+    wait = (t[:, :, 7] & 0xffffffff)[valid]      # wave 0: ticks in the wait for its own loads in front of the stage's barrier
+    bar = (t[:, :, 7] >> 32)[valid]              # ... and in the barrier itself (each includes one clock read)
     first = np.broadcast_to(np.arange(TILES)[None, :] == 0, valid.shape)[valid]
     per_k = {}
     for k in np.unique(nk):
         sel = nk == k
         rec = {"tiles": int(sel.sum()), "loop_ticks_per_stage": round(float(loop[sel].mean() / k)),
-               "tile_us": round(float(real_us[sel].mean()), 2)}
+               "tile_us": round(float(real_us[sel].mean()), 2),
+               "of_a_stage_wave0_waits_for_its_loads_ticks": round(float(wait[sel].mean() / k)),
+               "of_a_stage_wave0_waits_in_the_barrier_ticks": round(float(bar[sel].mean() / k))}
         for name, which in (("first_tile_of_a_workgroup", first), ("later_tiles", ~first)):
             if (sel & which).any():
                 rec["loop_ticks_per_stage_" + name] = round(float(loop[sel & which].mean() / k))
@@ -778,7 +782,8 @@ def list_timeline(mi, wl, dev, s):
            "workgroup_end_before_the_last_one_us": {"mean": round(float(ends.max() - ends.mean()) / 100.0, 2),
                                                     "p10": round(float(ends.max() - np.percentile(ends, 10)) / 100.0, 2)},
            "note": "k_w8a8_list, one launch over the four cfg3 projections; clock ticks = s_memtime read by wave 0 of "
-                   "every workgroup at three points of every tile; instrumented build"}
+                   "every workgroup at three points of every tile and around the wait and the barrier of every stage "
+                   "(three reads a stage, about 100 ticks); instrumented build"}
     batch.destroy()
     dev.reset_to(mark)
     return res

@@ -7,6 +7,9 @@
 //   - one and two waves per SIMD (one wave cannot issue the instruction back to back at the pipe's full rate);
 //   - operands all zero, and int8 codes drawn like rotated, quantized activations (normal, sigma 30, clipped to 127);
 //   - with and without the LDS fragment reads of the 8 x 6 wave tile (14 ds_read_b128 to 48 matrix instructions).
+//   - "loop_variants": two waves per SIMD, activation-like codes, with what a GEMM's stage adds to the loop: more
+//     fragment reads (20 and 28 to 48 matrix instructions), direct-to-LDS loads from a small cache-resident buffer
+//     (7 and 14 KB per wave and 48 instructions), and a workgroup barrier every 48 instructions.
 // Prints one JSON line.  Measurement tool only: nothing in the library uses it.
 #include <hip/hip_runtime.h>
 
@@ -35,6 +38,15 @@ template <int OFF>
 __device__ __forceinline__ void rd(v4i &dst, unsigned addr)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+// direct-to-LDS load of 16 bytes per lane: global address = sbase + voff + OFF, LDS address = ldsaddr + OFF + 16 * lane
+template <int OFF>
+__device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned ldsaddr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(ldsaddr), "n"(OFF)
+                 : "memory", "m0");
 }
 template <int N, class F>
 __device__ __forceinline__ void sfor(F &&f)
@@ -82,6 +94,51 @@ __global__ __launch_bounds__(512) void k_mfma_loop(const unsigned *__restrict__ 
     if (lane == 0) ticks[blockIdx.x * 8 + wave] = t1 - t0;
 }
 
+// The loop of k_mfma_loop<true> with EXTRA more fragment reads per 48 matrix instructions (into a register nobody
+// uses), DMA direct-to-LDS loads of 1 KB per wave (four cache-resident lines of the code buffer, written behind
+// the fragment area), and, BAR = 1, a workgroup barrier after every 48 instructions.
+template <int EXTRA, int DMA, int BAR>
+__global__ __launch_bounds__(512) void k_mfma_mix(const unsigned *__restrict__ codes, long long *__restrict__ ticks,
+                                                  int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    asm volatile("" ::: "a0", "a31", "a63", "a95", "a127", "a159", "a191");
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned *l32 = reinterpret_cast<unsigned *>(smem);
+    for (int q = threadIdx.x; q < 16384; q += blockDim.x) l32[q] = codes[(blockIdx.x & 15) * 16384 + q];
+    __syncthreads();
+    const unsigned base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)smem;
+    const unsigned addr = base + wave * 8192 + lane * 16;
+    const unsigned dbase = __builtin_amdgcn_readfirstlane(base + 65536 + wave * 8192);
+    const unsigned voff0 = (unsigned)(lane * 16 + (blockIdx.x & 15) * 65536);
+    v4i xa[8], wb[6], junk;
+    sfor<8>([&](auto I) { rd<decltype(I)::value * 1024>(xa[decltype(I)::value], addr); });
+    sfor<6>([&](auto I) { rd<decltype(I)::value * 1024 + 512>(wb[decltype(I)::value], addr); });
+    rd<0>(junk, addr);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    const long long t0 = __builtin_amdgcn_s_memtime();
+    for (int it = 0; it < iters; ++it) {
+        sfor<48>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            mfma_acc<4 * i>(wb[i / 8], xa[i % 8]);
+            if constexpr (i >= 40) rd<(i - 40) * 1024>(xa[i - 40], addr);
+            if constexpr (i % 8 == 7 && i < 40) rd<(i / 8) * 1024 + 512>(wb[i / 8], addr);
+            if constexpr (i == 47) rd<5 * 1024 + 512>(wb[5], addr);
+            if constexpr (EXTRA > 0 && i < 40 && (i * EXTRA / 40) != ((i + 1) * EXTRA / 40)) rd<(i % 8) * 1024>(junk, addr);
+            if constexpr (DMA > 0 && i < 40 && (i * DMA / 40) != ((i + 1) * DMA / 40))
+                dma16<(i % 4) * 1024>(codes, voff0, dbase);
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (BAR) __builtin_amdgcn_s_barrier();
+        asm volatile("" ::"v"(junk));
+    }
+    asm volatile("s_nop 15\ns_nop 15" ::: "memory");
+    const long long t1 = __builtin_amdgcn_s_memtime();
+    if (lane == 0) ticks[blockIdx.x * 8 + wave] = t1 - t0;
+}
+
 struct Result {
     double ns_per_mfma, tops, tick_mhz, ticks_per_mfma;
 };
@@ -119,13 +176,43 @@ static Result run(const unsigned *codes, long long *ticks, int waves_per_simd, i
     return r;
 }
 
+template <int EXTRA, int DMA, int BAR>
+static void run_mix(const unsigned *codes, long long *ticks, int cus, bool first)
+{
+    const int iters = 4000;
+    CK(hipFuncSetAttribute((const void *)k_mfma_mix<EXTRA, DMA, BAR>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    float ms = 0;
+    for (int rep = 0; rep < 8; ++rep) {
+        CK(hipEventRecord(e0, 0));
+        hipLaunchKernelGGL((k_mfma_mix<EXTRA, DMA, BAR>), dim3(cus), dim3(512), 128 * 1024, 0, codes, ticks, iters);
+        CK(hipEventRecord(e1, 0));
+        CK(hipDeviceSynchronize());
+        CK(hipEventElapsedTime(&ms, e0, e1));
+    }
+    std::vector<long long> h((size_t)cus * 8);
+    CK(hipMemcpy(h.data(), ticks, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+    double mean = 0;
+    for (auto v : h) mean += (double)v;
+    mean /= (double)h.size();
+    const double per_simd = 48.0 * iters * 2;
+    printf("%s{\"fragment_reads_per_48\": %d, \"direct_to_lds_kb_per_48\": %d, \"barrier_per_48\": %s, \"tops\": %.0f, "
+           "\"ns_per_mfma\": %.2f, \"clock_ticks_per_mfma\": %.2f, \"clock_mhz\": %.0f}",
+           first ? "" : ", ", 14 + EXTRA, DMA, BAR ? "true" : "false",
+           2.0 * 16 * 16 * 64 * per_simd * 4 * cus / (ms * 1e-3) / 1e12, ms * 1e6 / per_simd, mean / per_simd, mean / (ms * 1e3));
+    CK(hipEventDestroy(e0));
+    CK(hipEventDestroy(e1));
+}
+
 int main()
 {
     hipDeviceProp_t prop;
     CK(hipGetDeviceProperties(&prop, 0));
     const int cus = prop.multiProcessorCount;
     // int8 codes like rotated, quantized activations: normal, sigma 30, clipped to +-127 (a fixed LCG + Box-Muller)
-    std::vector<unsigned> gauss(16 * 16384), zeros(16 * 16384, 0u);
+    std::vector<unsigned> gauss(17 * 16384), zeros(17 * 16384, 0u);   // (one more block: the mix loop's loads run past the 16th)
     unsigned long long st = 88172645463325252ull;
     auto uni = [&]() {
         st = st * 6364136223846793005ull + 1442695040888963407ull;
@@ -161,6 +248,15 @@ int main()
                 first = false;
             }
     }
+    printf("], \"loop_variants\": [");
+    run_mix<0, 0, 0>(dcodes, ticks, cus, true);
+    run_mix<6, 0, 0>(dcodes, ticks, cus, false);
+    run_mix<14, 0, 0>(dcodes, ticks, cus, false);
+    run_mix<0, 7, 0>(dcodes, ticks, cus, false);
+    run_mix<6, 7, 0>(dcodes, ticks, cus, false);
+    run_mix<6, 14, 0>(dcodes, ticks, cus, false);
+    run_mix<0, 0, 1>(dcodes, ticks, cus, false);
+    run_mix<6, 7, 1>(dcodes, ticks, cus, false);
     printf("]}}\n");
     CK(hipFree(dcodes));
     CK(hipFree(ticks));
