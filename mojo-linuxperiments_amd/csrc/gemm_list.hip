@@ -372,24 +372,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                 const char *sbase = base + i * rows16 + j * 64;
                 const char *sbase8 = sbase + rows8;
                 const unsigned vo_ = vo;   // (named outside the asm so that the lambda captures it)
-                // a0: column tile j, a1: column tile j + 1 of row tile i, read and cleared
-                v4i a0, a1;
-                asm volatile("v_mov_b32 %0, v%c4\n\tv_mov_b32 %1, v%c5\n\tv_mov_b32 %2, v%c6\n\tv_mov_b32 %3, v%c7\n\t"
-                             "v_mov_b32 v%c4, 0\n\tv_mov_b32 v%c5, 0\n\tv_mov_b32 v%c6, 0\n\tv_mov_b32 v%c7, 0"
-                             : "=&v"(a0[0]), "=&v"(a0[1]), "=&v"(a0[2]), "=&v"(a0[3])
-                             : "n"(r0), "n"(r0 + 1), "n"(r0 + 2), "n"(r0 + 3));
-                asm volatile("v_mov_b32 %0, v%c4\n\tv_mov_b32 %1, v%c5\n\tv_mov_b32 %2, v%c6\n\tv_mov_b32 %3, v%c7\n\t"
-                             "v_mov_b32 v%c4, 0\n\tv_mov_b32 v%c5, 0\n\tv_mov_b32 v%c6, 0\n\tv_mov_b32 v%c7, 0"
-                             : "=&v"(a1[0]), "=&v"(a1[1]), "=&v"(a1[2]), "=&v"(a1[3])
-                             : "n"(r1), "n"(r1 + 1), "n"(r1 + 2), "n"(r1 + 3));
-                v4i t0, t1;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    t0[q] = ror8(a0[q]);
-                    t1[q] = ror8(a1[q]);
-                }
-                const v4i vA = lo ? a0 : t1;  // rows 0-7:  lanes r<8 tile j (own), lanes r>=8 tile j+1 (from lane r-8)
-                const v4i vB = lo ? t0 : a1;  // rows 8-15: lanes r>=8 tile j+1 (own), lanes r<8 tile j (from lane r+8)
+                // vA: rows 0-7 of the pair's 16 rows: lanes r < 8 keep column tile j (their own), lanes r >= 8 take
+                // column tile j + 1 from lane r - 8; vB: rows 8-15: lanes r >= 8 keep tile j + 1, lanes r < 8 take
+                // tile j from lane r + 8.  One select with the rotation by eight lanes on its first source does both
+                // the exchange and the choice; the accumulators are read where they live and cleared behind it.
+                v4i vA, vB;
+                asm volatile("s_mov_b32 vcc_lo, 0x00ff00ff\n\ts_mov_b32 vcc_hi, 0x00ff00ff\n\t"
+                             "v_cndmask_b32_dpp %0, v%c12, v%c8, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %1, v%c13, v%c9, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %2, v%c14, v%c10, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %3, v%c15, v%c11, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "s_mov_b32 vcc_lo, 0xff00ff00\n\ts_mov_b32 vcc_hi, 0xff00ff00\n\t"
+                             "v_cndmask_b32_dpp %4, v%c8, v%c12, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %5, v%c9, v%c13, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %6, v%c10, v%c14, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_cndmask_b32_dpp %7, v%c11, v%c15, vcc row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+                             "v_mov_b32 v%c8, 0\n\tv_mov_b32 v%c9, 0\n\tv_mov_b32 v%c10, 0\n\tv_mov_b32 v%c11, 0\n\t"
+                             "v_mov_b32 v%c12, 0\n\tv_mov_b32 v%c13, 0\n\tv_mov_b32 v%c14, 0\n\tv_mov_b32 v%c15, 0"
+                             : "=&v"(vA[0]), "=&v"(vA[1]), "=&v"(vA[2]), "=&v"(vA[3]), "=&v"(vB[0]), "=&v"(vB[1]),
+                               "=&v"(vB[2]), "=&v"(vB[3])
+                             : "n"(r0), "n"(r0 + 1), "n"(r0 + 2), "n"(r0 + 3), "n"(r1), "n"(r1 + 1), "n"(r1 + 2), "n"(r1 + 3)
+                             : "vcc");
                 if constexpr (DEQ) {
                     // rows 0-7 use the scale of row r % 8, rows 8-15 that of row 8 + r % 8 of this 16-row tile
                     v4f fA, fB;

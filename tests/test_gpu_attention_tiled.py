@@ -241,7 +241,7 @@ def test_vt_append_matches_row_major_append(mi, dev, orc):
 
 @pytest.mark.parametrize("B,Hq,Hkv,T_cap,N", [(1, 32, 8, 4096, 4096), (1, 16, 4, 1024, 2048), (1, 32, 8, 64, 6144),
                                                (1, 8, 2, 256, 1024), (3, 32, 8, 512, 4096), (16, 32, 8, 256, 4096)])
-def test_vt_attention_with_projection_is_the_two_calls(mi, dev, B, Hq, Hkv, T_cap, N):
+def test_vt_attention_with_projection_is_the_two_calls(mi, dev, orc, B, Hq, Hkv, T_cap, N):
     """mi_gqa_decode_attn_tiled_linear_f32 = mi_gqa_decode_attn_tiled_quant_i8 + mi_w8a8_gemm_dequant_f32, bit for bit,
     also where it divides the work differently (one token with 2048 or 4096 attention values: merge over many
     workgroups, quantizer inside the projection's GEMV); ragged lengths; the merged row comes back on request."""
@@ -273,6 +273,23 @@ def test_vt_attention_with_projection_is_the_two_calls(mi, dev, B, Hq, Hkv, T_ca
     mi.check(lib.mi_gqa_decode_attn_tiled_linear_f32(*args, None, dqw.ptr, dsw.ptr, y2.ptr, *tail))
     a, b, c = dev.download(y0), dev.download(y1), dev.download(y2)
     r0, r1 = dev.download(orot), dev.download(orot2)
+    # ... and against the oracle, stage by stage, whatever the division of the work: the merged rows are the
+    # oracle's attention (rotated basis) on every sequence's prefix; the codes and the scale the one call left in its
+    # workspace are the oracle's quantizer on the device's own merged row; y is the oracle's contraction and
+    # dequantization of those codes
+    al = lambda n: (n + 255) // 256 * 256
+    wsh = dev.download(ws2)
+    codes = wsh[al(B * K * 4):al(B * K * 4) + B * K].view(np.int8).reshape(B, K)
+    scales = wsh[al(B * K * 4) + al(B * K):al(B * K * 4) + al(B * K) + 4 * B].view(np.float32)
+    qw_h, sw_h = dev.download(dqw), dev.download(dsw)
+    for s in range(B):
+        L = int(lens[s])
+        oo = orc.gqa_decode(q[s:s + 1], kq[s:s + 1, :, :L], ks[s:s + 1, :, :L], vq[s:s + 1, :, :L], vs[s:s + 1, :, :L],
+                            out_rotated=True)
+        assert np.max(np.abs(r1[s] - oo[0])) <= 2e-5, s
+        cq, cs = orc.quant_row(r1[s].reshape(-1))
+        assert np.array_equal(codes[s], cq) and scales[s] == cs, s
+    assert np.array_equal(b, orc.dequant(orc.gemm_i8_i32(codes, qw_h), scales, sw_h))
     assert lib.mi_gqa_decode_attn_tiled_linear_f32(*args, None, dqw.ptr, dsw.ptr, y2.ptr, B, Hq, Hkv, D, T_cap, dl.ptr, T_cap,
                                                    N, ws2.ptr, need - 256, None) == mi.ENOSPC
     dev.reset_to(mark)
