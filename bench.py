@@ -208,6 +208,7 @@ def main():
         shapes[(K, N)] = bufs
         del w
     acts = {K: dev.upload(wl.activations(2025, M, K, stream=K)) for K in (4096, 14336)}
+    acts_qkv = dev.upload(wl.activations(2025, M, 4096, stream=1))   # the attention block's input: a matrix of its own
     # every projection writes an output of its own (318 MB in all: more than the memory-side cache holds)
     ybufs = {name: dev.empty((M, N), np.float32) for name, K, N in wl.PROJECTIONS}
     ybuf = ybufs["gate"]
@@ -223,7 +224,7 @@ def main():
 
     # One cfg3 step = the four projections of a decoder layer's prefill.  gate and up read the same activation
     # matrix (as they do in the layer), so its rotate + quantize prologue runs once and both contractions take the
-    # codes; qkv and down each quantize their own input.  Three prologues, then ONE launch for the four
+    # codes; qkv and down each quantize their own input.  ONE launch for the three prologues, then ONE launch for the four
     # contractions (mi_gemm_batch_*: a workgroup per compute unit walks a balanced list of 256 x 192 tiles drawn from
     # all four problems).  The same step with four launches (one per projection, the single-problem kernels) and as
     # four whole linears (a prologue each) is timed beside it.
@@ -240,9 +241,9 @@ def main():
         return ops
 
     def prefill_step():
-        mi.fwht_quant(acts[4096], *qx_qkv, wl.HADAMARD_BLOCK, stream=s)            # qkv's input
-        mi.fwht_quant(acts[4096], *qx_ws[4096], wl.HADAMARD_BLOCK, stream=s)       # gate's and up's input
-        mi.fwht_quant(acts[14336], *qx_ws[14336], wl.HADAMARD_BLOCK, stream=s)     # down's input
+        # the three inputs (qkv's, gate's and up's, down's) are rotated and quantized by ONE launch
+        mi.fwht_quant_batch([(acts_qkv,) + qx_qkv, (acts[4096],) + qx_ws[4096], (acts[14336],) + qx_ws[14336]],
+                            wl.HADAMARD_BLOCK, stream=s)
         batch.run_f32(batch_ops(lambda name, K: qx_qkv if name == "qkv" else qx_ws[K]), stream=s)
 
     def prefill_step_four_launches():
@@ -379,7 +380,7 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "cfg3 prefill: the 4 rotated W8A8 projections of a layer (4096->6144, 4096->14336 x2, "
                                "14336->4096) at M=2048, Hadamard block 128, rotate+quant prologues included; gate and up share "
-                               "one input, which is rotated and quantized once (3 prologues per step), and the four "
+                               "one input, which is rotated and quantized once (3 prologues per step, run as ONE launch: mi_fwht_quant_batch_f32_i8), and the four "
                                "contractions run as ONE launch (mi_gemm_batch_run_f32); every projection writes an output of "
                                "its own (318 MB per step; weights rotate through >256 MB of copies); the K steps are recorded "
                                "into one HIP graph and replayed - the timed method; eager launches from Python are reported "

@@ -161,6 +161,16 @@ MI_API int32_t mi_event_elapsed_ms(mi_event *start, mi_event *stop, float *ms);
  * -127 for the infinite ones. */
 MI_API int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale,
                                     int64_t M, int64_t K, int32_t block, void *stream);
+/* The same for several row sets in ONE launch (n <= 8; the prefill step's prologues: one set per distinct linear
+ * input): every set as mi_fwht_quant_f32_i8 would do it, bit for bit; sets with K < 2048 or no rows make the call
+ * fall back to one launch per set.  Sets must not overlap.  No upstream counterpart. */
+typedef struct mi_quant_rows {
+    const float *x;   /* fp32 [M,K] */
+    int8_t *q;        /* int8 [M,K] */
+    float *scale;     /* fp32 [M]   */
+    int64_t M, K;
+} mi_quant_rows;
+MI_API int32_t mi_fwht_quant_batch_f32_i8(const mi_quant_rows *sets, int32_t n, int32_t block, void *stream);
 /* a1 alone: out fp32 [M,K] = rotated rows (out may alias x). */
 MI_API int32_t mi_fwht_f32(const float *x, float *out, int64_t M, int64_t K,
                            int32_t block, void *stream);

@@ -24,14 +24,13 @@ namespace mi {
 // One workgroup per row; thread t owns chunks t, t + T, ... (C of them).
 // QUANT: write int8 codes + scale; otherwise write the rotated fp32 row.
 template <int BLOCK, int C, bool QUANT>
-__global__ __launch_bounds__(256) void k_fwht_rows(const float *x, int8_t *__restrict__ q,
-                                                    float *__restrict__ scale, float *xrot, int K)
+__device__ __forceinline__ void fwht_row_body(const float *x, int8_t *__restrict__ q, float *__restrict__ scale,
+                                              float *xrot, int K, int64_t row)
 {
     constexpr int LPB = BLOCK / 8;
     const int t = threadIdx.x, T = blockDim.x;
     const int j = t % LPB;
     const int nchunk = K / 8;
-    const int64_t row = blockIdx.x;
     const float *xr = x + row * (int64_t)K;
 
     float v[C][8];
@@ -88,6 +87,46 @@ __global__ __launch_bounds__(256) void k_fwht_rows(const float *x, int8_t *__res
             }
         }
     }
+}
+
+template <int BLOCK, int C, bool QUANT>
+__global__ __launch_bounds__(256) void k_fwht_rows(const float *x, int8_t *__restrict__ q,
+                                                    float *__restrict__ scale, float *xrot, int K)
+{
+    fwht_row_body<BLOCK, C, QUANT>(x, q, scale, xrot, K, (int64_t)blockIdx.x);
+}
+
+// Several row sets in ONE launch (the prefill step's three rotate + quantize prologues): workgroup b finds its set
+// by the sets' cumulative row counts and runs the body of k_fwht_rows on its row, with the chunk count of that set's
+// K.  Same code per row, hence the same codes and scales as separate launches; 256 threads, K >= 2048.
+constexpr int QUANT_BATCH_MAX = 8;
+struct QuantSet {
+    const float *x;
+    int8_t *q;
+    float *scale;
+    int K;
+    int first_row;   // of this set in the grid
+};
+struct QuantBatch {
+    QuantSet s[QUANT_BATCH_MAX];
+    int n;
+};
+template <int BLOCK>
+__global__ __launch_bounds__(256) void k_fwht_rows_batch(const QuantBatch b)
+{
+    int i = 0;
+#pragma unroll
+    for (int k = 1; k < QUANT_BATCH_MAX; ++k)
+        if (k < b.n && (int)blockIdx.x >= b.s[k].first_row) i = k;
+    const QuantSet &S = b.s[i];
+    const int64_t row = (int64_t)blockIdx.x - S.first_row;
+    const int C = (S.K / 8 + 255) / 256;
+    if (C <= 1) fwht_row_body<BLOCK, 1, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if (C <= 2) fwht_row_body<BLOCK, 2, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if (C <= 4) fwht_row_body<BLOCK, 4, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if (C <= 7) fwht_row_body<BLOCK, 7, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if (C <= 8) fwht_row_body<BLOCK, 8, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else fwht_row_body<BLOCK, 16, true>(S.x, S.q, S.scale, nullptr, S.K, row);
 }
 
 // Short rows (K <= 2048): one wave per row, four rows per workgroup; lane l owns chunks l, l + 64, ...
@@ -304,6 +343,41 @@ extern "C" int32_t mi_fwht_quant_f32_i8(const float *x, int8_t *q, float *scale,
     if (M == 0) return MI_OK;
     return block == 128 ? launch_rows<128, true>(x, q, scale, nullptr, M, K, as_stream(stream))
                         : launch_rows<256, true>(x, q, scale, nullptr, M, K, as_stream(stream));
+}
+
+extern "C" int32_t mi_fwht_quant_batch_f32_i8(const mi_quant_rows *sets, int32_t n, int32_t block, void *stream)
+{
+    if (!sets || n < 1 || n > QUANT_BATCH_MAX) return MI_EINVAL;
+    QuantBatch b = {};
+    int64_t rows = 0;
+    bool one_launch = true;
+    for (int i = 0; i < n; ++i) {
+        const mi_quant_rows &s = sets[i];
+        int32_t rc = check_rows(s.x, s.q, s.M, s.K, block);
+        if (rc) return rc;
+        if (!s.scale || !aligned4(s.q) || !aligned4(s.scale)) return MI_EINVAL;
+        // the batched kernel is the row-per-workgroup form at 256 threads; shorter rows (or a set without rows)
+        // take the single launches, whose results are the same
+        if (s.K < 2048 || s.M == 0) one_launch = false;
+        b.s[i].x = s.x;
+        b.s[i].q = s.q;
+        b.s[i].scale = s.scale;
+        b.s[i].K = (int)s.K;
+        b.s[i].first_row = (int)rows;
+        rows += s.M;
+    }
+    if (rows > 0x7fffffffLL) return MI_ERANGE;
+    if (!one_launch) {
+        for (int i = 0; i < n; ++i) {
+            int32_t rc = mi_fwht_quant_f32_i8(sets[i].x, sets[i].q, sets[i].scale, sets[i].M, sets[i].K, block, stream);
+            if (rc) return rc;
+        }
+        return MI_OK;
+    }
+    b.n = n;
+    if (block == 128) hipLaunchKernelGGL(k_fwht_rows_batch<128>, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), b);
+    else hipLaunchKernelGGL(k_fwht_rows_batch<256>, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), b);
+    return launch_status();
 }
 
 extern "C" int32_t mi_kv_append_f32_i8(const float *k_new, const float *v_new, int64_t row_stride, int8_t *kq,

@@ -81,6 +81,7 @@ SIGNATURES = {
     "mi_event_synchronize": (i32, [vp]),
     "mi_event_elapsed_ms": (i32, [vp, vp, f32p]),
     "mi_fwht_quant_f32_i8": (i32, [vp, vp, vp, i64, i64, i32, vp]),
+    "mi_fwht_quant_batch_f32_i8": (i32, [vp, i32, i32, vp]),
     "mi_fwht_f32": (i32, [vp, vp, i64, i64, i32, vp]),
     "mi_w8a8_gemm_i32": (i32, [vp, vp, vp, i64, i64, i64, vp]),
     "mi_w8a8_gemm_dequant_f32": (i32, [vp, vp, vp, vp, vp, i64, i64, i64, vp]),
@@ -331,6 +332,19 @@ class Graph:
 def fwht_quant(x, q, scale, block, stream=None):
     M, K = x.shape
     check(lib.mi_fwht_quant_f32_i8(x.ptr, q.ptr, scale.ptr, M, K, block, stream), "mi_fwht_quant_f32_i8")
+
+
+class QuantRows(C.Structure):
+    """mi_quant_rows of the header: one row set of a batched rotate + quantize call."""
+    _fields_ = [("x", vp), ("q", vp), ("scale", vp), ("M", i64), ("K", i64)]
+
+
+def fwht_quant_batch(sets, block, stream=None):
+    """sets: [(x, q, scale)] DevBufs, x fp32 [M,K]: one launch for all of them."""
+    arr = (QuantRows * len(sets))()
+    for a, (x, q, scale) in zip(arr, sets):
+        a.x, a.q, a.scale, a.M, a.K = x.ptr, q.ptr, scale.ptr, x.shape[0], x.shape[1]
+    check(lib.mi_fwht_quant_batch_f32_i8(arr, len(sets), block, stream), "mi_fwht_quant_batch_f32_i8")
 
 
 def fwht(x, out, block, stream=None):

@@ -42,6 +42,52 @@ def test_codes_and_scales_bit_exact(mi, dev, orc, M, K, block):
     assert np.array_equal(s, so)
     assert np.array_equal(q, qo)
 
+@pytest.mark.parametrize("shapes,block", [
+    ([(33, 4096), (17, 4096), (9, 14336)], 128),            # the prefill step's three inputs, small
+    ([(5, 2048), (3, 32768), (2, 6144), (4, 8192)], 128),   # 1, 16, 3 -> 4 and 4 chunks per thread in one launch
+    ([(7, 4096), (6, 2048)], 256),
+    ([(8, 4096), (5, 768)], 256),                           # a short-row set: the call takes one launch per set
+    ([(40, 2048)] * 8, 128),                                # the most sets a call takes
+])
+def test_batched_quantizer_is_the_single_calls(mi, dev, orc, shapes, block):
+    """mi_fwht_quant_batch_f32_i8: every set's codes and scales are the oracle's (and so those of separate calls);
+    the rows of one set do not leak into the next (poisoned outputs, sets of different K side by side)."""
+    mark = dev.mark()
+    xs = [workload.activations(77 + i, M, K, stream=K + i) for i, (M, K) in enumerate(shapes)]
+    sets = []
+    for x in xs:
+        q, s = dev.empty(x.shape, np.int8), dev.empty(x.shape[0], np.float32)
+        mi.check(mi.lib.mi_fill_u32(q.ptr, 0x7F7F7F7F, q.nbytes // 4, None))
+        sets.append((dev.upload(x), q, s))
+    mi.fwht_quant_batch(sets, block)
+    for x, (_, dq, ds) in zip(xs, sets):
+        qo, so = orc.rotate_quant_rows(x, block)
+        assert np.array_equal(dev.download(ds), so)
+        assert np.array_equal(dev.download(dq), qo)
+    dev.reset_to(mark)
+
+
+def test_batched_quantizer_full_size_and_errors(mi, dev, orc):
+    """The three inputs of the prefill configuration in one launch against three launches, bit for bit; argument
+    errors as the single call reports them."""
+    mark = dev.mark()
+    shapes = [(2048, 4096), (2048, 4096), (2048, 14336)]
+    xs = [dev.upload(workload.activations(5, M, K, stream=i)) for i, (M, K) in enumerate(shapes)]
+    one = [(x, dev.empty(x.shape, np.int8), dev.empty(x.shape[0], np.float32)) for x in xs]
+    three = [(x, dev.empty(x.shape, np.int8), dev.empty(x.shape[0], np.float32)) for x in xs]
+    mi.fwht_quant_batch(one, 128)
+    for x, q, s in three:
+        mi.fwht_quant(x, q, s, 128)
+    for (_, q1, s1), (_, q3, s3) in zip(one, three):
+        assert np.array_equal(dev.download(q1), dev.download(q3)) and np.array_equal(dev.download(s1), dev.download(s3))
+    arr = (mi.QuantRows * 9)()
+    assert mi.lib.mi_fwht_quant_batch_f32_i8(arr, 9, 128, None) == mi.EINVAL      # more than eight sets
+    assert mi.lib.mi_fwht_quant_batch_f32_i8(arr, 0, 128, None) == mi.EINVAL
+    assert mi.lib.mi_fwht_quant_batch_f32_i8(None, 1, 128, None) == mi.EINVAL
+    arr[0].x, arr[0].q, arr[0].scale, arr[0].M, arr[0].K = one[0][0].ptr, one[0][1].ptr, one[0][2].ptr, 4, 4000
+    assert mi.lib.mi_fwht_quant_batch_f32_i8(arr, 1, 128, None) == mi.EINVAL      # K % block
+    dev.reset_to(mark)
+
 
 def test_weight_prep_bit_exact(mi, dev, orc):
     w = workload.weights(7, 1024, 4096)
