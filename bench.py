@@ -400,6 +400,9 @@ def main():
     }
 
     sub = {"prefill_quant_prologue_us": {str(K): round(v * 1e3, 2) for K, v in quant_ms.items()}}
+    prologue_sets = [(acts_qkv,) + qx_qkv, (acts[4096],) + qx_ws[4096], (acts[14336],) + qx_ws[14336]]
+    sub["prefill_quant_prologue_us"]["the_step_s_three_inputs_as_one_launch"] = round(
+        timer.run(lambda: mi.fwht_quant_batch(prologue_sets, wl.HADAMARD_BLOCK, stream=s), 20) * 1e3, 2)
     if not args.skip_sub:
         sub.update(decode_gemv(mi, wl, dev, pool, s, timer, shapes, next_w))
         sub.update(decode_attention(mi, wl, dev, s, timer))

@@ -194,6 +194,46 @@ static void test_quant_linear(const Context &ctx)
     report("quant_linear_vs_oracle", ok && rel <= 1e-3, "rel-L2 " + std::to_string(rel));
 }
 
+// A prefill step through the host layer: two inputs rotated and quantized by one launch (mi_fwht_quant_batch_f32_i8),
+// two contractions by one launch (GemmBatch), both against the oracle's linear on each problem: codes, scales and
+// accumulators equal, outputs equal (the same fp32 operations).
+static void test_gemm_batch(const Context &ctx)
+{
+    const int64_t M = 300, K0 = 2048, N0 = 272, K1 = 4096, N1 = 192;   // ragged in rows and columns: tiles moved inwards
+    DeviceArena<256> arena(ctx, 128 << 20);
+    Rng rng{77};
+    auto gauss = [&](int64_t n, float s) { std::vector<float> v((size_t)n); for (auto &e : v) e = s * rng.normal(); return v; };
+    std::vector<float> x0 = gauss(M * K0, 1.0f), x1 = gauss(M * K1, 1.0f), w0 = gauss(N0 * K0, 0.02f), w1 = gauss(N1 * K1, 0.02f);
+    float *dx0 = upload(arena, x0), *dx1 = upload(arena, x1);
+    QuantLinear<128> l0, l1;   // weight preparation only
+    bool ok = dx0 && dx1 && l0.prepare(arena, upload(arena, w0), N0, K0, 1, nullptr) && l1.prepare(arena, upload(arena, w1), N1, K1, 1, nullptr);
+    int8_t *q0 = arena.alloc<int8_t>(M * K0), *q1 = arena.alloc<int8_t>(M * K1);
+    float *s0 = arena.alloc<float>(M), *s1 = arena.alloc<float>(M), *y0 = arena.alloc<float>(M * N0), *y1 = arena.alloc<float>(M * N1);
+    ok = ok && q0 && q1 && s0 && s1 && y0 && y1;
+    const mi_quant_rows sets[2] = {{dx0, q0, s0, M, K0}, {dx1, q1, s1, M, K1}};
+    ok = ok && mi_fwht_quant_batch_f32_i8(sets, 2, 128, nullptr) == MI_OK;
+    const int64_t mnk[6] = {M, N0, K0, M, N1, K1};
+    GemmBatch batch;
+    ok = ok && batch.prepare(arena, mnk, 2) == MI_OK && (bool)batch;
+    const mi_gemm_problem p[2] = {{q0, s0, l0.qw, l0.sw, y0, M, N0, K0}, {q1, s1, l1.qw, l1.sw, y1, M, N1, K1}};
+    ok = ok && batch.run(p, nullptr) == MI_OK;
+    const mi_gemm_problem bad[2] = {{q0, s0, l0.qw, l0.sw, y0, M, N0, K0}, {q1, s1, l1.qw, l1.sw, y1, M, N1, K1 + 128}};
+    ok = ok && batch.run(bad, nullptr) == MI_EINVAL;   // a shape that is not the batch's
+    bool same = true;
+    for (int i = 0; i < 2; ++i) {
+        const int64_t N = i ? N1 : N0, K = i ? K1 : K0;
+        const std::vector<float> &x = i ? x1 : x0, &w = i ? w1 : w0;
+        std::vector<int8_t> qw_ref(N * K), qx_ref(M * K);
+        std::vector<float> sw_ref(N), sx_ref(M), y_ref(M * N);
+        std::vector<int32_t> acc_ref(M * N);
+        orc_rotate_quant_rows(w.data(), N, K, 128, qw_ref.data(), sw_ref.data(), nullptr);
+        orc_w8a8_linear(x.data(), qw_ref.data(), sw_ref.data(), y_ref.data(), M, N, K, 128, qx_ref.data(), sx_ref.data(), acc_ref.data());
+        same = same && download(i ? q1 : q0, (size_t)(M * K)) == qx_ref && download(i ? s1 : s0, (size_t)M) == sx_ref &&
+               download(i ? y1 : y0, (size_t)(M * N)) == y_ref;
+    }
+    report("gemm_batch_and_quant_batch_vs_oracle", ok && same, same ? "codes, scales and outputs equal" : "differ");
+}
+
 static void test_decode_attention(const Context &ctx)
 {
     const int64_t B = 2, Hq = 8, Hkv = 2, D = 128, T = 200;
@@ -580,6 +620,7 @@ int main()
     test_host_arena(ctx);
     test_stream_pool(ctx);
     test_quant_linear(ctx);
+    test_gemm_batch(ctx);
     test_decode_attention(ctx);
     test_kv_cache(ctx, 40, "kv_cache_append_attend_vs_oracle");
     test_kv_cache(ctx, 64, "kv_cache_tiled_layouts_append_attend_vs_oracle");
