@@ -766,7 +766,7 @@ def list_timeline(mi, wl, dev, s):
     buf = np.zeros(WGS * TILES * 8, np.uint64)
     mi.check(f(buf.ctypes.data, buf.size, 0))
     t = buf.reshape(WGS, TILES, 8).astype(np.int64)
-    valid = t[:, :, 6] == 1
+    valid = (t[:, :, 6] & 1) == 1
     wgs = int(valid.any(axis=1).sum())
     nk = t[:, :, 5][valid]
     loop = (t[:, :, 1] - t[:, :, 0])[valid]
@@ -774,6 +774,8 @@ def list_timeline(mi, wl, dev, s):
     real_us = (t[:, :, 4] - t[:, :, 3])[valid] / 100.0
     wait = (t[:, :, 7] & 0xffffffff)[valid]      # wave 0: ticks in the wait for its own loads in front of the stage's barrier
     bar = (t[:, :, 7] >> 32)[valid]              # ... and in the barrier itself (each includes one clock read)
+    wait1 = (t[:, :, 6] >> 8)[valid]             # ... the wait of a tile's second stage alone: the first that must see
+                                                 # the stores of the tile before acknowledged (loads complete in order)
     first = np.broadcast_to(np.arange(TILES)[None, :] == 0, valid.shape)[valid]
     per_k = {}
     for k in np.unique(nk):
@@ -792,6 +794,8 @@ def list_timeline(mi, wl, dev, s):
            "clock_mhz": round(float(((t[:, :, 2] - t[:, :, 0])[valid] / real_us).mean())),
            "per_tile_depth": per_k, "mfma_per_simd_and_stage": 4 * 6 * 2 * 2,
            "convert_and_store_ticks_per_tile": round(float(fin.mean())),
+           "second_stage_wait_ticks_of_later_tiles": {"mean": round(float(wait1[~first].mean())),
+                                                      "p90": round(float(np.percentile(wait1[~first], 90)))},
            "loop_ticks_all_tiles": int(loop.sum()), "convert_and_store_ticks_all_tiles": int(fin.sum()),
            "first_tile_start_to_last_store_us": round(float(ends.max() - start) / 100.0, 2),
            "workgroup_end_before_the_last_one_us": {"mean": round(float(ends.max() - ends.mean()) / 100.0, 2),

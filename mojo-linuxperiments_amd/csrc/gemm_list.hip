@@ -247,6 +247,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     // free for the stage after that (its loads are issued during the next stage's first half).
 #ifdef MI_GEMM_TIMELINE
     unsigned tl_wait = 0, tl_bar = 0;   // ticks of a tile spent in the wait in front of the barrier / in the barrier
+    unsigned tl_wait1 = 0;              // ... of which in the tile's second stage
 #endif
     auto stage = [&]() {
         const bool ld = ldv;
@@ -309,6 +310,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
             __builtin_amdgcn_s_barrier();
 #ifdef MI_GEMM_TIMELINE
             tl_wait += tl_s1 - tl_s0;
+            if (kt == 1 && !first_tile) tl_wait1 = tl_s1 - tl_s0;   // the first wait that has to see the previous tile's stores acknowledged
             tl_bar += (unsigned)__builtin_amdgcn_s_memtime() - tl_s1;
 #endif
             const unsigned nax0 = add_vs(xo0, xnxt), naw0 = add_vs(wo0, wnxt);
@@ -477,10 +479,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                 o[3] = tl_ra;   // real time (100 MHz) at o[0]
                 o[4] = tl_rc;   // real time at o[2]
                 o[5] = (unsigned long long)nk;
-                o[6] = 1;
+                o[6] = 1ull | ((unsigned long long)tl_wait1 << 8);
                 o[7] = ((unsigned long long)tl_bar << 32) | tl_wait;
             }
-            tl_wait = tl_bar = 0;
+            tl_wait = tl_bar = tl_wait1 = 0;
         }
 #endif
         if (!more) break;
