@@ -225,7 +225,7 @@ def main():
     # One cfg3 step = the four projections of a decoder layer's prefill.  gate and up read the same activation
     # matrix (as they do in the layer), so its rotate + quantize prologue runs once and both contractions take the
     # codes; qkv and down each quantize their own input.  ONE launch for the three prologues, then ONE launch for the four
-    # contractions (mi_gemm_batch_*: a workgroup per compute unit walks a balanced list of 256 x 192 tiles drawn from
+    # contractions (mi_gemm_batch_*: a workgroup per compute unit walks a balanced list of 256 x 256 tiles drawn from
     # all four problems).  The same step with four launches (one per projection, the single-problem kernels) and as
     # four whole linears (a prologue each) is timed beside it.
     qx_ws = {K: (dev.empty((M, K), np.int8), dev.empty(M, np.float32)) for K in (4096, 14336)}
@@ -339,8 +339,8 @@ def main():
             traffic = rec["batched_gemm_bytes_per_launch"]
             traffic_total = traffic["fetch"] + traffic["write"]
     roofline = {
-        "kernel": "k_w8a8_list, v_mfma_i32_16x16x64_i8: ONE launch for the four cfg3 contractions (1,632 tiles of "
-                  "256 x 192 on a balanced work list), dequantization fused",
+        "kernel": "k_w8a8_list, v_mfma_i32_16x16x64_i8: ONE launch for the four cfg3 contractions (1,216 tiles of "
+                  "256 x 256 on a balanced work list), dequantization fused",
         "bound": "mfma", "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": round(gemm_tops / PEAK_INT8_TOPS, 4), "traffic": traffic_total,
         "traffic_unit": "bytes per launch (fetched + written), rocprofv3 PMC, calibrated",

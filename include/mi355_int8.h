@@ -186,11 +186,11 @@ MI_API int32_t mi_w8a8_gemm_i32(const int8_t *qx, const int8_t *qw, int32_t *acc
 MI_API int32_t mi_w8a8_gemm_dequant_f32(const int8_t *qx, const float *sx,
                                         const int8_t *qw, const float *sw, float *y,
                                         int64_t M, int64_t N, int64_t K, void *stream);
-/* a4 for several contractions at once: ONE launch whose workgroups (one per compute unit) walk a list of 256 x 192
+/* a4 for several contractions at once: ONE launch whose workgroups (one per compute unit) walk a list of 256 x 256
  * output tiles drawn from every problem of the batch, so that no problem's tile count has to divide by the number
  * of compute units, and no launch gap or first memory round trip lies between the problems.  No upstream
  * counterpart.  A batch is made once for a list of shapes
- * (mnk int64 [n][3] = M, N, K per problem; n <= 8; M >= 256, N >= 192, N % 16 == 0, K % 128 == 0, K >= 384, 127 * 127 * K < 2^31): the tile lists
+ * (mnk int64 [n][3] = M, N, K per problem; n <= 8; M >= 256, N >= 256, N % 16 == 0, K % 128 == 0, K >= 384, 127 * 127 * K < 2^31): the tile lists
  * are computed on the host and copied (synchronously) into `plan`, device memory of the caller of at least
  * mi_gemm_batch_plan_bytes(mnk, n) bytes that must stay untouched while the batch lives.  A run takes the operands
  * of this call (shapes must equal the batch's) and is an ordinary asynchronous launch: it may be captured into a

@@ -6,29 +6,34 @@
 // previous kernel, the first memory round trip of 256 workgroups asking at once, and an epilogue in which the matrix
 // pipe idles while 196 KB per compute unit are converted and stored.  Its tile shape is also dictated by how the
 // tile count divides by the number of compute units.  Here
-//   - the tiles of all problems form one work list of 256 x 192 tiles, balanced as a whole on the host;
+//   - the tiles of all problems form one work list of 256 x 256 tiles, balanced as a whole on the host;
 //   - the direct-to-LDS loads run two stages ahead of the matrix instructions ACROSS tile boundaries (the stage
 //     buffers rotate for the whole life of the workgroup and never drain between tiles);
-//   - a wave owns 64 x 96 outputs over the WHOLE of K (96 accumulation registers), so no partial sums are exchanged
-//     between waves: when a tile's last stage has been issued the wave converts, scales, stores and clears its 24
-//     accumulators in one straight run of vector instructions, while the loads of the next tile (requested two
-//     stages ago) are already landing.
+//   - a wave owns 64 x 128 outputs over the WHOLE of K (128 accumulation registers), so no partial sums are
+//     exchanged between waves: when a tile's last stage has been issued the wave converts, scales, stores and clears
+//     its 32 accumulators in one straight run of vector instructions, while the loads of the next tile (requested
+//     two stages ago) are already landing.
+//     (The tile is as large as the unit's LDS allows: two activation and three weight stage buffers of 32 KB fill its
+//     160 KB.  Against 256 x 192 tiles it moves a tenth fewer bytes from LDS and a seventh fewer from L2 per matrix
+//     instruction, and the matrix pipe of this part runs against a power limit that every byte moved lowers:
+//     measured 3 to 4 % faster on the four prefill projections, although the coarser tiles balance a little worse.)
 //     (Measured and not kept: a second accumulator set, drained one accumulator per stage under the next tile's
 //     matrix instructions.  Both waves of a SIMD reach the drain at the same point of a stage, so the matrix pipe
 //     idles all the same, and the store queues behind the stage's direct-to-LDS loads on the unit's one memory path:
 //     it cost 1,000 ticks per stage, more than the straight run at the end of the tile.)
 // A tile that would cross the edge of its matrix is moved inwards until it fits: the overlap with its neighbour
 // is computed twice, both times to the same values (exact integers, the same fp32 operations), so every problem
-// needs only M >= 256, N >= 192; no ragged code path exists.
+// needs only M >= 256, N >= 256; no ragged code path exists.
 //
-// Waves: 8 = 4 (rows) x 2 (columns), two per SIMD; wave tile 4 x 6 matrix-instruction tiles.  A 128-byte K stage
-// is two halves of 64 bytes; a half is six groups (one weight fragment against the four activation fragments).
-// LDS layout, swizzle and load shapes are those of gemm_pair.hip.  Per wave and half: 6 weight and 4 activation
+// Waves: 8 = 4 (rows) x 2 (columns), two per SIMD; wave tile 4 x 8 matrix-instruction tiles.  A 128-byte K stage
+// is two halves of 64 bytes; a half is eight groups (one weight fragment against the four activation fragments).
+// LDS layout, swizzle and load shapes are those of gemm_pair.hip.  Per wave and half: 8 weight and 4 activation
 // fragment reads, all of them requested half a stage before they are used (see the stage below), and ONE barrier
 // a stage.
 //
-// Registers: v[160..255] are the accumulators, named by hand; the kernel is limited to v0..v159 for everything the
-// compiler places (see gemm_pair_ops.h): fragments for two K halves and the addresses.
+// Registers: v[128..255] are the accumulators and v[104..127] hold the scales of the wave's rows and columns for
+// the tile in work (LDS has no room for them), all named by hand; the kernel is limited to v0..v103 for everything
+// the compiler places (see gemm_pair_ops.h): fragments for two K halves and the addresses.
 //
 // Memory operations complete in issue order (one counter for loads and stores), and every wait below is written
 // against that order.  Every wave issues an eighth of the loads and stores its own results.
@@ -70,30 +75,23 @@ struct Batch {
 };
 
 struct Cfg {
-    static constexpr int TM = 4, TN = 6;                // matrix-instruction tiles of a wave
-    static constexpr int BM = 256, BN = 192;            // 4 x 2 waves
+    static constexpr int TM = 4, TN = 8;                // matrix-instruction tiles of a wave
+    static constexpr int BM = 256, BN = 256;            // 4 x 2 waves
     static constexpr int NBX = BM / 8, NBW = BN / 8;    // 1 KB blocks (8 rows x 128 B) per stage
     static constexpr int XSTAGE = NBX * 1024, WSTAGE = NBW * 1024, XAREA = 2 * XSTAGE;
-    static constexpr int STAGES = XAREA + 3 * WSTAGE;   // two activation buffers, three weight buffers
-    static constexpr int SCALES = (BM + BN) * 4;        // of one tile: BM row scales, then BN column scales
-    static constexpr int SCALES_AT = STAGES;
-    static constexpr int LDS = SCALES_AT + 2 * SCALES;  // two scale areas, by tile parity
+    static constexpr int LDS = XAREA + 3 * WSTAGE;      // two activation buffers, three weight buffers
     static constexpr int LX = NBX / 8, LW = NBW / 8;    // loads of a wave per stage
     static constexpr int NACC = TM * TN;                // accumulators of a set
+    // a lane's scales for its wave's tile: of rows r % 8 and 8 + r % 8 of each of the TM row tiles (v[SCL0 + 2i],
+    // v[SCL0 + 2i + 1]), and four column scales for each pair of column tiles (v[SCL0 + 2 TM + 4 jp ..])
+    static constexpr int NSCL = 2 * TM + 4 * (TN / 2), SCL0 = vacc::ACC0 - NSCL;
+    static constexpr int LSCL = 2 * TM + TN / 2;        // loads that bring them, per wave and tile
     static constexpr int MIN_STAGES = 3;                // the loads run up to three stages ahead, into the next tile at most
-    static_assert(LX == 4 && LW == 3, "the stage's load slots are written out for four and three parts");
+    static_assert(LX <= TM && LW <= TN && TN >= TM + 2, "where the stage issues its loads and what its waits count");
     static_assert(vacc::ACC0 + 4 * NACC <= 256, "the accumulators lie above the compiler's registers");
     static_assert(LDS <= 160 * 1024, "LDS of a compute unit");
 };
 
-// direct-to-LDS load of 4 bytes per lane: global address = sbase + voff, LDS address = ldsaddr + 4 * lane
-__device__ __forceinline__ void dma4(const float *sbase, unsigned voff, unsigned ldsaddr)
-{
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 4\n\tglobal_load_lds_dword %0, %1"
-                 :
-                 : "v"(voff), "s"(sbase), "s"(ldsaddr)
-                 : "memory", "m0");
-}
 #ifdef MI_GEMM_TIMELINE
 // The measurement build keeps a few more scalars alive and may spill some: a base the compiler brings back with a
 // vector instruction needs five wait states before a memory instruction reads it (see the build check of the
@@ -135,31 +133,51 @@ __device__ __forceinline__ unsigned add_vs(unsigned a, unsigned s)
     asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(s), "v"(a));
     return r;
 }
-__device__ __forceinline__ void lds_read32(float &dst, unsigned addr)
+// the scales of rows (r % 8) and (8 + r % 8) of a 16-row tile into v[R], v[R + 1]; four column scales into v[R .. R + 3]
+template <int R, int OFF>
+__device__ __forceinline__ void scale_load_pair(unsigned voff, const float *sbase)
 {
-    asm volatile("ds_read_b32 %0, %1" : "=v"(dst) : "v"(addr));
+#ifdef MI_GEMM_TIMELINE
+    asm volatile("s_nop 4" ::: "memory");   // (a scalar base brought back from a spill: see dma16 above)
+#endif
+    asm volatile("global_load_dword v%c2, %0, %1 offset:%c4\n\tglobal_load_dword v%c3, %0, %1 offset:%c5"
+                 :
+                 : "v"(voff), "s"(sbase), "n"(R), "n"(R + 1), "n"(OFF), "n"(OFF + 32)
+                 : "memory");
 }
-__device__ __forceinline__ void lds_read128f(v4f &dst, unsigned addr)
+template <int R, int OFF>
+__device__ __forceinline__ void scale_load4(unsigned voff, const float *sbase)
 {
-    asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(addr));
+#ifdef MI_GEMM_TIMELINE
+    asm volatile("s_nop 4" ::: "memory");
+#endif
+    asm volatile("global_load_dwordx4 v[%c2:%c3], %0, %1 offset:%c4" : : "v"(voff), "s"(sbase), "n"(R), "n"(R + 3), "n"(OFF) : "memory");
+}
+template <int R>
+__device__ __forceinline__ float scale_reg()
+{
+    float v;
+    asm volatile("v_mov_b32 %0, v%c1" : "=v"(v) : "n"(R));
+    return v;
 }
 
 template <bool DEQ>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2))) void k_w8a8_list(
+__global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(Cfg::SCL0 / 2))) void k_w8a8_list(
     const Batch bt, const v4i *__restrict__ lists, int per_wg)
 {
     using C = Cfg;
-    constexpr int TM = C::TM, TN = C::TN, BM = C::BM;
+    constexpr int TM = C::TM, TN = C::TN;
     constexpr int XSTAGE = C::XSTAGE, WSTAGE = C::WSTAGE, XAREA = C::XAREA;
     constexpr int NACC = C::NACC;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    // v[160 .. 255] are this kernel's accumulators, named by hand: the attribute above keeps everything the compiler
-    // places below v160, and this clobber makes the wave's register count cover them
-    asm volatile("" ::: "v160", "v255");
+    // v[128 .. 255] are this kernel's accumulators and v[104 .. 127] its scales, named by hand: the attribute above
+    // keeps everything the compiler places below v104, and this clobber makes the wave's register count cover them
+    asm volatile("" ::: "v104", "v255");
+    static_assert(C::SCL0 == 104 && vacc::ACC0 == 128, "the clobber above names the first register by hand");
 
     const int tid = threadIdx.x, lane0 = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;   // wave tile: rows wm*64.., columns wn*96..
+    const int wm = wave >> 1, wn = wave & 1;   // wave tile: rows wm*64.., columns wn*128..
     const unsigned lds_base = (unsigned)(uintptr_t)(lptr_t)smem;
     const unsigned lds_x = lds_base + wave * 1024, lds_w = lds_base + XAREA + wave * 1024;
 
@@ -173,11 +191,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
         e_n0 = e[2];
     }
     if (e_p < 0) return;
+    // the scales of the tile's rows and columns (fetched where the tile is entered: a scalar load inside the stage
+    // would have to wait for every LDS read in flight with it)
+    const float *e_sx = bt.p[e_p].sx + e_m0, *e_sw = bt.p[e_p].sw + e_n0;
     static_for<NACC>([&](auto I) { vacc::acc_zero4<4 * decltype(I)::value>(); });
 
     // ---- load side.  The load cursor (a tile and a stage of it) runs two stages ahead of the matrix instructions.
     // lane l = 8*rho + c fetches the 16-byte chunk c ^ sigma of row rho of a block; wave w fills blocks w + 8q of
-    // a stage (four of the activations, three of the weights): every wave issues the same share of the loads, and
+    // a stage (four of the activations, four of the weights): every wave issues the same share of the loads, and
     // one lane offset serves every block of a tile: base of the tile (two scalars) + this lane's offset + a scalar
     // that moves with q and with the stage (one scalar and one vector addition a load; 64-bit scalar address
     // arithmetic for every load, on four waves only, made those four waves the last at every barrier by 500 ticks)
@@ -230,15 +251,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     // ---- the tile being computed
     int kt = 0, nk = 0;
     bool first_tile = true;   // no stores of a tile before this one are in flight
-    unsigned cur_scales = C::SCALES_AT;   // two scale areas, by tile parity: the next tile's scales are requested in
-                                          // its first stage, when a slower wave may still be reading this tile's
 
     // one stage.  There is ONE copy of this code and one loop around it: a fragment register is written by an LDS
     // read the compiler cannot follow (its data arrives later), so no value of xa / xc / w may ever have to be moved
     // where two paths of the control flow meet.  The last stage of a workgroup therefore also requests "next"
     // fragments (from a buffer that holds nothing new; they are never used).
     //
-    // Fragments are requested half a stage ahead: while the six groups of a K half run, the four activation
+    // Fragments are requested half a stage ahead: while the eight groups of a K half run, the four activation
     // fragments of the next half arrive in the other activation set (xa: first halves, xc: second halves) and weight
     // fragment k of the next half is requested into w[k] right behind group k, the last reader of the old w[k].
     // One barrier a stage, behind the first group of the second half: by then every read of this stage's buffers has
@@ -249,6 +268,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     unsigned tl_wait = 0, tl_bar = 0;   // ticks of a tile spent in the wait in front of the barrier / in the barrier
     unsigned tl_wait1 = 0;              // ... of which in the tile's second stage
 #endif
+    // The scales of the tile in work, requested in its first stage: 2 TM single row scales and TN / 2 groups of four
+    // column scales per lane, into v[SCL0 ..].  They are read when the tile's last stage has been issued: a tile has
+    // at least three stages, and the wait in front of the second stage's barrier already covers these loads.
+    auto load_scales = [&]() {
+        const float *bx = e_sx, *bw = e_sw;
+        const int l = opaque(lane0);
+        const int r = l & 15, g_ = l >> 4;
+        const unsigned vx = (unsigned)((wm * 64 + (r & 7)) * 4);
+        const unsigned vw = (unsigned)((wn * (16 * TN) + (r < 8 ? 0 : 16) + 4 * g_) * 4);
+        static_for<TM>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            scale_load_pair<C::SCL0 + 2 * i, 64 * i>(vx, bx);
+        });
+        static_for<TN / 2>([&](auto JP) {
+            constexpr int jp = decltype(JP)::value;
+            scale_load4<C::SCL0 + 2 * TM + 4 * jp, 128 * jp>(vw, bw);
+        });
+    };
     auto stage = [&]() {
         const bool ld = ldv;
         using I0 = std::integral_constant<int, 0>;
@@ -256,28 +293,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
         using I2 = std::integral_constant<int, 2>;
         using I3 = std::integral_constant<int, 3>;
         // ---- K half 0 (fragments xa, w).  In flight, oldest first, from the stage before:
-        //      W0 | x0 W1 | x1 W2 | x2 W3 | x3 W4 | W5
+        //      W0 | x0 W1 | x1 W2 | x2 W3 | x3 W4 | W5 | W6 | W7
         {
             const unsigned ax1 = add_vs(xo1, xcur), aw1 = add_vs(wo1, wcur);
             static_for<TN>([&](auto J) {
                 constexpr int j = decltype(J)::value;
                 if constexpr (j < TM) ds_read128<j * 2048>(xc[j], ax1);
-                if constexpr (j < 3) {
+                if constexpr (j < C::LW) {
                     if (ld) issue_w(J, wnn);
                 }
-                if constexpr (j == 0) wait_lgkm<3>();        // x0..x3 and W0..W3 are in; W4, W5 and the read above may not be
-                if constexpr (j >= 4) wait_lgkm<9>();        // W4 (W5) is in: 8 reads of this half and W5 (W4') are younger
-                if constexpr (j == 4) {
-                    if (kt == 0) {   // this tile's scales, for the end of the tile
-                        if constexpr (DEQ) {
-                            // waves 0..3: row scales 64 w ..; waves 4..6: column scales 64 (w - 4) ..; wave 7 has
-                            // none left and fetches wave 3's again (every wave counts the same memory operations)
-                            const Problem &P = bt.p[e_p];
-                            const int part = wave < 7 ? wave : 3;
-                            const float *s0 = part < 4 ? P.sx + e_m0 + part * 64 : P.sw + e_n0 + (part - 4) * 64;
-                            const unsigned lo4 = (unsigned)opaque(lane0) * 4u;
-                            dma4(s0, lo4, lds_base + cur_scales + (part < 4 ? part * 256 : BM * 4 + (part - 4) * 256));
-                        }
+                // x0..x3 and W0..W3 are in; W4..W7 and the read above may not be
+                if constexpr (j == 0) wait_lgkm<TN - TM + 1>();
+                // Wj is in: the 2 TM reads of this half's first TM groups and the TN - TM - 1 weight fragments
+                // requested last (of this half behind it, of the next half before it) are younger
+                if constexpr (j >= TM) wait_lgkm<TN + TM - 1>();
+                if constexpr (j == C::LW) {
+                    if (kt == 0) {   // this tile's scales, for the end of the tile, into their registers
+                        if constexpr (DEQ) load_scales();
                     }
                 }
                 static_for<TM>([&](auto I) {
@@ -286,19 +318,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
                 ds_read128<j * 2048>(w[j], aw1);   // w[j] has been read for the last time
             });
         }
-        // ---- K half 1 (fragments xc, w).  In flight: x0 W0 | x1 W1 | x2 W2 | x3 W3 | W4 | W5
+        // ---- K half 1 (fragments xc, w).  In flight: x0 W0 | x1 W1 | x2 W2 | x3 W3 | W4 | W5 | W6 | W7
         {
-            wait_lgkm<3>();   // x0..x3 and W0..W2 are in
+            wait_lgkm<TN - TM + 1>();   // x0..x3 and W0..W2 are in
             static_for<TM>([&](auto I) { vacc::mfma_acc<4 * decltype(I)::value>(w[0], xc[decltype(I)::value]); });
             // The barrier.  Every read of this stage's buffers has landed in this wave, and a loading wave's share of
             // the next stage as well.  Memory operations complete in order; issued since the last load of the next
             // stage (its fourth activation part, in the stage before): in a tile's first stage the NACC stores of
-            // the tile before it; this stage's three weight parts; in a tile's first stage its scales.
+            // the tile before it; this stage's four weight parts; in a tile's first stage the loads of its scales.
 #ifdef MI_GEMM_TIMELINE
             const unsigned tl_s0 = (unsigned)__builtin_amdgcn_s_memtime();
 #endif
             {
-                constexpr int SC = DEQ ? 1 : 0, LW = C::LW;
+                constexpr int SC = DEQ ? C::LSCL : 0, LW = C::LW;
                 if (!ldv) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 else if (kt == 0 && !first_tile) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LW + SC + NACC) : "memory");
                 else if (kt == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LW + SC) : "memory");
@@ -332,24 +364,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
             const unsigned u = wcur; wcur = wnxt; wnxt = wnn; wnn = u;
         }
     };
-    static_assert(C::LW + 1 + NACC + C::LX <= 63, "the memory counter has six bits");
+    static_assert(C::LW + C::LSCL + NACC + C::LX <= 63, "the memory counter has six bits");
 
     // The tile's accumulators leave: converted, scaled by the row and the column scale, stored and cleared for the
     // next tile; accumulator (j, i) is named at compile time.  Two neighbouring column tiles are paired and swap
     // halves between lanes r and r ^ 8, so that a store instruction writes 8 rows x 128 B: whole cache lines
     // (stores of 16 rows x 64 B, half lines, cost three times as much here and slowed the next tile's loads).  The first
-    // fragments of the next tile are in flight the whole time (6 LDS reads that the waits below count).
-    auto finish_tile = [&](const void *out, int N, int m0, int n0, unsigned scales_at) {
+    // fragments of the next tile are in flight the whole time.
+    auto finish_tile = [&](const void *out, int N, int m0, int n0) {
         const int l = opaque(lane0);
         const int r = l & 15, g_ = l >> 4;
-        const unsigned asx = lds_base + scales_at + (unsigned)((wm * 64 + (r & 7)) * 4);
-        const unsigned asw = lds_base + scales_at + BM * 4 + (unsigned)((wn * 96 + 4 * g_) * 4);
         float sxA[TM], sxB[TM];   // row r % 8 and row 8 + r % 8 of each 16-row tile
         v4f sw4 = {1.0f, 1.0f, 1.0f, 1.0f};
         if constexpr (DEQ) {
             static_for<TM>([&](auto I) {
-                lds_read32(sxA[decltype(I)::value], asx + 64 * decltype(I)::value);
-                lds_read32(sxB[decltype(I)::value], asx + 64 * decltype(I)::value + 32);
+                sxA[decltype(I)::value] = scale_reg<C::SCL0 + 2 * decltype(I)::value>();
+                sxB[decltype(I)::value] = scale_reg<C::SCL0 + 2 * decltype(I)::value + 1>();
             });
         }
         const char *const base = static_cast<const char *>(out) + ((int64_t)m0 * N + n0) * 4;
@@ -358,16 +388,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
         const bool lo = r < 8;
         // this lane's place in a store of 8 rows x 128 B: row r % 8, and the 16 bytes 4g of column tile j (lanes
         // r < 8) or of column tile j + 1 (lanes r >= 8)
-        unsigned vo = (unsigned)(((wm * 64 + (r & 7)) * N + wn * 96 + (lo ? 0 : 16) + 4 * g_) * 4);
-        const unsigned asw2 = asw + (lo ? 0u : 64u);
+        unsigned vo = (unsigned)(((wm * 64 + (r & 7)) * N + wn * (16 * TN) + (lo ? 0 : 16) + 4 * g_) * 4);
         static_for<TN / 2>([&](auto JP) {
             constexpr int j = 2 * decltype(JP)::value;
             if constexpr (DEQ) {
-                lds_read128f(sw4, asw2 + 64 * j);
-                wait_lgkm<0>();
+                sw4[0] = scale_reg<C::SCL0 + 2 * TM + 2 * j>();
+                sw4[1] = scale_reg<C::SCL0 + 2 * TM + 2 * j + 1>();
+                sw4[2] = scale_reg<C::SCL0 + 2 * TM + 2 * j + 2>();
+                sw4[3] = scale_reg<C::SCL0 + 2 * TM + 2 * j + 3>();
             }
-            // the matrix instructions of the stage's last two groups wrote column tiles 4 and 5 a moment ago
-            if constexpr (j == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+            // the matrix instructions of the stage's last two groups wrote the last two column tiles a moment ago
+            if constexpr (j == TN - 2) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             static_for<TM>([&](auto I) {
                 constexpr int i = decltype(I)::value;
                 constexpr int r0 = vacc::ACC0 + 4 * (j * TM + i), r1 = vacc::ACC0 + 4 * ((j + 1) * TM + i);
@@ -422,12 +453,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     cursor_to((v4i){e_p, e_m0, e_n0, 0});
     nk = bt.p[e_p].K >> 7;
     {
-        static_for<4>([&](auto I) { issue_x(I, 0u); });
-        static_for<3>([&](auto I) { issue_w(I, 0u); });
+        static_for<C::LX>([&](auto I) { issue_x(I, 0u); });
+        static_for<C::LW>([&](auto I) { issue_w(I, 0u); });
         lkt = 1;
-        static_for<4>([&](auto I) { issue_x(I, (unsigned)XSTAGE); });
-        static_for<3>([&](auto I) { issue_w(I, (unsigned)WSTAGE); });
-        wait_vm<7>();   // stage 0 has landed
+        static_for<C::LX>([&](auto I) { issue_x(I, (unsigned)XSTAGE); });
+        static_for<C::LW>([&](auto I) { issue_w(I, (unsigned)WSTAGE); });
+        wait_vm<C::LX + C::LW>();   // stage 0 has landed
     }
     lkt = 2;
     __syncthreads();
@@ -440,7 +471,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
     });
 
     for (int it = 0;; ++it) {
-        cur_scales = (unsigned)(C::SCALES_AT + (it & 1) * C::SCALES);
         // (the list is read again where the next entry is needed: it is not worth four scalar registers for a tile)
         const bool more = sload4(my + it + 1)[0] >= 0;
         bool in_cur = true;   // the cursor stands in this tile (it entered it two stages ago)
@@ -461,12 +491,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
 #endif
         {
             const Problem &P = bt.p[e_p];
-            if (!more) {
-                // nothing follows: the scales must be visible whatever the tile's length, and no load is in flight
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-            }
-            finish_tile(P.out, P.N, e_m0, e_n0, cur_scales);
+            finish_tile(P.out, P.N, e_m0, e_n0);
         }
 #ifdef MI_GEMM_TIMELINE
         {
@@ -492,6 +517,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(vacc::ACC0 / 2)
         e_m0 = e[1];
         e_n0 = e[2];
         nk = bt.p[e_p].K >> 7;
+        e_sx = bt.p[e_p].sx + e_m0;
+        e_sw = bt.p[e_p].sw + e_n0;
     }
 }
 

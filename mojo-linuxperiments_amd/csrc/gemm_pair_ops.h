@@ -69,15 +69,16 @@ __device__ __forceinline__ void acc_zero()
 
 // ---- the same with the accumulators in ORDINARY registers v[ACC0 ..] that the compiler cannot allocate.
 // The unified register file of this part lets a matrix instruction add into ordinary registers as well as into
-// accumulation registers.  A kernel that carries __attribute__((amdgpu_num_vgpr(ACC0 / 2))) and uses no
-// accumulation register is limited to v0 .. v(ACC0-1) for everything the compiler places (a spill goes to scratch
+// accumulation registers.  A kernel that carries __attribute__((amdgpu_num_vgpr(L / 2))), L <= ACC0, and uses no
+// accumulation register is limited to v0 .. v(L-1) for everything the compiler places (a spill goes to scratch
 // memory, which the build checks for), while v[ACC0 .. 255] are named by hand in the asm below and claimed for the
-// wave by a clobber of v255 (the register count of the kernel's descriptor).  ACC0 = 160 leaves the compiler 160
-// registers (fragments two K halves deep) and 96 accumulators.  Unlike accumulation registers, which
+// wave by a clobber of v255 (the register count of the kernel's descriptor).  ACC0 = 128 leaves 128 accumulators (a wave
+// tile of 4 x 8 matrix-instruction tiles) and 128 registers below them (fragments two K halves deep; the kernel may
+// name some of the highest of these by hand as well and set its limit lower).  Unlike accumulation registers, which
 // the register allocator may use to split a live range whenever ordinary registers run short, nothing but this
 // code can write them.
 namespace vacc {
-constexpr int ACC0 = 160;
+constexpr int ACC0 = 128;
 template <int LO>
 __device__ __forceinline__ void mfma_acc(const v4i &a, const v4i &b)
 {

@@ -199,7 +199,7 @@ static void test_quant_linear(const Context &ctx)
 // accumulators equal, outputs equal (the same fp32 operations).
 static void test_gemm_batch(const Context &ctx)
 {
-    const int64_t M = 300, K0 = 2048, N0 = 272, K1 = 4096, N1 = 192;   // ragged in rows and columns: tiles moved inwards
+    const int64_t M = 300, K0 = 2048, N0 = 272, K1 = 4096, N1 = 256;   // ragged in rows and columns: tiles moved inwards
     DeviceArena<256> arena(ctx, 128 << 20);
     Rng rng{77};
     auto gauss = [&](int64_t n, float s) { std::vector<float> v((size_t)n); for (auto &e : v) e = s * rng.normal(); return v; };

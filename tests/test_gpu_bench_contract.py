@@ -64,8 +64,8 @@ def test_probe_and_timeline_modes_print_one_json_line_each():
         assert 0.9 * parts <= t["whole_kernel"] <= 1.1 * (parts + 3000)
         assert tl[name]["workgroups"] > 0 and tl[name]["stages"] in (32, 112) and tl[name]["kernel_us_event"] > 0
     b = tl["batch"]
-    # every tile of the four projections left its three clock reads: 8 row tiles x (32 + 75 + 75 + 22) column tiles
-    assert b["tiles"] == 8 * (32 + 75 + 75 + 22) and 0 < b["workgroups"] <= 512
+    # every tile of the four projections left its three clock reads: 8 row tiles x (24 + 56 + 56 + 16) column tiles
+    assert b["tiles"] == 8 * (24 + 56 + 56 + 16) and 0 < b["workgroups"] <= 512
     assert set(b["per_tile_depth"]) == {"stages_32", "stages_112"}
     assert sum(v["tiles"] for v in b["per_tile_depth"].values()) == b["tiles"]
     assert b["loop_ticks_all_tiles"] > 0 and b["convert_and_store_ticks_all_tiles"] > 0

@@ -1,5 +1,5 @@
 """GPU parity: several W8A8 contractions in one launch (mi_gemm_batch_*), the kernel whose workgroups walk a list of
-256 x 192 tiles.  Gates: int32 accumulators bit-exact against the oracle; the dequantized form equal to the
+256 x 256 tiles.  Gates: int32 accumulators bit-exact against the oracle; the dequantized form equal to the
 oracle's fp32 operations; both equal, bit for bit, to the single-problem entry points."""
 import numpy as np
 import pytest
@@ -25,14 +25,14 @@ def make_ops(dev, shapes, seed, dtype):
     return ops, host
 
 
-# K of 3 to 7 stages (short tiles: the tile before them is not drained by the time they end) and of 24, 25 and 32
-# (the previous tile's 24 accumulators leave one per stage); shapes that are no multiple of the tile exercise the
-# tiles that are moved inwards (rows: 300 = 256 + 44, columns: 272 = 192 + 80, 14336 = 74 * 192 + 128); several tiles
-# per workgroup exercise the load stream across tile boundaries, both accumulator sets and the clearing of a
-# drained set; mixed K in one batch exercises a cursor that changes its stride between tiles.
+# K of 3 to 7 stages (short tiles: the stores of the tile before them are still in flight when they end) and of 24, 25
+# and 32; shapes that are no multiple of the tile exercise the tiles that are moved inwards (rows: 300 = 256 + 44,
+# columns: 272 = 256 + 16, 1168 = 4 * 256 + 144); several tiles per workgroup exercise the load
+# stream across tile boundaries, the scales that change registers' contents between tiles and the clearing of the
+# accumulators; mixed K in one batch exercises a cursor that changes its stride between tiles.
 @pytest.mark.parametrize("shapes", [
-    [(256, 192, 384)],
-    [(256, 192, 512)],
+    [(256, 256, 384)],
+    [(256, 256, 512)],
     [(300, 272, 640)],
     [(2048, 6144, 384)],
     [(2048, 6144, 896)],
@@ -40,9 +40,9 @@ def make_ops(dev, shapes, seed, dtype):
     [(4096, 4096, 512)],
     [(2048, 4608, 3072)],
     [(2048, 6144, 3200)],
-    [(512, 384, 896), (256, 208, 384)],
+    [(512, 384, 896), (256, 272, 384)],
     [(2048, 6144, 384), (2048, 4096, 4096), (264, 14336, 512)],
-    [(1024, 1152, 768)] * 8,
+    [(1024, 1168, 768)] * 8,
 ])
 def test_batch_accumulators_bit_exact(mi, dev, orc, shapes):
     mark = dev.mark()
@@ -59,7 +59,7 @@ def test_batch_accumulators_bit_exact(mi, dev, orc, shapes):
 
 
 @pytest.mark.parametrize("shapes", [
-    [(256, 192, 384)],
+    [(256, 256, 384)],
     [(300, 272, 512)],
     [(2048, 6144, 384), (520, 4096, 1024)],
     [(2048, 6144, 4096)],
@@ -113,17 +113,17 @@ def test_batch_rejects_what_it_cannot_run(mi, dev):
         arr = (i64 * (3 * len(shapes)))(*[v for s in shapes for v in s])
         return mi.lib.mi_gemm_batch_plan_bytes(arr, len(shapes))
 
-    assert plan_bytes([(255, 192, 384)]) == mi.EINVAL      # fewer rows than a tile
-    assert plan_bytes([(256, 176, 384)]) == mi.EINVAL      # fewer columns than a tile
-    assert plan_bytes([(256, 200, 384)]) == mi.EINVAL      # N % 16
-    assert plan_bytes([(256, 192, 448)]) == mi.EINVAL      # K % 128
-    assert plan_bytes([(256, 192, 256)]) == mi.EINVAL      # fewer than three K stages
-    assert plan_bytes([(256, 192, 384)] * 9) == mi.EINVAL  # more than eight problems
-    assert plan_bytes([(256, 192, 1 << 18)]) == mi.ERANGE  # the int32 accumulator could overflow
-    assert plan_bytes([(256, 192, 384)]) > 0
+    assert plan_bytes([(255, 256, 384)]) == mi.EINVAL      # fewer rows than a tile
+    assert plan_bytes([(256, 240, 384)]) == mi.EINVAL      # fewer columns than a tile
+    assert plan_bytes([(256, 264, 384)]) == mi.EINVAL      # N % 16
+    assert plan_bytes([(256, 256, 448)]) == mi.EINVAL      # K % 128
+    assert plan_bytes([(256, 256, 256)]) == mi.EINVAL      # fewer than three K stages
+    assert plan_bytes([(256, 256, 384)] * 9) == mi.EINVAL  # more than eight problems
+    assert plan_bytes([(256, 256, 1 << 18)]) == mi.ERANGE  # the int32 accumulator could overflow
+    assert plan_bytes([(256, 256, 384)]) > 0
     mark = dev.mark()
-    batch = mi.GemmBatch(dev, [(256, 192, 384)])
-    qx, qw, out = dev.empty((256, 512), np.int8), dev.empty((192, 512), np.int8), dev.empty((256, 192), np.int32)
+    batch = mi.GemmBatch(dev, [(256, 256, 384)])
+    qx, qw, out = dev.empty((256, 512), np.int8), dev.empty((256, 512), np.int8), dev.empty((256, 256), np.int32)
     with pytest.raises(mi.MiError) as e:   # K differs from the batch's
         batch.run_i32([(qx, None, qw, None, out)])
     assert e.value.status == mi.EINVAL
