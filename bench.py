@@ -792,7 +792,7 @@ def list_timeline(mi, wl, dev, s):
     ends = np.array([t[w, np.where(valid[w])[0][-1], 4] for w in range(WGS) if valid[w].any()])
     res = {"kernel_us_event": round(us, 2), "workgroups": wgs, "tiles": int(valid.sum()),
            "clock_mhz": round(float(((t[:, :, 2] - t[:, :, 0])[valid] / real_us).mean())),
-           "per_tile_depth": per_k, "mfma_per_simd_and_stage": 4 * 6 * 2 * 2,
+           "per_tile_depth": per_k, "mfma_per_simd_and_stage": 4 * 8 * 2 * 2,
            "convert_and_store_ticks_per_tile": round(float(fin.mean())),
            "second_stage_wait_ticks_of_later_tiles": {"mean": round(float(wait1[~first].mean())),
                                                       "p90": round(float(np.percentile(wait1[~first], 90)))},
