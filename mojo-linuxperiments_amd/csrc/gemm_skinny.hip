@@ -517,21 +517,23 @@ __device__ __forceinline__ void wait_vm()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// NG groups of 16 weight rows per workgroup, MT groups of 16 tokens, ring of D stages per wave.
-// A stage = one 128-byte K step of (16*NG weight rows + 16*MT token rows) as 1 KB blocks of 8 rows.
-template <int NG, int MT, int D, bool DEQ>
-__global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
-                                                     const float *__restrict__ sx, const float *__restrict__ sw,
-                                                     int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
-                                                     int N, int K)
+// NB blocks of 8 weight rows per workgroup, MT groups of 16 tokens, ring of D stages per wave.
+// A stage = one 128-byte K step of (8*NB weight rows + 16*MT token rows) as 1 KB blocks of 8 rows.  The matrix
+// instruction takes 16 weight rows: with NB odd the last group's second half reads whatever block follows (the first
+// token block) and its 8 result rows are never stored.  8-row granularity lets the launcher give every compute
+// unit the same number of rows (N / 8 blocks over the units: 3 a unit for N = 6144, 7 for N = 14336).
+template <int NB, int MT, int D, bool DEQ>
+__device__ __forceinline__ void ring_body(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                          const float *__restrict__ sx, const float *__restrict__ sw,
+                                          int32_t *__restrict__ acc_out, float *__restrict__ y, int M, int N, int K,
+                                          const int n0, char *smem)
 {
-    constexpr int BLK = 2 * (NG + MT);       // 1 KB blocks (= load instructions) per stage
+    constexpr int NG = (NB + 1) / 2;         // 16-row groups the matrix instructions work on
+    constexpr int BLK = NB + 2 * MT;         // 1 KB blocks (= load instructions) per stage
     constexpr int STAGE = BLK * 1024;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = blockDim.x >> 6;
     char *ring = smem + wave * (D * STAGE);
-    const int n0 = blockIdx.x * 16 * NG;
 
     // load side: lane l = 8*rho + c fetches chunk c ^ sigma of row rho of the block
     const int8_t *src[BLK];
@@ -539,14 +541,15 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
         const int rho = lane >> 3, c = lane & 7;
 #pragma unroll
         for (int b = 0; b < BLK; ++b) {
-            const int sigma = ((b & 1) << 2) | (rho >> 1);
+            // (the swizzle goes by the block's place in its own 16-row group: weight blocks and token blocks count apart)
+            const int sigma = ((((b < NB) ? b : b - NB) & 1) << 2) | (rho >> 1);
             const int8_t *base;
-            if (b < 2 * NG) {
+            if (b < NB) {
                 int rowi = n0 + b * 8 + rho;
                 if (rowi > N - 1) rowi = N - 1;
                 base = qw + (int64_t)rowi * K;
             } else {
-                int tok = (b - 2 * NG) * 8 + rho;
+                int tok = (b - NB) * 8 + rho;
                 if (tok > M - 1) tok = M - 1;   // tokens past M repeat the last one and are never stored
                 base = qx + (int64_t)tok * K;
             }
@@ -592,7 +595,7 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
 #pragma unroll
                 for (int a = 0; a < NG; ++a) wf[a][kk] = *reinterpret_cast<const v4i *>(sb + a * 2048 + roff[kk]);
 #pragma unroll
-                for (int b = 0; b < MT; ++b) xf[b][kk] = *reinterpret_cast<const v4i *>(sb + (NG + b) * 2048 + roff[kk]);
+                for (int b = 0; b < MT; ++b) xf[b][kk] = *reinterpret_cast<const v4i *>(sb + NB * 1024 + b * 2048 + roff[kk]);
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot may be refilled
             issue(slot, s + D);
@@ -622,7 +625,7 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
     for (int o = tid; o < 256 * NG * MT; o += blockDim.x) {
         const int nl = o % (16 * NG), m = o / (16 * NG);
         const int n = n0 + nl;
-        if (m >= M || n >= N) continue;
+        if (m >= M || n >= N || nl >= 8 * NB) continue;
         const int a = nl >> 4, nn = nl & 15, b = m >> 4;
         const int src_lane = (nn >> 2) * 16 + (m & 15), e = nn & 3;
         int sum = 0;
@@ -630,6 +633,31 @@ __global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ 
         if constexpr (DEQ) y[(int64_t)m * N + n] = ((float)sum * sx[m]) * sw[n];
         else acc_out[(int64_t)m * N + n] = sum;
     }
+}
+
+template <int NB, int MT, int D, bool DEQ>
+__global__ __launch_bounds__(512) void k_skinny_ring(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                                     const float *__restrict__ sx, const float *__restrict__ sw,
+                                                     int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
+                                                     int N, int K)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    ring_body<NB, MT, D, DEQ>(qx, qw, sx, sw, acc_out, y, M, N, K, (int)blockIdx.x * 8 * NB, smem);
+}
+
+// An odd number of 8-row blocks per compute unit, dealt to two workgroups of four waves that share the unit: the
+// first half of the grid takes NBA blocks each, the second half NBB = NBA - 1 (the dispatcher fills every unit once
+// before it places a second workgroup anywhere, so a unit gets one of each).
+template <int NBA, int NBB, int MT, int D, bool DEQ>
+__global__ __launch_bounds__(256) void k_skinny_ring_mixed(const int8_t *__restrict__ qx, const int8_t *__restrict__ qw,
+                                                           const float *__restrict__ sx, const float *__restrict__ sw,
+                                                           int32_t *__restrict__ acc_out, float *__restrict__ y, int M,
+                                                           int N, int K)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int half = (int)(gridDim.x >> 1), id = (int)blockIdx.x;
+    if (id < half) ring_body<NBA, MT, D, DEQ>(qx, qw, sx, sw, acc_out, y, M, N, K, id * 8 * NBA, smem);
+    else ring_body<NBB, MT, D, DEQ>(qx, qw, sx, sw, acc_out, y, M, N, K, half * 8 * NBA + (id - half) * 8 * NBB, smem);
 }
 
 template <int MB, bool DEQ>
@@ -672,18 +700,34 @@ static int32_t launch_reg_cw(const int8_t *qx, const float *sx, const int8_t *qw
     }
 }
 
-template <int NG, int MT, int D, bool DEQ>
+template <int NB, int MT, int D, bool DEQ>
 static int32_t launch_ring(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
                            float *y, int M, int N, int K, int nwave, hipStream_t s)
 {
-    constexpr int STAGE = 2 * (NG + MT) * 1024;
+    constexpr int STAGE = (NB + 2 * MT) * 1024;
+    constexpr int NG = (NB + 1) / 2;
     size_t lds = (size_t)nwave * D * STAGE;
     const size_t part = (size_t)nwave * NG * MT * 4 * 64 * sizeof(int);
     if (part > lds) lds = part;
-    MI_LDS_OPT_IN((&k_skinny_ring<NG, MT, D, DEQ>), 160 * 1024);
-    const unsigned grid = (unsigned)((N + 16 * NG - 1) / (16 * NG));
-    hipLaunchKernelGGL((k_skinny_ring<NG, MT, D, DEQ>), dim3(grid), dim3((unsigned)(64 * nwave)), lds, s, qx, qw, sx,
+    if (lds > 160 * 1024) return MI_ENOSPC;
+    MI_LDS_OPT_IN((&k_skinny_ring<NB, MT, D, DEQ>), 160 * 1024);
+    const unsigned grid = (unsigned)((N + 8 * NB - 1) / (8 * NB));
+    hipLaunchKernelGGL((k_skinny_ring<NB, MT, D, DEQ>), dim3(grid), dim3((unsigned)(64 * nwave)), lds, s, qx, qw, sx,
                        sw, acc, y, M, N, K);
+    return launch_status();
+}
+
+template <int NBA, int NBB, int MT, int D, bool DEQ>
+static int32_t launch_ring_mixed(const int8_t *qx, const float *sx, const int8_t *qw, const float *sw, int32_t *acc,
+                                 float *y, int M, int N, int K, int cus, hipStream_t s)
+{
+    constexpr int nwave = 4;
+    constexpr size_t lds = (size_t)nwave * D * (NBA + 2 * MT) * 1024;   // also covers the partial sums (<= 16 KB)
+    static_assert(2 * lds <= 160 * 1024 && NBB == NBA - 1 && NBB >= 1, "two workgroups share a compute unit");
+    if (N != 8 * cus * (NBA + NBB)) return MI_EINVAL;
+    MI_LDS_OPT_IN((&k_skinny_ring_mixed<NBA, NBB, MT, D, DEQ>), 160 * 1024);
+    hipLaunchKernelGGL((k_skinny_ring_mixed<NBA, NBB, MT, D, DEQ>), dim3((unsigned)(2 * cus)), dim3(64 * nwave), lds, s,
+                       qx, qw, sx, sw, acc, y, M, N, K);
     return launch_status();
 }
 
@@ -715,6 +759,25 @@ int32_t launch_skinny(const int8_t *qx, const float *sx, const int8_t *qw, const
     const int cus = compute_units();
     const int steps = K >> 7;
     const int MT = (M + 15) / 16;
+    // Up to 16 tokens and rows that deal out evenly: every compute unit gets the same number of 8-row blocks in two
+    // workgroups of four waves (3, 5, 7 blocks a unit: one workgroup with a block more than the other; 10, 12, 14:
+    // equal ones).  With 16-row workgroups on N = 6144 half of the units stream twice as many rows as the other half,
+    // and on N = 14336 or 28672 a quarter of them four groups to the others' three.  Measured at M = 16, K = 4096,
+    // weights from HBM: 9.17 -> 8.50 us (N = 6144), 14.8 -> 14.1 us (14336), 26.8 -> 24.4 us (28672).  N = 4096 stays
+    // with one 16-row workgroup of eight waves per unit (two 8-row workgroups read the activation codes twice as
+    // often: 17.2 against 14.4 us at K = 14336).
+    if (MT == 1 && N % (8 * cus) == 0 && steps >= 8) {
+        const int per_cu = N / (8 * cus);
+        switch (per_cu) {
+        case 3: return launch_ring_mixed<2, 1, 1, 4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, cus, s);
+        case 5: return launch_ring_mixed<3, 2, 1, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, cus, s);
+        case 7: return launch_ring_mixed<4, 3, 1, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, cus, s);
+        case 10: return launch_ring<5, 1, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, 4, s);
+        case 12: return launch_ring<6, 1, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, 4, s);
+        case 14: return launch_ring<7, 1, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, 4, s);
+        default: break;
+        }
+    }
     // Two 16-row groups per workgroup halve the activation traffic when there are rows enough to fill the
     // chip.  Four waves (a 64-72 KB ring set, so two workgroups share a compute unit and overlap their
     // prologues and epilogues) when there are workgroups enough, else eight waves to keep bytes in flight.
@@ -724,11 +787,11 @@ int32_t launch_skinny(const int8_t *qx, const float *sx, const int8_t *qw, const
     while (nwave > 1 && nwave > steps) nwave >>= 1;
     switch (MT) {
     case 1:
-        return two ? launch_ring<2, 1, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s)
-                   : launch_ring<1, 1, 4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
-    case 2: return launch_ring<1, 2, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
+        return two ? launch_ring<4, 1, 3, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s)
+                   : launch_ring<2, 1, 4, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
+    case 2: return launch_ring<2, 2, 2, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
     case 3:
-    case 4: return launch_ring<1, 4, 1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
+    case 4: return launch_ring<2, 4, 1, DEQ>(qx, sx, qw, sw, acc, y, M, N, K, nwave, s);
     default: return MI_ERANGE;
     }
 }
