@@ -27,6 +27,10 @@ def gpu_gemm_i32(mi, dev, qx, qw):
     (1, 64, 128), (1, 6144, 4096), (4, 4096, 14336), (16, 256, 4096), (13, 48, 1024),
     (17, 64, 768), (32, 4096, 4096), (33, 128, 2048), (48, 160, 256), (64, 512, 1408),
     (2, 96, 9216), (3, 80, 11264),    # K that the register-resident GEMV cannot split: the LDS-staged one
+    # 5 to 16 tokens with N = 8 * 256 * P rows: the ring kernel with the rows dealt to the compute units in 8-row
+    # blocks, P = 3, 5, 7 as two workgroups of unequal size per unit, P = 10, 12, 14 as two equal ones
+    (16, 6144, 4096), (5, 6144, 1024), (16, 10240, 1024), (9, 14336, 2048), (16, 14336, 4096),
+    (16, 20480, 1024), (12, 24576, 1024), (16, 28672, 4096), (7, 28672, 1024),
 ])
 def test_skinny_accumulators_bit_exact(mi, dev, orc, M, N, K):
     qx, qw = rand_codes(M * 7 + N, (M, K)), rand_codes(K + 1, (N, K))
