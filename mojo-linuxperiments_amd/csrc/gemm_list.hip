@@ -252,10 +252,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(Cfg::SCL0 / 2))
     int kt = 0, nk = 0;
     bool first_tile = true;   // no stores of a tile before this one are in flight
 
-    // one stage.  There is ONE copy of this code and one loop around it: a fragment register is written by an LDS
-    // read the compiler cannot follow (its data arrives later), so no value of xa / xc / w may ever have to be moved
-    // where two paths of the control flow meet.  The last stage of a workgroup therefore also requests "next"
-    // fragments (from a buffer that holds nothing new; they are never used).
+    // one stage.  There is ONE copy of this code in the source and one loop around it: a fragment register is written
+    // by an LDS read the compiler cannot follow (its data arrives later), so no value of xa / xc / w may ever have to
+    // be moved where two paths of the control flow meet.  The last stage of a workgroup therefore also requests "next"
+    // fragments (from a buffer that holds nothing new; they are never used).  (The compiler may still duplicate the
+    // body, and does: it peels a tile's first stage off the loop.  That is harmless as long as every fragment keeps
+    // its registers from one copy to the next; the build reads the assembly and stops if a fragment register is ever
+    // the source of a move or if the LDS reads write more register ranges than there are fragments.)
     //
     // Fragments are requested half a stage ahead: while the eight groups of a K half run, the four activation
     // fragments of the next half arrive in the other activation set (xa: first halves, xc: second halves) and weight

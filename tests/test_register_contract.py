@@ -9,6 +9,7 @@ import os
 import re
 import struct
 import subprocess
+import sys
 import tempfile
 
 import pytest
@@ -71,11 +72,11 @@ def test_the_library_holds_gfx950_kernels(notes):
     assert len(notes) > 50 and any("k_w8a8_list" in k for k in notes)
 
 
-def test_batched_gemm_keeps_its_96_accumulators_to_itself(notes):
+def test_batched_gemm_keeps_its_128_accumulators_to_itself(notes):
     mine = {k: v for k, v in notes.items() if "k_w8a8_list" in k}
     assert len(mine) == 2   # dequantized and int32 form
     for name, f in mine.items():
-        # v0..v159 for the compiler, v160..v255 named by hand: the wave's count is the full 256 (two waves per SIMD),
+        # v0..v103 for the compiler, v104..v255 named by hand: the wave's count is the full 256 (two waves per SIMD),
         # no accumulation register, nothing in scratch, no vector and no scalar register spilled
         assert f["vgpr_count"] == 256 and f["agpr_count"] == 0, (name, f)
         assert f["vgpr_spill_count"] == 0 and f["sgpr_spill_count"] == 0 and f["private_segment_fixed_size"] == 0, (name, f)
@@ -97,3 +98,46 @@ def test_no_kernel_with_memory_instructions_in_asm_spills_a_scalar(notes):
     for name, f in notes.items():
         if any(k in name for k in ("k_w8a8_tiled", "k_w8a8_pair", "k_w8a8_list")):
             assert f["sgpr_spill_count"] == 0, (name, f)
+
+
+# ---- the batched GEMM's operand fragments: written by LDS reads behind the compiler's back, never to be copied
+
+CHECK = os.path.join(ROOT, "mojo-linuxperiments_amd", "csrc", "check_fragment_registers.py")
+ASM = os.path.join(ROOT, "mojo-linuxperiments_amd", "csrc", "gemm_list.s")
+
+FAKE = """\
+k_fake_list: ; @k_fake_list
+\tds_read_b128 v[0:3], v70
+\tds_read_b128 v[4:7], v70 offset:2048
+\tv_mfma_i32_16x16x64_i8 v[128:131], v[4:7], v[0:3], v[128:131]
+%s
+\ts_endpgm
+.Lfunc_end0:
+"""
+
+
+def run_check(path, *args):
+    return subprocess.run([sys.executable, CHECK, path, *args], capture_output=True, text=True)
+
+
+def test_fragment_check_passes_on_the_built_kernel():
+    if not os.path.exists(ASM):
+        pytest.skip("gemm_list.s is written by the build (make -C mojo-linuxperiments_amd/csrc)")
+    out = run_check(ASM, "k_w8a8_list", "16")
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert "2 kernel(s)" in out.stdout
+
+
+def test_fragment_check_fails_on_a_copied_fragment_and_on_a_fragment_that_moved(tmp_path):
+    good = tmp_path / "good.s"
+    good.write_text(FAKE % "\tv_mov_b32_e32 v9, v64")            # a move INTO a dead fragment register is fine
+    assert run_check(str(good), "k_fake_list", "2").returncode == 0
+    copied = tmp_path / "copied.s"
+    copied.write_text(FAKE % "\tv_mov_b32_e32 v9, v5")           # a move OUT of one is not
+    out = run_check(str(copied), "k_fake_list", "2")
+    assert out.returncode != 0 and "copies fragment register v5" in out.stderr
+    moved = tmp_path / "moved.s"
+    moved.write_text(FAKE % "\tds_read_b128 v[8:11], v70")       # a third range where two are expected
+    out = run_check(str(moved), "k_fake_list", "2")
+    assert out.returncode != 0 and "3 distinct register ranges" in out.stderr
+    assert run_check(str(good), "k_absent").returncode != 0
