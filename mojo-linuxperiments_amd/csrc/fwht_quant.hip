@@ -111,7 +111,10 @@ struct QuantBatch {
     QuantSet s[QUANT_BATCH_MAX];
     int n;
 };
-template <int BLOCK>
+// CMAX: the most 8-float chunks per thread any set of the batch needs.  The kernel's registers are those of its
+// widest row body whichever set a workgroup works on, so a batch of rows up to K = 14336 is not made to run at the
+// occupancy of the K = 32768 body (160 registers, three waves per SIMD).
+template <int BLOCK, int CMAX>
 __global__ __launch_bounds__(256) void k_fwht_rows_batch(const QuantBatch b)
 {
     int i = 0;
@@ -123,8 +126,11 @@ __global__ __launch_bounds__(256) void k_fwht_rows_batch(const QuantBatch b)
     const int C = (S.K / 8 + 255) / 256;
     if (C <= 1) fwht_row_body<BLOCK, 1, true>(S.x, S.q, S.scale, nullptr, S.K, row);
     else if (C <= 2) fwht_row_body<BLOCK, 2, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if constexpr (CMAX <= 2) return;
     else if (C <= 4) fwht_row_body<BLOCK, 4, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if constexpr (CMAX <= 4) return;
     else if (C <= 7) fwht_row_body<BLOCK, 7, true>(S.x, S.q, S.scale, nullptr, S.K, row);
+    else if constexpr (CMAX <= 7) return;
     else if (C <= 8) fwht_row_body<BLOCK, 8, true>(S.x, S.q, S.scale, nullptr, S.K, row);
     else fwht_row_body<BLOCK, 16, true>(S.x, S.q, S.scale, nullptr, S.K, row);
 }
@@ -375,8 +381,22 @@ extern "C" int32_t mi_fwht_quant_batch_f32_i8(const mi_quant_rows *sets, int32_t
         return MI_OK;
     }
     b.n = n;
-    if (block == 128) hipLaunchKernelGGL(k_fwht_rows_batch<128>, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), b);
-    else hipLaunchKernelGGL(k_fwht_rows_batch<256>, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), b);
+    int cmax = 1;
+    for (int i = 0; i < n; ++i) cmax = std::max(cmax, (b.s[i].K / 8 + 255) / 256);
+#define MI_QBATCH(BLOCK_, CMAX_) \
+    hipLaunchKernelGGL((k_fwht_rows_batch<BLOCK_, CMAX_>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream), b)
+    if (block == 128) {
+        if (cmax <= 2) MI_QBATCH(128, 2);
+        else if (cmax <= 4) MI_QBATCH(128, 4);
+        else if (cmax <= 7) MI_QBATCH(128, 7);
+        else MI_QBATCH(128, 16);
+    } else {
+        if (cmax <= 2) MI_QBATCH(256, 2);
+        else if (cmax <= 4) MI_QBATCH(256, 4);
+        else if (cmax <= 7) MI_QBATCH(256, 7);
+        else MI_QBATCH(256, 16);
+    }
+#undef MI_QBATCH
     return launch_status();
 }
 
