@@ -39,8 +39,8 @@ __device__ __forceinline__ float shfl_xor_f(float v, int m) { return __shfl_xor(
 // to its partner and keeps the other half, so each addition joins exactly the
 // two operands the plain butterfly would join (float add is commutative) and
 // 63 shuffles finish 64 dot products.  Lane l ends with pair l.
-template <int OFF, int N>
-__device__ __forceinline__ void fold(float (&p)[64], int lane)
+template <int OFF, int N, int NP>
+__device__ __forceinline__ void fold(float (&p)[NP], int lane)
 {
     const bool hi = (lane & OFF) != 0;
 #pragma unroll
@@ -51,19 +51,23 @@ __device__ __forceinline__ void fold(float (&p)[64], int lane)
     }
 }
 
-// grid = (T/16, E/16): a workgroup of 4 waves covers 16 tokens x 16 experts, so the router weights are read
-// T/16 times and the activations E/16 times in all (both from L2), and every compute unit gets work.
+// grid = (T/16, E/EW): a workgroup of 4 waves covers 16 tokens x EW experts, so the router weights are read
+// T/16 times and the activations E/EW times in all (both from L2), and every compute unit gets work.
 // CQ > 0: the kernel also rotates (block 128) and quantizes the token rows for the expert FFN, a wave per row with CQ
 // chunks per lane (H = 512 * CQ at most), the arithmetic of the stand-alone quantizer: the 16 tokens of a group are
 // dealt to the waves of the group's workgroups, so that the layer launches one kernel less.
-template <int CQ>
+// EW = 8: a wave owns 8 experts for its 4 tokens (32 dot products a lane, half the registers, twice the workgroups):
+// two waves share a SIMD where EW = 16 leaves one alone with its memory round trips (cfg4: 17.2 -> 13.8 us; four
+// experts a wave, or loads two rounds ahead in three register sets, measured the same 13.8).  The first butterfly
+// round (offset 32) is then the plain one; lanes l and l ^ 32 end with the same pair.
+template <int CQ, int EW>
 __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x, const float *__restrict__ wr,
                                                     float *__restrict__ logits, int T, int H, int E,
                                                     int8_t *__restrict__ qx, float *__restrict__ sx)
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = blockIdx.x * 16 + wave * 4;
-    const int e0 = blockIdx.y * 16;
+    const int e0 = blockIdx.y * EW;
 
     // the token row this wave quantizes (if any) is requested first: its loads then fly under the logits' rounds
     // instead of costing a memory round trip after them
@@ -93,9 +97,9 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
         }
     }
 
-    float p[64];
+    float p[4 * EW];
 #pragma unroll
-    for (int i = 0; i < 64; ++i) p[i] = 0.0f;
+    for (int i = 0; i < 4 * EW; ++i) p[i] = 0.0f;
     const float *xr[4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) xr[tt] = x + (int64_t)min(t0 + tt, T - 1) * H + 4 * lane;
@@ -104,53 +108,99 @@ __global__ __launch_bounds__(256) void k_moe_logits(const float *__restrict__ x,
     // second half, the token rows of the next round) are already on their way; with one wave per SIMD the loop is
     // otherwise a chain of memory round trips.  Every dot product still takes its terms in the same order.
     const int nj = H / 256;
-    float4 xv[4], xn[4], wa[8], wb[8];
+    if constexpr (EW == 16) {
+        float4 xv[4], xn[4], wa[8], wb[8];
+    #pragma unroll
+        for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt]);
+    #pragma unroll
+        for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H);
+        for (int j = 0; j < nj; ++j) {
+    #pragma unroll
+            for (int e = 0; e < 8; ++e) wb[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)(8 + e) * H + 256 * j);
+    #pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float a = p[tt * 16 + e];
+                    a = __builtin_fmaf(xv[tt].x, wa[e].x, a);
+                    a = __builtin_fmaf(xv[tt].y, wa[e].y, a);
+                    a = __builtin_fmaf(xv[tt].z, wa[e].z, a);
+                    a = __builtin_fmaf(xv[tt].w, wa[e].w, a);
+                    p[tt * 16 + e] = a;
+                }
+            const int jn = min(j + 1, nj - 1);   // (the last round fetches itself again: no branch around loads)
+    #pragma unroll
+            for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H + 256 * jn);
+    #pragma unroll
+            for (int tt = 0; tt < 4; ++tt) xn[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * jn);
+    #pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float a = p[tt * 16 + 8 + e];
+                    a = __builtin_fmaf(xv[tt].x, wb[e].x, a);
+                    a = __builtin_fmaf(xv[tt].y, wb[e].y, a);
+                    a = __builtin_fmaf(xv[tt].z, wb[e].z, a);
+                    a = __builtin_fmaf(xv[tt].w, wb[e].w, a);
+                    p[tt * 16 + 8 + e] = a;
+                }
+    #pragma unroll
+            for (int tt = 0; tt < 4; ++tt) xv[tt] = xn[tt];
+        }
+    } else {
+        // one group of eight experts: the next round's weights and token rows are requested before this round's
+        // 128 FMAs
+        float4 xv[4], xn[4], wa[8], wn[8];
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt]);
+        for (int tt = 0; tt < 4; ++tt) xv[tt] = *reinterpret_cast<const float4 *>(xr[tt]);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H);
-    for (int j = 0; j < nj; ++j) {
+        for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H);
+        for (int j = 0; j < nj; ++j) {
+            const int jn = min(j + 1, nj - 1);   // (the last round fetches itself again: no branch around loads)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) wb[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)(8 + e) * H + 256 * j);
+            for (int e = 0; e < 8; ++e) wn[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H + 256 * jn);
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
+            for (int tt = 0; tt < 4; ++tt) xn[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * jn);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float a = p[tt * 16 + e];
-                a = __builtin_fmaf(xv[tt].x, wa[e].x, a);
-                a = __builtin_fmaf(xv[tt].y, wa[e].y, a);
-                a = __builtin_fmaf(xv[tt].z, wa[e].z, a);
-                a = __builtin_fmaf(xv[tt].w, wa[e].w, a);
-                p[tt * 16 + e] = a;
-            }
-        const int jn = min(j + 1, nj - 1);   // (the last round fetches itself again: no branch around loads)
+            for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) wa[e] = *reinterpret_cast<const float4 *>(wp + (int64_t)e * H + 256 * jn);
+                for (int e = 0; e < 8; ++e) {
+                    float a = p[tt * 8 + e];
+                    a = __builtin_fmaf(xv[tt].x, wa[e].x, a);
+                    a = __builtin_fmaf(xv[tt].y, wa[e].y, a);
+                    a = __builtin_fmaf(xv[tt].z, wa[e].z, a);
+                    a = __builtin_fmaf(xv[tt].w, wa[e].w, a);
+                    p[tt * 8 + e] = a;
+                }
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) xn[tt] = *reinterpret_cast<const float4 *>(xr[tt] + 256 * jn);
+            for (int e = 0; e < 8; ++e) wa[e] = wn[e];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float a = p[tt * 16 + 8 + e];
-                a = __builtin_fmaf(xv[tt].x, wb[e].x, a);
-                a = __builtin_fmaf(xv[tt].y, wb[e].y, a);
-                a = __builtin_fmaf(xv[tt].z, wb[e].z, a);
-                a = __builtin_fmaf(xv[tt].w, wb[e].w, a);
-                p[tt * 16 + 8 + e] = a;
-            }
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) xv[tt] = xn[tt];
+            for (int tt = 0; tt < 4; ++tt) xv[tt] = xn[tt];
+        }
     }
-    fold<32, 32>(p, lane);
-    fold<16, 16>(p, lane);
-    fold<8, 8>(p, lane);
-    fold<4, 4>(p, lane);
-    fold<2, 2>(p, lane);
-    fold<1, 1>(p, lane);
-    // lane l now holds pair l: token l/16, expert e0 + l%16
-    const int t = t0 + (lane >> 4);
-    if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
+    if constexpr (EW == 16) {
+        fold<32, 32>(p, lane);
+        fold<16, 16>(p, lane);
+        fold<8, 8>(p, lane);
+        fold<4, 4>(p, lane);
+        fold<2, 2>(p, lane);
+        fold<1, 1>(p, lane);
+        // lane l now holds pair l: token l/16, expert e0 + l%16
+        const int t = t0 + (lane >> 4);
+        if (t < T) logits[(int64_t)t * E + e0 + (lane & 15)] = p[0];
+    } else {
+        static_assert(EW == 8, "experts per wave");
+#pragma unroll
+        for (int i = 0; i < 32; ++i) p[i] = p[i] + shfl_xor_f(p[i], 32);
+        fold<16, 16>(p, lane);
+        fold<8, 8>(p, lane);
+        fold<4, 4>(p, lane);
+        fold<2, 2>(p, lane);
+        fold<1, 1>(p, lane);
+        // lanes l and l ^ 32 now hold pair l % 32: token (l % 32) / 8, expert e0 + l % 8
+        const int t = t0 + ((lane & 31) >> 3);
+        if (lane < 32 && t < T) logits[(int64_t)t * E + e0 + (lane & 7)] = p[0];
+    }
     if constexpr (CQ > 0) {
         if (has_row) {
             float amax = 0.0f;
@@ -917,9 +967,19 @@ static bool route_can_quantize(int64_t H) { return H % 128 == 0 && H <= 2048; }
 static int32_t launch_route(const float *x, const float *wr, int32_t *idx, float *w, int64_t T, int64_t H, int64_t E,
                             int32_t topk, float *logits, int8_t *qx, float *sx, void *stream)
 {
-    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)(E / 16));
+    // eight experts a wave (twice the workgroups) while sixteen would leave at most two workgroups to a compute unit
+    const bool narrow = (int64_t)((T + 15) / 16) * (E / 16) <= 2 * (int64_t)compute_units();
+    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)(E / (narrow ? 8 : 16)));
     const int cq = qx ? (int)((H / 8 + 63) / 64) : 0;
-#define MI_LOGITS(CQ_) hipLaunchKernelGGL(k_moe_logits<CQ_>, grid, dim3(256), 0, as_stream(stream), x, wr, logits, (int)T, (int)H, (int)E, qx, sx)
+#define MI_LOGITS(CQ_)                                                                                                  \
+    do {                                                                                                                \
+        if (narrow)                                                                                                     \
+            hipLaunchKernelGGL((k_moe_logits<CQ_, 8>), grid, dim3(256), 0, as_stream(stream), x, wr, logits, (int)T,    \
+                               (int)H, (int)E, qx, sx);                                                                 \
+        else                                                                                                            \
+            hipLaunchKernelGGL((k_moe_logits<CQ_, 16>), grid, dim3(256), 0, as_stream(stream), x, wr, logits, (int)T,   \
+                               (int)H, (int)E, qx, sx);                                                                 \
+    } while (0)
     switch (cq) {
     case 0: MI_LOGITS(0); break;
     case 1: MI_LOGITS(1); break;
