@@ -730,13 +730,15 @@ def gemm_timeline(mi, wl):
 def list_timeline(mi, wl, dev, s):
     """The batched GEMM (k_w8a8_list) on the four cfg3 projections as one launch: 240 launches on the benchmark's
     codes, then the clock reads one more launch left for every tile of every workgroup: first stage begins, last
-    stage issued, last store of the tile issued."""
+    stage issued, last store of the tile issued.  Measured twice: with the same weights every launch (they stay in
+    the memory-side cache) and, under "with_weights_from_hbm", with four copies of the weights taken in turn (as the
+    timed step of the bench does)."""
     import ctypes as C
     lib = mi.lib
     M = wl.PREFILL_M
     shapes = [(M, 6144, 4096), (M, 14336, 4096), (M, 14336, 4096), (M, 4096, 14336)]
     mark = dev.mark()
-    ops = []
+    ops, copies = [], []
     for i, (_, N, K) in enumerate(shapes):
         m2 = dev.mark()
         qx, sx = dev.empty((M, K), np.int8), dev.empty(M, np.float32)
@@ -747,21 +749,38 @@ def list_timeline(mi, wl, dev, s):
         host = [dev.download(b) for b in (qx, sx, qw, sw)]
         dev.reset_to(m2)
         ops.append(tuple(dev.upload(h) for h in host) + (dev.empty((M, N), np.float32),))
+        copies.append([(ops[-1][2], ops[-1][3])] + [(dev.upload(host[2]), dev.upload(host[3])) for _ in range(3)])
     batch = mi.GemmBatch(dev, shapes)
+    f = lib.mi_debug_gemm_list_timeline
+    f.restype, f.argtypes = C.c_int32, [C.c_void_p, C.c_int32, C.c_int32]
+    turn = [0]
+
+    def launch_ops(rotate):
+        if not rotate:
+            return ops
+        turn[0] += 1
+        return [(o[0], o[1]) + c[turn[0] % 4] + (o[4],) for o, c in zip(ops, copies)]
+
+    res = measure_list_timeline(mi, dev, s, batch, f, lambda: launch_ops(False))
+    res["with_weights_from_hbm"] = measure_list_timeline(mi, dev, s, batch, f, lambda: launch_ops(True))
+    batch.destroy()
+    dev.reset_to(mark)
+    return res
+
+
+def measure_list_timeline(mi, dev, s, batch, f, next_ops):
     for _ in range(200):
-        batch.run_f32(ops, stream=s)
+        batch.run_f32(next_ops(), stream=s)
     e0, e1 = mi.Event(), mi.Event()
     e0.record(s)
     for _ in range(40):
-        batch.run_f32(ops, stream=s)
+        batch.run_f32(next_ops(), stream=s)
     e1.record(s)
     e1.synchronize()
     us = e0.elapsed_ms(e1) / 40 * 1e3
     WGS, TILES = 512, 16
-    f = lib.mi_debug_gemm_list_timeline
-    f.restype, f.argtypes = C.c_int32, [C.c_void_p, C.c_int32, C.c_int32]
     mi.check(f(None, 0, 1))
-    batch.run_f32(ops, stream=s)
+    batch.run_f32(next_ops(), stream=s)
     dev.sync(s)
     buf = np.zeros(WGS * TILES * 8, np.uint64)
     mi.check(f(buf.ctypes.data, buf.size, 0))
@@ -803,8 +822,6 @@ def list_timeline(mi, wl, dev, s):
            "note": "k_w8a8_list, one launch over the four cfg3 projections; clock ticks = s_memtime read by wave 0 of "
                    "every workgroup at three points of every tile and around the wait and the barrier of every stage "
                    "(three reads a stage, about 100 ticks); instrumented build"}
-    batch.destroy()
-    dev.reset_to(mark)
     return res
 
 
