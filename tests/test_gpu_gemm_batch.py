@@ -129,3 +129,31 @@ def test_batch_rejects_what_it_cannot_run(mi, dev):
     assert e.value.status == mi.EINVAL
     batch.destroy()
     dev.reset_to(mark)
+
+
+def test_random_batches_equal_the_single_problem_kernels(mi, dev):
+    """Seeded random batches (1 to 4 problems, ragged M and N, 3 to 19 K stages, mixed K in one batch): every
+    dequantized output equals, bit for bit, what the single-problem entry point writes for the same operands."""
+    rng = np.random.default_rng(20251125)
+    for _ in range(12):
+        shapes = [(int(rng.integers(256, 1200)), max(256, int(rng.integers(16, 90)) * 16), int(rng.integers(3, 20)) * 128)
+                  for _ in range(int(rng.integers(1, 5)))]
+        mark = dev.mark()
+        ops, refs = [], []
+        for M, N, K in shapes:
+            qx = dev.upload(rng.integers(-127, 128, (M, K)).astype(np.int8))
+            qw = dev.upload(rng.integers(-127, 128, (N, K)).astype(np.int8))
+            sx = dev.upload(rng.uniform(0.01, 1, M).astype(np.float32))
+            sw = dev.upload(rng.uniform(0.001, 0.1, N).astype(np.float32))
+            y, ref = dev.empty((M, N), np.float32), dev.empty((M, N), np.float32)
+            mi.check(mi.lib.mi_fill_u32(y.ptr, 0x7F7F7F7F, y.nbytes // 4, None))   # poison: every element must be written
+            mi.check(mi.lib.mi_w8a8_gemm_dequant_f32(qx.ptr, sx.ptr, qw.ptr, sw.ptr, ref.ptr, M, N, K, None))
+            ops.append((qx, sx, qw, sw, y))
+            refs.append(ref)
+        batch = mi.GemmBatch(dev, shapes)
+        batch.run_f32(ops)
+        dev.sync()
+        for s, o, r in zip(shapes, ops, refs):
+            assert np.array_equal(dev.download(o[4]), dev.download(r)), (shapes, s)
+        batch.destroy()
+        dev.reset_to(mark)
