@@ -71,16 +71,16 @@ def test_paired_wave_kernel_bit_exact(mi, dev, orc, M, N, K):
     assert np.array_equal(y, orc.dequant(want, sx, sw))
 
 
-def test_random_skinny_shapes_bit_exact(mi, dev):
+def test_random_skinny_shapes_bit_exact(mi, dev, orc):
     """Seeded random shapes over every skinny path (1 to 64 tokens, K of 1 to 39 stages, N any multiple of 16 or a
-    multiple of 2048, which takes the evenly dealt ring kernels): exact against numpy's int32 product."""
+    multiple of 2048, which takes the evenly dealt ring kernels): exact against the oracle."""
     rng = np.random.default_rng(7)
     for _ in range(60):
         M, K = int(rng.integers(1, 65)), int(rng.integers(1, 40)) * 128
         N = int(rng.choice([int(rng.integers(1, 300)) * 16, 2048 * int(rng.integers(1, 15))]))
         qx = rng.integers(-127, 128, (M, K)).astype(np.int8)
         qw = rng.integers(-127, 128, (N, K)).astype(np.int8)
-        assert np.array_equal(gpu_gemm_i32(mi, dev, qx, qw), qx.astype(np.int32) @ qw.astype(np.int32).T), (M, N, K)
+        assert np.array_equal(gpu_gemm_i32(mi, dev, qx, qw), orc.gemm_i8_i32(qx, qw)), (M, N, K)
 
 
 def test_extreme_codes_do_not_overflow(mi, dev):
